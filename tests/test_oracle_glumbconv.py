@@ -1,0 +1,109 @@
+"""Pins for the oracle's GLUMBConv (Mix-FFN): brute-force taps in C, library
+reductions (1x1 conv == linear) and the a/g split."""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from oracle import cbrute
+from oracle import sana_oracle as O
+
+
+def _mlp(C, Hd, seed=0):
+    torch.manual_seed(seed)
+    m = O.GLUMBConv(C, Hd, use_bias=(True, True, False), norm=(None, None, None), act=("silu", "silu", None)).double()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(torch.randn_like(p) * 0.3)
+    return m
+
+
+def test_state_dict_keys_and_shapes():
+    m = O.GLUMBConv(16, 40, use_bias=(True, True, False))
+    sd = m.state_dict()
+    assert sorted(sd) == ["depth_conv.conv.bias", "depth_conv.conv.weight", "inverted_conv.conv.bias",
+                          "inverted_conv.conv.weight", "point_conv.conv.weight"]
+    assert sd["inverted_conv.conv.weight"].shape == (80, 16, 1, 1)
+    assert sd["depth_conv.conv.weight"].shape == (80, 1, 3, 3)
+    assert sd["point_conv.conv.weight"].shape == (16, 40, 1, 1)
+
+
+def test_against_bruteforce_taps_on_4x5_grid():
+    C, Hd, B, Hh, Ww = 6, 10, 2, 4, 5
+    m = _mlp(C, Hd)
+    x = torch.randn(B, Hh * Ww, C, dtype=torch.float64)
+    # stage 1 by library reduction: 1x1 conv == linear, then SiLU
+    w1 = m.inverted_conv.conv.weight.flatten(1)
+    u = F.silu(x @ w1.T + m.inverted_conv.conv.bias)                      # [B, N, 2H] channels-last
+    # stage 2 by brute force in C
+    y = cbrute.dwconv_gate(u.view(B, Hh, Ww, 2 * Hd).detach().numpy(),
+                           m.depth_conv.conv.weight.view(2 * Hd, 3, 3).detach().numpy(),
+                           m.depth_conv.conv.bias.detach().numpy())
+    # stage 3: 1x1 conv == linear, no bias
+    ref = torch.from_numpy(y).view(B, Hh * Ww, Hd) @ m.point_conv.conv.weight.flatten(1).T
+    torch.testing.assert_close(m(x, HW=(Hh, Ww)), ref, rtol=1e-10, atol=1e-12)
+
+
+def test_gate_is_on_the_second_half():
+    """Zeroing the depthwise filter+bias of the FIRST half zeroes the output;
+    zeroing the second half gives a * silu(0) = 0 as well, but a bias of +40 on
+    the second half (silu(g) ~= g) must scale the output, not gate it off."""
+    C, Hd = 4, 6
+    m = _mlp(C, Hd, seed=1)
+    x = torch.randn(1, 9, C, dtype=torch.float64)
+    with torch.no_grad():
+        m.depth_conv.conv.weight[Hd:].zero_()
+        m.depth_conv.conv.bias[Hd:].fill_(40.0)
+    y40 = m(x, HW=(3, 3))
+    with torch.no_grad():
+        m.depth_conv.conv.bias[Hd:].fill_(20.0)
+    y20 = m(x, HW=(3, 3))
+    torch.testing.assert_close(y40, 2 * y20, rtol=1e-6, atol=1e-9)
+    with torch.no_grad():
+        m.depth_conv.conv.weight[:Hd].zero_()
+        m.depth_conv.conv.bias[:Hd].zero_()
+    assert m(x, HW=(3, 3)).abs().max() == 0
+
+
+def test_video_hw_is_per_frame():
+    """HW=(T,H,W) applies the 3x3 independently per frame (basic_modules.py:187-189)."""
+    C, Hd, T, Hh, Ww = 4, 6, 3, 3, 4
+    m = _mlp(C, Hd, seed=2)
+    x = torch.randn(2, T * Hh * Ww, C, dtype=torch.float64)
+    y = m(x, HW=(T, Hh, Ww))
+    per_frame = torch.cat([m(x[:, t * Hh * Ww:(t + 1) * Hh * Ww], HW=(Hh, Ww)) for t in range(T)], dim=1)
+    torch.testing.assert_close(y, per_frame, rtol=1e-12, atol=1e-12)
+
+
+def test_autochunk_splits_are_transparent(monkeypatch):
+    C, Hd = 4, 6
+    m = _mlp(C, Hd, seed=3)
+    x = torch.randn(5, 12, C, dtype=torch.float64)
+    y = m(x, HW=(3, 4))
+    monkeypatch.setattr(O, "INT32_SAFE_CONV_ELEMENTS", 2 * 2 * Hd * 12)  # two images per call
+    torch.testing.assert_close(m(x, HW=(3, 4)), y, rtol=0, atol=0)
+
+
+def test_bf16_rounding_points():
+    """Six roundings in bf16 (each torch op returns bf16): conv1x1+bias, SiLU,
+    depthwise+bias, SiLU(g), a*g, conv1x1 — reproduced by hand with fp32 math
+    between explicit bf16 round trips."""
+    C, Hd, Hh, Ww = 32, 80, 6, 7
+    torch.manual_seed(5)
+    m = O.GLUMBConv(C, Hd, use_bias=(True, True, False)).bfloat16()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_((torch.randn(p.shape) * 0.2).bfloat16())
+    x = torch.randn(1, Hh * Ww, C).bfloat16()
+    y = m(x, HW=(Hh, Ww))
+    r = lambda t: t.bfloat16().float()
+    w1 = m.inverted_conv.conv.weight.flatten(1).float()
+    u = r(F.silu(r(x.float() @ w1.T + m.inverted_conv.conv.bias.float())))
+    un = u.view(1, Hh, Ww, 2 * Hd).permute(0, 3, 1, 2)
+    dw = r(F.conv2d(un, m.depth_conv.conv.weight.float(), m.depth_conv.conv.bias.float(), padding=1, groups=2 * Hd))
+    a, g = dw[:, :Hd], dw[:, Hd:]
+    z = r(a * r(F.silu(g)))
+    ref = r(z.permute(0, 2, 3, 1).reshape(1, Hh * Ww, Hd) @ m.point_conv.conv.weight.flatten(1).float().T)
+    err = (y.float() - ref).abs().max().item()
+    # identical up to fp32 accumulation order inside the library GEMM/conv: at most an ulp of bf16 here and there
+    assert err <= 2 ** -7 * ref.abs().max().item(), err
+    assert ((y.float() - ref).norm() / ref.norm()).item() < 2e-3
