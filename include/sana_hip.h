@@ -1,0 +1,166 @@
+/* sana_hip.h — C ABI of libsana_hip.so: hand-written gfx950 (MI355X) kernels
+ * for the SanaMSBlock hot path (LiteLA linear attention + GLUMBConv Mix-FFN).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the comment says "host".
+ *   - The caller owns every buffer.  The library allocates nothing and keeps
+ *     no global state; scratch space is passed in as `workspace`.
+ *   - All work is enqueued on `stream` (a hipStream_t passed as void*; NULL is
+ *     the default stream).  No entry point synchronises with the host.
+ *   - Return value: SANA_OK (0) or a negative SANA_ERR_* code.  Nothing is
+ *     launched when an error is returned.  sana_hip_strerror() names a code.
+ *   - Strides are in ELEMENTS of the io dtype.  The channel stride is always 1.
+ *   - Channel c belongs to head c / d, lane c % d (d = head_dim = 32).
+ *
+ * The reference (NVlabs/Sana) has no native seam for this path: its seam is the
+ * Python module API (attn_type / ffn_type selection,
+ * diffusion/model/nets/sana_multi_scale.py:77-140).  Each entry point below
+ * names the reference code it replaces.
+ */
+#ifndef SANA_HIP_H_
+#define SANA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SANA_HIP_ABI_VERSION 1
+
+/* io dtypes */
+#define SANA_DT_F32 0
+#define SANA_DT_BF16 1
+#define SANA_DT_F16 2
+
+/* error codes */
+#define SANA_OK 0
+#define SANA_ERR_ARG (-1)        /* null pointer, negative size, unknown enum      */
+#define SANA_ERR_SHAPE (-2)      /* shape outside what the kernels support         */
+#define SANA_ERR_ALIGN (-3)      /* pointer or stride not 16-byte aligned          */
+#define SANA_ERR_WORKSPACE (-4)  /* workspace missing or too small                 */
+#define SANA_ERR_LAUNCH (-5)     /* hipLaunchKernel reported an error              */
+#define SANA_ERR_DTYPE (-6)      /* dtype not supported by this entry point        */
+
+/* GEMM epilogues */
+#define SANA_EPI_NONE 0       /* C = A W^T                       */
+#define SANA_EPI_BIAS 1       /* C = A W^T + bias                */
+#define SANA_EPI_BIAS_SILU 2  /* C = silu(A W^T + bias)          */
+
+int sana_hip_abi_version(void);
+const char* sana_hip_strerror(int code);
+
+/* ---------------------------------------------------------------------------
+ * ReLU linear attention, phase 1: per-(batch, head[, chunk]) state
+ *
+ *   state[b][h][c][i][j] = sum over tokens n of chunk c of
+ *                          vpad[n][i] * relu(k[n][j]),   i in 0..d, j in 0..d-1
+ *   vpad[n][d] = 1, so row d is sum_n relu(k[n]).
+ *
+ * Replaces `relu(k)`, `F.pad(v, value=1)` and `vk = v @ k` of
+ * LiteLA.attn_matmul (diffusion/model/nets/sana_blocks.py:248-256) and the
+ * reference's Triton kernel pad_vk_mm_fwd
+ * (diffusion/model/nets/fastlinear/modules/triton_lite_mla_kernels/pad_vk_mm_fwd.py:60-151).
+ * With n_chunks > 1 and causal != 0 the states are additionally turned into an
+ * inclusive prefix sum over chunks (cumsum_vk / cumsum_k_sum of
+ * ChunkCausalAttention.forward, sana_blocks.py:481-485, rotary = identity).
+ *
+ *   k, v          [B][N][h*d] views: element (b, n, c) at b*stride_b + n*stride_n + c
+ *   state         fp32 [B][h][n_chunks][d+1][d], contiguous
+ *   chunk_starts  int32 [n_chunks+1] token offsets (0 = first, N = last), or NULL
+ *                 when n_chunks == 1
+ *   max_chunk_tokens  host value: the longest chunk, in tokens
+ *   workspace     at least sana_hip_linattn_workspace_bytes(...) bytes, 16-byte aligned
+ *                 (may be NULL when that function returns 0)
+ * Accumulation is fp32 and deterministic (fixed summation order, no atomics).
+ */
+size_t sana_hip_linattn_workspace_bytes(int B, int h, int d, int n_chunks, int max_chunk_tokens,
+                                        int io_dtype);
+
+int sana_hip_linattn_state(const void* k, const void* v, float* state,
+                           void* workspace, size_t workspace_bytes,
+                           int B, int N, int h, int d,
+                           int64_t stride_b, int64_t stride_n,
+                           const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+                           int causal, int io_dtype, void* stream);
+
+/* Inclusive prefix sum over the chunk axis of fp32 [B][h][n_chunks][d+1][d],
+ * in place.  The accumulation the streaming pipeline performs on the host side
+ * (diffusion/longsana/pipeline/sana_inference_pipeline.py:242-263). */
+int sana_hip_linattn_chunk_scan(float* state, int B, int h, int d, int n_chunks, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * ReLU linear attention, phase 2: apply the state to relu(q) and divide
+ *
+ *   out[n][i] = sum_j state[i][j] relu(q[n][j])
+ *               / (sum_j state[d][j] relu(q[n][j]) + eps)
+ * with the state of the chunk token n belongs to.
+ *
+ * Replaces `relu(q)`, `out = vk @ q`, `.float()`, the slice/divide of
+ * LiteLA.attn_matmul (sana_blocks.py:248,257-261) and the `.to(dtype)` of
+ * LiteLA.forward (:286); Triton twin vk_q_mm_divide_fwd
+ * (triton_lite_mla_kernels/vk_q_mm_divide_fwd.py:60-164).  eps is a runtime
+ * value (1e-15 class default, 1e-8 inside SanaMSBlock).
+ *
+ *   q    [B][N][h*d] view (q_stride_b, q_stride_n), io dtype
+ *   out  [B][N][h*d] view (o_stride_b, o_stride_n), out_dtype = io dtype or SANA_DT_F32
+ */
+int sana_hip_linattn_apply(const void* q, const float* state, void* out,
+                           int B, int N, int h, int d,
+                           int64_t q_stride_b, int64_t q_stride_n,
+                           int64_t o_stride_b, int64_t o_stride_n,
+                           const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+                           float eps, int io_dtype, int out_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Depthwise 3x3 conv (zero pad 1, stride 1) + bias + SiLU gate, channels-last
+ *
+ *   t[c]  = bias[c] + sum_{dy,dx} u[y+dy][x+dx][c] * w[c][dy+1][dx+1],  c in 0..2*Ch-1
+ *   y[c]  = t[c] * silu(t[Ch + c]),                                     c in 0..Ch-1
+ *
+ * Replaces depth_conv, torch.chunk, glu_act and the multiply of
+ * GLUMBConv._apply_spatial (diffusion/model/nets/basic_modules.py:164-167).
+ *
+ *   u     [BT][H][W][2*Ch] contiguous (the inverted conv's output, channels-last)
+ *   w     [2*Ch][3][3] (= depth_conv.conv.weight [2Ch,1,3,3]), io dtype
+ *   bias  [2*Ch] io dtype, or NULL
+ *   y     [BT][H][W][Ch] contiguous
+ *   round_like_reference != 0 rounds t, silu(t_g) and the product to the io
+ *   dtype one after the other, as the reference's three separate torch ops do;
+ *   0 keeps fp32 until the single final rounding.
+ */
+int sana_hip_dwconv3x3_silu_gate(const void* u, const void* w, const void* bias, void* y,
+                                 int BT, int H, int W, int Ch,
+                                 int round_like_reference, int io_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * GEMM  C[M][N] = epilogue(A[M][K] . W[N][K]^T), bf16 in, fp32 accumulate, bf16 out
+ *
+ * Replaces nn.Linear qkv / proj (sana_blocks.py:270,289) and the 1x1 convs
+ * inverted_conv (+ bias + SiLU) / point_conv (basic_modules.py:163,167).
+ *
+ *   A     [M][K] row-major with row stride lda
+ *   W     [N][K] row-major with row stride ldw  (nn.Linear / 1x1-conv weight layout)
+ *   bias  [N] bf16 or NULL (must be non-NULL for SANA_EPI_BIAS*)
+ *   C     [M][N] row-major with row stride ldc
+ * K must be a multiple of 32; lda, ldw, ldc multiples of 8.
+ */
+int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
+                       int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
+                       int epilogue, void* stream);
+
+/* W8A16: W is int8 [N][K] with a per-output-channel fp32 scale [N].  Each
+ * weight is dequantised in registers as bf16_rne(float(q) * scale[n]) — the same
+ * value as torch's (q.float() * scale).bfloat16() — before the MFMA, so the
+ * result equals sana_hip_gemm_bf16 on the dequantised weight.  No reference
+ * counterpart (the reference has no W8A16 code); the quantiser is defined by the
+ * benchmark configuration. */
+int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias,
+                        void* C, int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
+                        int epilogue, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SANA_HIP_H_ */

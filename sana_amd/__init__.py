@@ -1,0 +1,6 @@
+"""MI355X-native SanaMSBlock hot path: LiteLA linear attention and GLUMBConv
+Mix-FFN as drop-in modules over hand-written gfx950 kernels (C ABI in
+``include/sana_hip.h``, built by ``python -m sana_amd.build``)."""
+from ._lib import LIB_PATH, SanaHipError  # noqa: F401
+
+__all__ = ["LIB_PATH", "SanaHipError"]

@@ -1,0 +1,83 @@
+// Shared device helpers for the gfx950 kernels (wave64, MFMA, bf16/f16 bit tricks).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/sana_hip.h"
+
+namespace sana {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x2_t __attribute__((ext_vector_type(2)));
+
+struct BF16 {};  // tag types for the 16-bit io dtypes
+struct F16 {};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// round-to-nearest-even fp32 -> bf16 bits (NaN stays NaN)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  __bf16 b = (__bf16)f;
+  return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+}
+
+// ReLU on two packed 16-bit floats (bf16 or f16: both sign-magnitude, so a
+// signed-integer max against 0 clears negatives and -0).
+__device__ __forceinline__ uint32_t relu_pk16(uint32_t x) {
+  s16x2_t v = __builtin_bit_cast(s16x2_t, x);
+  s16x2_t z = {0, 0};
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(v, z));
+}
+__device__ __forceinline__ u32x4_t relu_pk16(u32x4_t x) {
+  u32x4_t r;
+  r.x = relu_pk16(x.x);
+  r.y = relu_pk16(x.y);
+  r.z = relu_pk16(x.z);
+  r.w = relu_pk16(x.w);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(u32x4_t a, u32x4_t b, f32x16_t c);
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16<BF16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma_32x32x16<F16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mfma_16x16x32_bf16(u32x4_t a, u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float silu_f32(float g) {
+  // g * sigmoid(g) = g / (1 + exp(-g)); exp via the hardware exp2
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g));
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace sana

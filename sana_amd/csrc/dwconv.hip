@@ -1,0 +1,220 @@
+// Depthwise 3x3 (zero pad 1) + bias + SiLU gate, channels-last, for gfx950.
+//
+//   u [BT][H][W][2*Ch] -> y [BT][H][W][Ch],  y[c] = t[c] * silu(t[Ch+c]),
+//   t[c] = bias[c] + sum_taps u[..][c] * w[c][tap]
+//
+// HBM-bound (no reuse across channels; 9-fold reuse across pixels).  Lanes run
+// along the channel axis: a lane owns the channel pair (c, c+1) of the first
+// half and (Ch+c, Ch+c+1) of the gate half, so a wave reads 256 contiguous
+// bytes per pixel and half.  A wave walks DOWN a strip of TW output columns
+// holding a rolling 3 x (TW+2) pixel window in fp32 registers: every input
+// element is loaded once per strip (plus the two halo columns) and converted
+// once; the next row's loads are in flight while the current row is computed.
+// The four waves of a workgroup take four adjacent strips so that the halo
+// columns hit in the CU's vector L1.
+#include "common.h"
+
+namespace sana {
+namespace {
+
+template <typename T>
+struct Pair;  // two adjacent channels
+template <>
+struct Pair<BF16> {
+  typedef uint32_t raw;
+  static __device__ __forceinline__ raw load(const void* p, int64_t elem) {
+    return *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p) + elem);
+  }
+  static __device__ __forceinline__ float lo(raw r) { return bf16_lo(r); }
+  static __device__ __forceinline__ float hi(raw r) { return bf16_hi(r); }
+  static __device__ __forceinline__ float one(const void* p, int64_t elem) {
+    return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[elem]);
+  }
+  static __device__ __forceinline__ float rnd(float x) { return round_bf16(x); }
+  static __device__ __forceinline__ void store(void* p, int64_t elem, float a, float b) {
+    *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p) + elem) = pack_bf16(a, b);
+  }
+};
+template <>
+struct Pair<F16> {
+  typedef uint32_t raw;
+  static __device__ __forceinline__ raw load(const void* p, int64_t elem) {
+    return *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p) + elem);
+  }
+  static __device__ __forceinline__ float lo(raw r) { return f16_bits_to_f32(r & 0xffffu); }
+  static __device__ __forceinline__ float hi(raw r) { return f16_bits_to_f32(r >> 16); }
+  static __device__ __forceinline__ float one(const void* p, int64_t elem) {
+    return f16_bits_to_f32(static_cast<const uint16_t*>(p)[elem]);
+  }
+  static __device__ __forceinline__ float rnd(float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); }
+  static __device__ __forceinline__ void store(void* p, int64_t elem, float a, float b) {
+    *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p) + elem) = pack_f16(a, b);
+  }
+};
+template <>
+struct Pair<float> {
+  typedef float2 raw;
+  static __device__ __forceinline__ raw load(const void* p, int64_t elem) {
+    return *reinterpret_cast<const float2*>(static_cast<const float*>(p) + elem);
+  }
+  static __device__ __forceinline__ float lo(raw r) { return r.x; }
+  static __device__ __forceinline__ float hi(raw r) { return r.y; }
+  static __device__ __forceinline__ float one(const void* p, int64_t elem) { return static_cast<const float*>(p)[elem]; }
+  static __device__ __forceinline__ float rnd(float x) { return x; }
+  static __device__ __forceinline__ void store(void* p, int64_t elem, float a, float b) {
+    *reinterpret_cast<float2*>(static_cast<float*>(p) + elem) = make_float2(a, b);
+  }
+};
+
+// grid: x = channel slabs of 128, y = x-groups (4 strips) * row bands, z = BT; block 256
+template <typename T, int TW, bool ROUND>
+__global__ __launch_bounds__(256) void dwconv_gate_kernel(const void* __restrict__ u, const void* __restrict__ w,
+                                                          const void* __restrict__ bias, void* __restrict__ y,
+                                                          int H, int W, int Ch, int R, int xgroups) {
+  typedef Pair<T> P;
+  typedef typename P::raw raw_t;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 128 + 2 * lane;
+  const int xg = blockIdx.y % xgroups, band = blockIdx.y / xgroups;
+  const int x0 = (xg * 4 + wave) * TW;
+  if (c >= Ch || x0 >= W) return;  // no barriers in this kernel
+  const int y0 = band * R, y1 = min(H, y0 + R);
+  const int C2 = 2 * Ch;
+  const int64_t img = (int64_t)blockIdx.z * H * W;
+
+  // filter taps and bias for the four channels of this lane: [a0, a1, g0, g1]
+  float wt[4][9], bs[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int ch = c + (q & 1) + (q >> 1) * Ch;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) wt[q][t] = P::one(w, (int64_t)ch * 9 + t);
+    bs[q] = bias ? P::one(bias, ch) : 0.f;
+  }
+
+  float win[3][TW + 2][4];
+  raw_t ra[TW + 2], rg[TW + 2];
+  bool rok[TW + 2];
+  // column validity is row independent
+  bool colok[TW + 2];
+#pragma unroll
+  for (int i = 0; i < TW + 2; ++i) colok[i] = (x0 - 1 + i >= 0) && (x0 - 1 + i < W);
+
+  // loads always hit a valid (clamped) address; out-of-image taps are zeroed at commit
+  auto issue = [&](int yy) {
+    const bool rowok = yy >= 0 && yy < H && yy <= y1;  // rows past the band's lower halo are never used
+    const int yc = min(max(yy, 0), H - 1);
+#pragma unroll
+    for (int i = 0; i < TW + 2; ++i) {
+      rok[i] = rowok && colok[i];
+      const int xc = min(max(x0 - 1 + i, 0), W - 1);
+      const int64_t e = (img + (int64_t)yc * W + xc) * C2 + c;
+      ra[i] = P::load(u, e);
+      rg[i] = P::load(u, e + Ch);
+    }
+  };
+  auto commit = [&](float (&row)[TW + 2][4]) {
+#pragma unroll
+    for (int i = 0; i < TW + 2; ++i) {
+      row[i][0] = rok[i] ? P::lo(ra[i]) : 0.f;
+      row[i][1] = rok[i] ? P::hi(ra[i]) : 0.f;
+      row[i][2] = rok[i] ? P::lo(rg[i]) : 0.f;
+      row[i][3] = rok[i] ? P::hi(rg[i]) : 0.f;
+    }
+  };
+  auto compute = [&](int yo, const float (&top)[TW + 2][4], const float (&mid)[TW + 2][4],
+                     const float (&bot)[TW + 2][4]) {
+#pragma unroll
+    for (int x = 0; x < TW; ++x) {
+      if (x0 + x >= W) break;
+      float acc[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float a = bs[q];
+#pragma unroll
+        for (int dx = 0; dx < 3; ++dx) {
+          a = fmaf(top[x + dx][q], wt[q][dx], a);
+          a = fmaf(mid[x + dx][q], wt[q][3 + dx], a);
+          a = fmaf(bot[x + dx][q], wt[q][6 + dx], a);
+        }
+        acc[q] = a;
+      }
+      float o0, o1;
+      if (ROUND) {
+        // the reference rounds after the conv, after SiLU and after the product
+        const float a0 = P::rnd(acc[0]), a1 = P::rnd(acc[1]);
+        const float g0 = P::rnd(acc[2]), g1 = P::rnd(acc[3]);
+        o0 = a0 * P::rnd(silu_f32(g0));
+        o1 = a1 * P::rnd(silu_f32(g1));
+      } else {
+        o0 = acc[0] * silu_f32(acc[2]);
+        o1 = acc[1] * silu_f32(acc[3]);
+      }
+      P::store(y, (img + (int64_t)yo * W + (x0 + x)) * Ch + c, o0, o1);
+    }
+  };
+
+  // prologue: rows y0-1 and y0 in the window, row y0+1 in flight
+  issue(y0 - 1);
+  commit(win[0]);
+  issue(y0);
+  commit(win[1]);
+  issue(y0 + 1);
+  for (int yo = y0; yo < y1; yo += 3) {
+    // sub-step s: window rows (top, mid, bot) = win[s], win[s+1], win[s+2] (mod 3)
+    commit(win[2]);
+    issue(yo + 2);
+    compute(yo, win[0], win[1], win[2]);
+    if (yo + 1 >= y1) break;
+    commit(win[0]);
+    issue(yo + 3);
+    compute(yo + 1, win[1], win[2], win[0]);
+    if (yo + 2 >= y1) break;
+    commit(win[1]);
+    issue(yo + 4);
+    compute(yo + 2, win[2], win[0], win[1]);
+  }
+}
+
+template <typename T, int TW>
+int launch(const void* u, const void* w, const void* bias, void* y, int BT, int H, int W, int Ch, int round_ref,
+           hipStream_t s) {
+  const int slabs = (Ch + 127) / 128;
+  const int xgroups = (W + 4 * TW - 1) / (4 * TW);
+  // pick the band height so that the launch has enough waves to fill 256 CUs,
+  // but keep bands >= 4 rows (two halo rows are re-read per band)
+  int R = H;
+  const int64_t strips = (int64_t)slabs * ((W + TW - 1) / TW) * BT;
+  while (R > 4 && strips * ((H + R - 1) / R) < 6144) R = (R + 1) / 2;
+  const int bands = (H + R - 1) / R;
+  if ((int64_t)xgroups * bands > 65535 || BT > 65535) return SANA_ERR_SHAPE;
+  dim3 grid(slabs, xgroups * bands, BT);
+  if (round_ref)
+    hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, true>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+  else
+    hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, false>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+}  // namespace
+}  // namespace sana
+
+using namespace sana;
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_dwconv3x3_silu_gate(
+    const void* u, const void* w, const void* bias, void* y, int BT, int H, int W, int Ch, int round_like_reference,
+    int io_dtype, void* stream) {
+  if (!u || !w || !y || BT <= 0 || H <= 0 || W <= 0 || Ch <= 0) return SANA_ERR_ARG;
+  if (Ch & 1) return SANA_ERR_SHAPE;  // a lane owns a channel pair
+  const int esz = io_dtype == SANA_DT_F32 ? 4 : 2;
+  const uintptr_t mask = 2 * esz - 1;
+  if ((reinterpret_cast<uintptr_t>(u) & mask) || (reinterpret_cast<uintptr_t>(y) & mask)) return SANA_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  constexpr int TW = 4;
+  switch (io_dtype) {
+    case SANA_DT_BF16: return launch<BF16, TW>(u, w, bias, y, BT, H, W, Ch, round_like_reference, s);
+    case SANA_DT_F16: return launch<F16, TW>(u, w, bias, y, BT, H, W, Ch, round_like_reference, s);
+    case SANA_DT_F32: return launch<float, TW>(u, w, bias, y, BT, H, W, Ch, round_like_reference, s);
+    default: return SANA_ERR_DTYPE;
+  }
+}

@@ -1,0 +1,582 @@
+// ReLU linear attention for gfx950: phase 1 (state = [V|1]^T relu(K) per head),
+// split reduction + chunk prefix scan, phase 2 (apply to relu(Q), divide).
+//
+// Data layout: q, k, v and out are token-major [B][N][h*32] views (channel
+// stride 1).  The state is fp32 [B][h][n_chunks][33][32]; row 32 holds
+// sum_n relu(k_n).
+//
+// 16-bit io (bf16 / f16)
+//   phase 1  one workgroup = (batch, pair of heads, chunk, token split); its four
+//            waves take interleaved 32-token tiles.  A tile is loaded with
+//            16-byte coalesced loads, written to wave-private LDS and read back
+//            transposed (token-contiguous per channel) as MFMA 32x32x16
+//            operands: S += V^T K and ksum += 1^T K.  Waves are summed in LDS.
+//   phase 2  one wave = (pair of heads, token range); the fp32 state is split
+//            into three bf16 terms (hi + mid + lo = all 24 mantissa bits) and
+//            applied with MFMA 16x16x32; rows 32..47 of the A operand all carry
+//            ksum so every lane gets its token's denominator in-lane.
+// fp32 io (and f16 phase 2) uses MFMA 32x32x2 f32 directly from global memory.
+#include <type_traits>
+
+#include "common.h"
+
+namespace sana {
+namespace {
+
+constexpr int D = 32;
+constexpr int STATE_ELEMS = (D + 1) * D;  // 1056
+constexpr int TILE = 32;                  // tokens per phase-1 tile
+
+struct ChunkRange {
+  int begin, end;
+};
+__device__ __forceinline__ ChunkRange chunk_range(const int32_t* chunk_starts, int c, int N) {
+  ChunkRange r;
+  if (chunk_starts) {
+    r.begin = chunk_starts[c];
+    r.end = chunk_starts[c + 1];
+  } else {
+    r.begin = 0;
+    r.end = N;
+  }
+  return r;
+}
+
+// ----------------------------------------------------------------------------
+// phase 1, 16-bit io
+// grid: x = nsplit, y = n_chunks, z = B * pairs;  block 256
+// dst: when nsplit == 1 the final state, else partial[(bh*n_chunks + c)*nsplit + split][1056]
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void linattn_state16_kernel(
+    const uint16_t* __restrict__ K, const uint16_t* __restrict__ V, float* __restrict__ dst,
+    const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int nsplit, int split_tokens,
+    int64_t stride_b, int64_t stride_n) {
+  // staging: per wave K tile [32 tok][64 ch] + V tile, 16-bit -> 8 KB per wave.
+  // reduction: per wave 2 heads x 1056 fp32 -> 8448 B per wave.  The two uses
+  // never overlap in time, so they share one buffer.
+  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * 2 * STATE_ELEMS * 4];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int pairs = (h + 1) >> 1;
+  const int b = blockIdx.z / pairs, p = blockIdx.z % pairs;
+  const int c = blockIdx.y, split = blockIdx.x;
+  const int C = h * D;
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + split * split_tokens;
+  const int t1 = min(cr.end, t0 + split_tokens);
+
+  uint16_t* stage = reinterpret_cast<uint16_t*>(smem) + wave * (2 * TILE * 64);
+  uint16_t* lds_k = stage;
+  uint16_t* lds_v = stage + TILE * 64;
+
+  // load mapping: lane -> token (lane/8 + 8*i), 16-byte channel chunk lane%8
+  const int ld_tok = lane >> 3;
+  const int ld_ch = p * 64 + (lane & 7) * 8;
+  const bool ch_ok = ld_ch < C;
+  const uint16_t* kbase = K + (int64_t)b * stride_b + ld_ch;
+  const uint16_t* vbase = V + (int64_t)b * stride_b + ld_ch;
+
+  f32x16_t accS[2], accK[2];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    accS[0][i] = 0.f;
+    accS[1][i] = 0.f;
+    accK[0][i] = 0.f;
+    accK[1][i] = 0.f;
+  }
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  const uint32_t one2 = std::is_same<T, BF16>::value ? 0x3f803f80u : 0x3c003c00u;
+  const u32x4_t ones = {one2, one2, one2, one2};
+
+  u32x4_t kreg[4], vreg[4];
+  auto issue_loads = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tok = tile + ld_tok + 8 * i;
+      if (ch_ok && tok < t1) {
+        kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n);
+        vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n);
+      } else {
+        kreg[i] = zero4;
+        vreg[i] = zero4;
+      }
+    }
+  };
+
+  int tile = t0 + wave * TILE;
+  if (tile < t1) issue_loads(tile);
+  // operand read mapping: lane -> channel j = lane%32 (of head hh), k-group g = lane/32;
+  // element r of k-step s is token 16*s + 2*r + g of the tile (any bijection works as
+  // long as both operands use the same one: the MFMA contracts over tokens).
+  const int j = lane & 31, g = lane >> 5;
+  for (; tile < t1; tile += 4 * TILE) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4_t*>(lds_k + (ld_tok + 8 * i) * 64 + (lane & 7) * 8) = relu_pk16(kreg[i]);
+      *reinterpret_cast<u32x4_t*>(lds_v + (ld_tok + 8 * i) * 64 + (lane & 7) * 8) = vreg[i];
+    }
+    if (tile + 4 * TILE < t1) issue_loads(tile + 4 * TILE);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        u32x4_t fk, fv;
+#pragma unroll
+        for (int r2 = 0; r2 < 4; ++r2) {
+          const int ta = 16 * s + 2 * (2 * r2) + g, tb = 16 * s + 2 * (2 * r2 + 1) + g;
+          const uint32_t klo = lds_k[ta * 64 + hh * 32 + j], khi = lds_k[tb * 64 + hh * 32 + j];
+          const uint32_t vlo = lds_v[ta * 64 + hh * 32 + j], vhi = lds_v[tb * 64 + hh * 32 + j];
+          fk[r2] = klo | (khi << 16);
+          fv[r2] = vlo | (vhi << 16);
+        }
+        accS[hh] = mfma_32x32x16<T>(fv, fk, accS[hh]);    // S[i][j] += sum_tok V[tok][i] K[tok][j]
+        accK[hh] = mfma_32x32x16<T>(ones, fk, accK[hh]);  // every row: sum_tok K[tok][j]
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites
+  }
+
+  // cross-wave reduction in LDS.  D layout of 32x32 MFMA: lane -> column j = lane%32,
+  // register r -> row 8*(r/4) + 4*(lane/32) + r%4.
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem) + wave * (2 * STATE_ELEMS);
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 8 * (r >> 2) + 4 * g + (r & 3);
+      red[hh * STATE_ELEMS + row * D + j] = accS[hh][r];
+    }
+    if (g == 0) red[hh * STATE_ELEMS + D * D + j] = accK[hh][0];
+  }
+  __syncthreads();
+  const float* all = reinterpret_cast<const float*>(smem);
+  for (int e = tid; e < 2 * STATE_ELEMS; e += 256) {
+    const int hh = e / STATE_ELEMS, idx = e - hh * STATE_ELEMS;
+    const int head = 2 * p + hh;
+    if (head >= h) continue;
+    const float sum = ((all[e] + all[2 * STATE_ELEMS + e]) + all[4 * STATE_ELEMS + e]) + all[6 * STATE_ELEMS + e];
+    const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nsplit + split;
+    dst[slot * STATE_ELEMS + idx] = sum;
+  }
+}
+
+// ----------------------------------------------------------------------------
+// phase 1, fp32 io: MFMA 32x32x2 f32 straight from global memory.
+// grid: x = nsplit, y = n_chunks, z = B * ceil(h/4); block 256, wave = one head.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void linattn_state32_kernel(
+    const float* __restrict__ K, const float* __restrict__ V, float* __restrict__ dst,
+    const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int nsplit, int split_tokens,
+    int64_t stride_b, int64_t stride_n) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int groups = (h + 3) >> 2;
+  const int b = blockIdx.z / groups, head = (blockIdx.z % groups) * 4 + wave;
+  if (head >= h) return;  // no barriers below
+  const int c = blockIdx.y, split = blockIdx.x;
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + split * split_tokens;
+  const int t1 = min(cr.end, t0 + split_tokens);
+  const int j = lane & 31, g = lane >> 5;
+  const float* kp = K + (int64_t)b * stride_b + head * D + j;
+  const float* vp = V + (int64_t)b * stride_b + head * D + j;
+  f32x16_t accS, accK;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    accS[i] = 0.f;
+    accK[i] = 0.f;
+  }
+  constexpr int U = 8;  // 16 tokens in flight per wave
+  for (int t = t0; t < t1; t += 2 * U) {
+    float kk[U], vv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tok = t + 2 * u + g;
+      const bool ok = tok < t1;
+      kk[u] = ok ? fmaxf(kp[(int64_t)tok * stride_n], 0.f) : 0.f;
+      vv[u] = ok ? vp[(int64_t)tok * stride_n] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      accS = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[u], kk[u], accS, 0, 0, 0);
+      accK = __builtin_amdgcn_mfma_f32_32x32x2f32(1.0f, kk[u], accK, 0, 0, 0);
+    }
+  }
+  const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nsplit + split;
+  float* o = dst + slot * STATE_ELEMS;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) o[(8 * (r >> 2) + 4 * g + (r & 3)) * D + j] = accS[r];
+  if (g == 0) o[D * D + j] = accK[0];
+}
+
+// ----------------------------------------------------------------------------
+// split reduction (+ inclusive prefix over chunks when causal).
+// One thread per (b*h, element); fixed summation order.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void linattn_reduce_scan_kernel(const float* __restrict__ partial,
+                                                                  float* __restrict__ state, int BH,
+                                                                  int n_chunks, int nsplit, int causal) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (int64_t)BH * STATE_ELEMS) return;
+  const int64_t bh = gid / STATE_ELEMS;
+  const int e = (int)(gid - bh * STATE_ELEMS);
+  float run = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const int64_t slot0 = (bh * n_chunks + c) * nsplit;
+    float s = partial[slot0 * STATE_ELEMS + e];
+    for (int sp = 1; sp < nsplit; ++sp) s += partial[(slot0 + sp) * STATE_ELEMS + e];
+    if (causal) {
+      run += s;
+      s = run;
+    }
+    state[(bh * n_chunks + c) * STATE_ELEMS + e] = s;
+  }
+}
+
+// ----------------------------------------------------------------------------
+// phase 2, bf16 io.  grid: x = token ranges per chunk, y = n_chunks,
+// z = B * ceil(pairs/4); block 256; wave = pair of heads.
+// ----------------------------------------------------------------------------
+struct SplitState {     // A operands of one head: 3 row blocks x 3 bf16 terms
+  u32x4_t a[3][3];
+};
+
+__device__ __forceinline__ void split3(const float x[8], u32x4_t out[3]) {
+  float r1[8], r2[8];
+  uint32_t hi[8], mid[8], lo[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    hi[e] = f32_to_bf16_bits(x[e]);
+    r1[e] = x[e] - bf16_bits_to_f32(hi[e]);
+    mid[e] = f32_to_bf16_bits(r1[e]);
+    r2[e] = r1[e] - bf16_bits_to_f32(mid[e]);
+    lo[e] = f32_to_bf16_bits(r2[e]);
+  }
+#pragma unroll
+  for (int e2 = 0; e2 < 4; ++e2) {
+    out[0][e2] = hi[2 * e2] | (hi[2 * e2 + 1] << 16);
+    out[1][e2] = mid[2 * e2] | (mid[2 * e2 + 1] << 16);
+    out[2][e2] = lo[2 * e2] | (lo[2 * e2 + 1] << 16);
+  }
+}
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
+    const uint16_t* __restrict__ Q, const float* __restrict__ state, void* __restrict__ out,
+    const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int wg_tokens,
+    int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pairs = (h + 1) >> 1;
+  const int pgroups = (pairs + 3) >> 2;
+  const int b = blockIdx.z / pgroups, p = (blockIdx.z % pgroups) * 4 + wave;
+  if (p >= pairs) return;  // no barriers below
+  const int c = blockIdx.y;
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + blockIdx.x * wg_tokens;
+  const int t1 = min(cr.end, t0 + wg_tokens);
+  if (t0 >= t1) return;
+  const int n = lane & 15, g = lane >> 4;
+  const int nheads = (2 * p + 1 < h) ? 2 : 1;
+
+  // A operands.  MFMA 16x16x32: A lane -> row lane%16, k = 8*(lane/16)+e.  Output
+  // lane (token n, g') register s of row block rb is row 4*g'+s; we place channel
+  // 8*(r/4) + 4*rb + r%4 in row r so that a lane ends up with 8 contiguous channels.
+  SplitState st[2];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {
+    const int head = min(2 * p + hh, h - 1);
+    const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * STATE_ELEMS;
+#pragma unroll
+    for (int rb = 0; rb < 3; ++rb) {
+      const int row = (rb < 2) ? (8 * (n >> 2) + 4 * rb + (n & 3)) : D;
+      const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(sp + row * D + 8 * g);
+      const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(sp + row * D + 8 * g + 4);
+      const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+      split3(x, st[hh].a[rb]);
+    }
+  }
+
+  const uint16_t* qp = Q + (int64_t)b * q_stride_b + p * 64 + 8 * g;
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  constexpr int U = 4;  // 16-token steps in flight
+  for (int t = t0; t < t1; t += 16 * U) {
+    u32x4_t qf[U][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tok = t + 16 * u + n;
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        qf[u][hh] = (tok < t1 && hh < nheads)
+                        ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + hh * D)
+                        : zero4;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tok = t + 16 * u + n;
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const u32x4_t qb = relu_pk16(qf[u][hh]);
+        f32x4_t acc[3];
+#pragma unroll
+        for (int rb = 0; rb < 3; ++rb) {
+          f32x4_t a = {0.f, 0.f, 0.f, 0.f};
+          a = mfma_16x16x32_bf16(st[hh].a[rb][2], qb, a);  // smallest term first
+          a = mfma_16x16x32_bf16(st[hh].a[rb][1], qb, a);
+          a = mfma_16x16x32_bf16(st[hh].a[rb][0], qb, a);
+          acc[rb] = a;
+        }
+        if (tok < t1 && hh < nheads) {
+          const float den = acc[2][0] + eps;
+          const int64_t o_off = (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + p * 64 + hh * D + 8 * g;
+          if (OUT_F32) {
+            f32x4_t o0, o1;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              o0[s] = acc[0][s] / den;
+              o1[s] = acc[1][s] / den;
+            }
+            float* op = reinterpret_cast<float*>(out) + o_off;
+            *reinterpret_cast<f32x4_t*>(op) = o0;
+            *reinterpret_cast<f32x4_t*>(op + 4) = o1;
+          } else {
+            const float inv = __builtin_amdgcn_rcpf(den);
+            u32x4_t o;
+            o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
+            o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
+            o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
+            o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + o_off) = o;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// phase 2, fp32 / f16 io: MFMA 32x32x2 f32.  grid as above but wave = one head,
+// z = B * ceil(h/4).  A lane -> state row lane%32, contraction index 16*(lane/32)+s;
+// B lane -> token lane%32, same contraction index.  The denominator MFMA uses the
+// ksum row in every A row, so the divide is lane-local.
+// ----------------------------------------------------------------------------
+template <typename TIn, typename TOut>
+__device__ __forceinline__ TOut cvt_out(float x);
+template <>
+__device__ __forceinline__ float cvt_out<float, float>(float x) { return x; }
+template <>
+__device__ __forceinline__ float cvt_out<_Float16, float>(float x) { return x; }
+template <>
+__device__ __forceinline__ _Float16 cvt_out<_Float16, _Float16>(float x) { return (_Float16)x; }
+
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256) void linattn_apply32_kernel(
+    const TIn* __restrict__ Q, const float* __restrict__ state, TOut* __restrict__ out,
+    const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int wg_tokens,
+    int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int groups = (h + 3) >> 2;
+  const int b = blockIdx.z / groups, head = (blockIdx.z % groups) * 4 + wave;
+  if (head >= h) return;
+  const int c = blockIdx.y;
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + blockIdx.x * wg_tokens;
+  const int t1 = min(cr.end, t0 + wg_tokens);
+  if (t0 >= t1) return;
+  const int n = lane & 31, g = lane >> 5;
+  const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * STATE_ELEMS;
+  float a_num[16], a_den[16];
+#pragma unroll
+  for (int s = 0; s < 16; ++s) {
+    a_num[s] = sp[n * D + 16 * g + s];
+    a_den[s] = sp[D * D + 16 * g + s];
+  }
+  for (int t = t0; t < t1; t += 32) {
+    const int tok = t + n;
+    const bool ok = tok < t1;
+    float qv[16];
+    const TIn* qp = Q + (int64_t)b * q_stride_b + (int64_t)tok * q_stride_n + head * D + 16 * g;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) qv[s] = ok ? fmaxf((float)qp[s], 0.f) : 0.f;
+    f32x16_t num, den;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      num[i] = 0.f;
+      den[i] = 0.f;
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      num = __builtin_amdgcn_mfma_f32_32x32x2f32(a_num[s], qv[s], num, 0, 0, 0);
+      den = __builtin_amdgcn_mfma_f32_32x32x2f32(a_den[s], qv[s], den, 0, 0, 0);
+    }
+    if (ok) {
+      // D layout: lane -> token (column) lane%32; register r -> channel 8*(r/4)+4*g+r%4
+      const float dd = den[0] + eps;
+      TOut* op = out + (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + head * D;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) op[8 * (r >> 2) + 4 * g + (r & 3)] = cvt_out<TIn, TOut>(num[r] / dd);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------- host side
+
+int pick_nsplit(int items, int max_chunk_tokens, int min_tokens) {
+  // aim for >= 512 workgroups, but keep >= min_tokens tokens per split
+  int ns = (512 + items - 1) / items;
+  const int cap = (max_chunk_tokens + min_tokens - 1) / min_tokens;
+  if (ns > cap) ns = cap;
+  if (ns < 1) ns = 1;
+  if (ns > 64) ns = 64;
+  return ns;
+}
+int split_len(int max_chunk_tokens, int nsplit, int granule) {
+  int len = (max_chunk_tokens + nsplit - 1) / nsplit;
+  return (len + granule - 1) / granule * granule;
+}
+
+struct StatePlan {
+  int items;   // workgroups before splitting
+  int nsplit;
+  int split_tokens;
+};
+StatePlan plan_state(int B, int h, int n_chunks, int max_chunk_tokens, int io_dtype) {
+  StatePlan pl;
+  const int per_b = (io_dtype == SANA_DT_F32) ? (h + 3) / 4 : (h + 1) / 2;
+  pl.items = B * per_b * n_chunks;
+  // 16-bit: four waves x 32-token tiles per round; fp32: 16 tokens per wave iteration
+  const bool f32 = io_dtype == SANA_DT_F32;
+  pl.nsplit = pick_nsplit(pl.items, max_chunk_tokens, f32 ? 64 : 256);
+  pl.split_tokens = split_len(max_chunk_tokens, pl.nsplit, f32 ? 16 : 128);
+  // drop splits that would be empty after rounding the length up
+  pl.nsplit = (max_chunk_tokens + pl.split_tokens - 1) / pl.split_tokens;
+  if (pl.nsplit < 1) pl.nsplit = 1;
+  return pl;
+}
+
+}  // namespace
+}  // namespace sana
+
+using namespace sana;
+
+extern "C" __attribute__((visibility("default"))) size_t sana_hip_linattn_workspace_bytes(int B, int h, int d,
+                                                                                          int n_chunks,
+                                                                                          int max_chunk_tokens,
+                                                                                          int io_dtype) {
+  if (B <= 0 || h <= 0 || d != D || n_chunks <= 0 || max_chunk_tokens <= 0) return 0;
+  const StatePlan pl = plan_state(B, h, n_chunks, max_chunk_tokens, io_dtype);
+  return pl.nsplit > 1 ? (size_t)B * h * n_chunks * pl.nsplit * STATE_ELEMS * sizeof(float) : 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(const void* k, const void* v, float* state, void* workspace,
+                                      size_t workspace_bytes, int B, int N, int h, int d, int64_t stride_b,
+                                      int64_t stride_n, const int32_t* chunk_starts, int n_chunks,
+                                      int max_chunk_tokens, int causal, int io_dtype, void* stream) {
+  if (!k || !v || !state || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  if (d != D) return SANA_ERR_SHAPE;
+  if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
+  if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
+  if (max_chunk_tokens <= 0 || max_chunk_tokens > N) return SANA_ERR_ARG;
+  if (io_dtype != SANA_DT_F32 && io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
+  if (stride_n < (int64_t)h * D || stride_b < 0) return SANA_ERR_ARG;
+  if ((int64_t)B * h > (1 << 22) || n_chunks > 65535) return SANA_ERR_SHAPE;
+  const int esz = io_dtype == SANA_DT_F32 ? 4 : 2;
+  if (!aligned16(k) || !aligned16(v) || !aligned16(state) || (stride_n * esz) % 16 || (stride_b * esz) % 16)
+    return SANA_ERR_ALIGN;
+  const StatePlan pl = plan_state(B, h, n_chunks, max_chunk_tokens, io_dtype);
+  float* dst = state;
+  if (pl.nsplit > 1) {
+    const size_t need = (size_t)B * h * n_chunks * pl.nsplit * STATE_ELEMS * sizeof(float);
+    if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return SANA_ERR_ALIGN;
+    dst = static_cast<float*>(workspace);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (io_dtype == SANA_DT_F32) {
+    dim3 grid(pl.nsplit, n_chunks, B * ((h + 3) / 4));
+    hipLaunchKernelGGL(linattn_state32_kernel, grid, dim3(256), 0, s, static_cast<const float*>(k),
+                       static_cast<const float*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
+                       pl.split_tokens, stride_b, stride_n);
+  } else {
+    dim3 grid(pl.nsplit, n_chunks, B * ((h + 1) / 2));
+    if (io_dtype == SANA_DT_BF16)
+      hipLaunchKernelGGL(linattn_state16_kernel<BF16>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
+                         static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
+                         pl.split_tokens, stride_b, stride_n);
+    else
+      hipLaunchKernelGGL(linattn_state16_kernel<F16>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
+                         static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
+                         pl.split_tokens, stride_b, stride_n);
+  }
+  if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+  const bool scan = causal && n_chunks > 1;
+  if (pl.nsplit > 1 || scan) {
+    const int64_t threads = (int64_t)B * h * STATE_ELEMS;
+    hipLaunchKernelGGL(linattn_reduce_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, dst,
+                       state, B * h, n_chunks, pl.nsplit, scan ? 1 : 0);
+    if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+  }
+  return SANA_OK;
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_chunk_scan(float* state, int B, int h, int d, int n_chunks, void* stream) {
+  if (!state || B <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  if (d != D) return SANA_ERR_SHAPE;
+  if (n_chunks == 1) return SANA_OK;
+  const int64_t threads = (int64_t)B * h * STATE_ELEMS;
+  hipLaunchKernelGGL(linattn_reduce_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), state, state, B * h, n_chunks, 1, 1);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(const void* q, const float* state, void* out, int B, int N, int h, int d,
+                                      int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b,
+                                      int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks,
+                                      int max_chunk_tokens, float eps, int io_dtype, int out_dtype, void* stream) {
+  if (!q || !state || !out || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  if (d != D) return SANA_ERR_SHAPE;
+  if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
+  if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
+  if (max_chunk_tokens <= 0 || max_chunk_tokens > N) return SANA_ERR_ARG;
+  if (io_dtype != SANA_DT_F32 && io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
+  if (out_dtype != io_dtype && out_dtype != SANA_DT_F32) return SANA_ERR_DTYPE;
+  if (q_stride_n < (int64_t)h * D || o_stride_n < (int64_t)h * D || q_stride_b < 0 || o_stride_b < 0)
+    return SANA_ERR_ARG;
+  if ((int64_t)B * h > (1 << 22) || n_chunks > 65535) return SANA_ERR_SHAPE;
+  const int qsz = io_dtype == SANA_DT_F32 ? 4 : 2, osz = out_dtype == SANA_DT_F32 ? 4 : 2;
+  if (!aligned16(q) || !aligned16(state) || !aligned16(out) || (q_stride_n * qsz) % 16 || (q_stride_b * qsz) % 16 ||
+      (o_stride_n * osz) % 16 || (o_stride_b * osz) % 16)
+    return SANA_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int wg_tokens = io_dtype == SANA_DT_BF16 ? 256 : 64;
+  const unsigned gx = (unsigned)((max_chunk_tokens + wg_tokens - 1) / wg_tokens);
+  if (io_dtype == SANA_DT_BF16) {
+    const int pairs = (h + 1) / 2;
+    dim3 grid(gx, n_chunks, B * ((pairs + 3) / 4));
+    if (out_dtype == SANA_DT_F32)
+      hipLaunchKernelGGL(linattn_apply_bf16_kernel<true>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(q),
+                         state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,
+                         o_stride_n, eps);
+    else
+      hipLaunchKernelGGL(linattn_apply_bf16_kernel<false>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(q),
+                         state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,
+                         o_stride_n, eps);
+  } else {
+    dim3 grid(gx, n_chunks, B * ((h + 3) / 4));
+    if (io_dtype == SANA_DT_F32)
+      hipLaunchKernelGGL((linattn_apply32_kernel<float, float>), grid, dim3(256), 0, s, static_cast<const float*>(q),
+                         state, static_cast<float*>(out), chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b,
+                         q_stride_n, o_stride_b, o_stride_n, eps);
+    else if (out_dtype == SANA_DT_F32)
+      hipLaunchKernelGGL((linattn_apply32_kernel<_Float16, float>), grid, dim3(256), 0, s,
+                         static_cast<const _Float16*>(q), state, static_cast<float*>(out), chunk_starts, N, h,
+                         n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps);
+    else
+      hipLaunchKernelGGL((linattn_apply32_kernel<_Float16, _Float16>), grid, dim3(256), 0, s,
+                         static_cast<const _Float16*>(q), state, static_cast<_Float16*>(out), chunk_starts, N, h,
+                         n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps);
+  }
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}

@@ -1,0 +1,220 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype/device checks, pointer and
+stride extraction, launch on torch's current stream.  Forward only, no autograd.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import DT_BF16, DT_F16, DT_F32, SanaHipError
+
+_DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
+HEAD_DIM = 32
+
+_workspaces = {}     # (device index) -> uint8 tensor, grown on demand
+_chunk_tables = {}   # (device index, tuple) -> int32 tensor
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise SanaHipError(f"unsupported dtype {t.dtype}") from None
+
+
+def _need_cuda(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise SanaHipError("the HIP kernels need device tensors (no CPU path exists)")
+
+
+def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    if nbytes == 0:
+        return None
+    key = device.index
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def chunk_table(chunk_tokens: Optional[Sequence[int]], N: int, device) -> Tuple[Optional[torch.Tensor], int, int]:
+    """chunk_tokens: token offsets of chunk starts (first is 0).  Returns
+    (int32 device tensor [n+1] or None, n_chunks, longest chunk)."""
+    if chunk_tokens is None or len(chunk_tokens) <= 1:
+        return None, 1, N
+    starts = list(chunk_tokens) + [N]
+    if starts[0] != 0 or any(b <= a for a, b in zip(starts[:-1], starts[1:])):
+        raise SanaHipError(f"chunk starts must begin at 0 and increase strictly below N={N}: {chunk_tokens}")
+    key = (torch.device(device).index, tuple(starts))
+    tab = _chunk_tables.get(key)
+    if tab is None:
+        tab = torch.tensor(starts, dtype=torch.int32, device=device)
+        _chunk_tables[key] = tab
+    return tab, len(starts) - 1, max(b - a for a, b in zip(starts[:-1], starts[1:]))
+
+
+def _token_major_view(t: torch.Tensor, what: str) -> Tuple[int, int]:
+    """t: [B, N, C] with unit channel stride -> (stride_b, stride_n) in elements."""
+    if t.dim() != 3 or t.stride(2) != 1:
+        raise SanaHipError(f"{what} must be a [B, N, C] view with unit channel stride, got strides {t.stride()}")
+    return t.stride(0), t.stride(1)
+
+
+def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False) -> torch.Tensor:
+    """Phase 1.  k, v: [B, N, C] token-major views (C = h*32).  Returns the fp32
+    state [B, h, n_chunks, 33, 32] (inclusive prefix over chunks when causal)."""
+    _need_cuda(k, v)
+    if k.shape != v.shape or k.dtype != v.dtype or k.stride() != v.stride():
+        raise SanaHipError("k and v must share shape, dtype and strides")
+    B, N, C = k.shape
+    if C % HEAD_DIM:
+        raise SanaHipError(f"C={C} is not a multiple of head_dim {HEAD_DIM}")
+    h = C // HEAD_DIM
+    sb, sn = _token_major_view(k, "k")
+    tab, n_chunks, longest = chunk_table(chunk_tokens, N, k.device)
+    lib = _lib.load()
+    state = torch.empty(B, h, n_chunks, HEAD_DIM + 1, HEAD_DIM, dtype=torch.float32, device=k.device)
+    nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, HEAD_DIM, n_chunks, longest, _dt(k))
+    ws = _workspace(k.device, nbytes)
+    code = lib.sana_hip_linattn_state(
+        k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
+        B, N, h, HEAD_DIM, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
+        1 if causal else 0, _dt(k), _stream())
+    _lib.check(code, "sana_hip_linattn_state")
+    return state
+
+
+def linattn_chunk_scan_(state: torch.Tensor) -> torch.Tensor:
+    """In-place inclusive prefix sum over the chunk axis of [B, h, n_chunks, 33, 32] fp32."""
+    _need_cuda(state)
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 5:
+        raise SanaHipError("state must be contiguous fp32 [B, h, n_chunks, 33, 32]")
+    B, h, n_chunks = state.shape[:3]
+    code = _lib.load().sana_hip_linattn_chunk_scan(state.data_ptr(), B, h, HEAD_DIM, n_chunks, _stream())
+    _lib.check(code, "sana_hip_linattn_chunk_scan")
+    return state
+
+
+def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens=None,
+                  out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Phase 2.  q: [B, N, C] token-major view; state from :func:`linattn_state`.
+    Returns [B, N, C] in ``out_dtype`` (q's dtype or fp32)."""
+    _need_cuda(q, state)
+    B, N, C = q.shape
+    h = C // HEAD_DIM
+    qsb, qsn = _token_major_view(q, "q")
+    tab, n_chunks, longest = chunk_table(chunk_tokens, N, q.device)
+    if state.dtype != torch.float32 or not state.is_contiguous() or \
+            tuple(state.shape) != (B, h, n_chunks, HEAD_DIM + 1, HEAD_DIM):
+        raise SanaHipError(f"state must be contiguous fp32 {(B, h, n_chunks, 33, 32)}, got {tuple(state.shape)}")
+    out_dtype = out_dtype or q.dtype
+    if out is None:
+        out = torch.empty(B, N, C, dtype=out_dtype, device=q.device)
+    elif out.shape != q.shape or out.dtype != out_dtype:
+        raise SanaHipError("out has the wrong shape or dtype")
+    osb, osn = _token_major_view(out, "out")
+    code = _lib.load().sana_hip_linattn_apply(
+        q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, HEAD_DIM, qsb, qsn, osb, osn,
+        tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype],
+        _stream())
+    _lib.check(code, "sana_hip_linattn_apply")
+    return out
+
+
+def relu_linear_attention(q, k, v, eps: float, chunk_tokens=None, out_dtype=None) -> torch.Tensor:
+    """Both phases on token-major [B, N, C] views; chunk-causal when ``chunk_tokens`` has > 1 entry."""
+    causal = chunk_tokens is not None and len(chunk_tokens) > 1
+    state = linattn_state(k, v, chunk_tokens, causal=causal)
+    return linattn_apply(q, state, eps, chunk_tokens, out_dtype)
+
+
+# --------------------------------------------------------------------------- Mix-FFN pieces
+
+def dwconv3x3_silu_gate(u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                        round_like_reference: bool = True) -> torch.Tensor:
+    """u: [BT, H, W, 2*Ch] contiguous channels-last; weight: [2*Ch, 1, 3, 3] or [2*Ch, 3, 3];
+    bias: [2*Ch] or None.  Returns [BT, H, W, Ch]."""
+    _need_cuda(u, weight, bias)
+    if u.dim() != 4 or not u.is_contiguous():
+        raise SanaHipError("u must be a contiguous [BT, H, W, 2*Ch] tensor")
+    BT, H, W, C2 = u.shape
+    if C2 % 2 or weight.numel() != C2 * 9 or not weight.is_contiguous() or weight.dtype != u.dtype:
+        raise SanaHipError("weight must be contiguous [2*Ch, 1, 3, 3] in u's dtype")
+    if bias is not None and (bias.numel() != C2 or bias.dtype != u.dtype or not bias.is_contiguous()):
+        raise SanaHipError("bias must be contiguous [2*Ch] in u's dtype")
+    y = torch.empty(BT, H, W, C2 // 2, dtype=u.dtype, device=u.device)
+    code = _lib.load().sana_hip_dwconv3x3_silu_gate(
+        u.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(),
+        BT, H, W, C2 // 2, 1 if round_like_reference else 0, _dt(u), _stream())
+    _lib.check(code, "sana_hip_dwconv3x3_silu_gate")
+    return y
+
+
+_EPI = {None: _lib.EPI_NONE, "none": _lib.EPI_NONE, "bias": _lib.EPI_BIAS, "bias_silu": _lib.EPI_BIAS_SILU}
+
+
+def _rows(t: torch.Tensor, what: str) -> Tuple[torch.Tensor, int]:
+    """2-d row-major view (unit inner stride) -> (tensor, leading stride)."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise SanaHipError(f"{what} must be 2-d with unit inner stride, got {tuple(t.shape)} / {t.stride()}")
+    return t, t.stride(0)
+
+
+def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a: [M, K] bf16; weight: [N, K] bf16 (nn.Linear layout).  Returns epilogue(a @ weight.T) [M, N] bf16."""
+    _need_cuda(a, weight, bias)
+    if a.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise SanaHipError("gemm_bf16 needs bf16 operands")
+    a, lda = _rows(a, "a")
+    weight, ldw = _rows(weight, "weight")
+    M, K = a.shape
+    N = weight.shape[0]
+    if weight.shape[1] != K:
+        raise SanaHipError(f"K mismatch: a {tuple(a.shape)} vs weight {tuple(weight.shape)}")
+    epi = _EPI[epilogue]
+    if bias is not None and epi == _lib.EPI_NONE:
+        epi = _lib.EPI_BIAS
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
+        raise SanaHipError("bias must be contiguous bf16 [N]")
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+    out, ldc = _rows(out, "out")
+    code = _lib.load().sana_hip_gemm_bf16(a.data_ptr(), weight.data_ptr(),
+                                          bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                                          M, N, K, lda, ldw, ldc, epi, _stream())
+    _lib.check(code, "sana_hip_gemm_bf16")
+    return out
+
+
+def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a: [M, K] bf16; wq: [N, K] int8; scale: [N] fp32.  Equals gemm_bf16 on (wq.float()*scale).bfloat16()."""
+    _need_cuda(a, wq, scale, bias)
+    if a.dtype != torch.bfloat16 or wq.dtype != torch.int8 or scale.dtype != torch.float32:
+        raise SanaHipError("gemm_w8a16 needs bf16 activations, int8 weights and fp32 scales")
+    a, lda = _rows(a, "a")
+    wq, ldw = _rows(wq, "wq")
+    M, K = a.shape
+    N = wq.shape[0]
+    if wq.shape[1] != K or scale.numel() != N or not scale.is_contiguous():
+        raise SanaHipError("shape mismatch between a, wq and scale")
+    epi = _EPI[epilogue]
+    if bias is not None and epi == _lib.EPI_NONE:
+        epi = _lib.EPI_BIAS
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+    out, ldc = _rows(out, "out")
+    code = _lib.load().sana_hip_gemm_w8a16(a.data_ptr(), wq.data_ptr(), scale.data_ptr(),
+                                           bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                                           M, N, K, lda, ldw, ldc, epi, _stream())
+    _lib.check(code, "sana_hip_gemm_w8a16")
+    return out

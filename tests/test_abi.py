@@ -1,0 +1,68 @@
+"""CPU checks of the boundary: the library loads and exports every symbol the
+header declares, argument validation works without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from sana_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sana_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sana_hip_\w+)\s*\(", text)))
+
+
+def test_library_is_built():
+    assert os.path.exists(_lib.LIB_PATH), "run `python -m sana_amd.build` first"
+
+
+def test_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared_symbols()
+    assert len(declared) >= 9
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/sana_hip.h but not exported"
+    assert sorted(_lib.SIGNATURES) == declared, "python signature table out of sync with the header"
+
+
+def test_version_and_strerror():
+    lib = _lib.load()
+    assert lib.sana_hip_abi_version() == 1
+    assert b"aligned" in lib.sana_hip_strerror(-3)
+    assert b"unknown" in lib.sana_hip_strerror(-99)
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    # null pointers / bad sizes are rejected before any launch
+    assert lib.sana_hip_linattn_state(None, None, None, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 1, None) == -1
+    assert lib.sana_hip_linattn_state(16, 16, 16, None, 0, 1, 16, 1, 64, 0, 64, None, 1, 16, 0, 1, None) == -2  # d != 32
+    assert lib.sana_hip_linattn_state(16, 16, 16, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 7, None) == -6  # dtype
+    assert lib.sana_hip_linattn_state(16, 18, 16, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 1, None) == -3  # align
+    assert lib.sana_hip_linattn_apply(16, 16, 16, 1, 16, 1, 32, 0, 32, 0, 32, None, 1, 16, 1e-8, 1, 2, None) == -6
+    assert lib.sana_hip_dwconv3x3_silu_gate(16, 16, None, 16, 1, 4, 4, 3, 1, 1, None) == -2  # odd Ch
+    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 24, 24, 24, 8, 0, None) == -2      # K % 32
+    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None) == -1      # bias epilogue, no bias
+    assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None) == -1  # no scale
+
+
+def test_workspace_query():
+    lib = _lib.load()
+    # 1.6B @ 16384 tokens: 70 heads -> splits of the token axis need partial states
+    n = lib.sana_hip_linattn_workspace_bytes(1, 70, 32, 1, 16384, 1)
+    assert n > 0 and n % (33 * 32 * 4) == 0
+    # many (batch, head) pairs at 1024 tokens: no split, no workspace
+    assert lib.sana_hip_linattn_workspace_bytes(16, 70, 32, 1, 1024, 1) == 0
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from sana_amd import ops
+    x = torch.zeros(1, 32, 32)
+    with pytest.raises(_lib.SanaHipError):
+        ops.linattn_state(x, x)

@@ -1,0 +1,154 @@
+"""GPU parity of the Mix-FFN kernels (depthwise+gate, GEMMs, W8A16) against the oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import cbrute
+from oracle import sana_oracle as O
+from sana_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+
+def _dw_ref(u, w, b, Ch):
+    """fp64 stock conv on the bf16-rounded values: dw -> split -> a * silu(g)."""
+    x = u.double().permute(0, 3, 1, 2)
+    t = F.conv2d(x, w.double().view(2 * Ch, 1, 3, 3), None if b is None else b.double(), padding=1, groups=2 * Ch)
+    a, g = t[:, :Ch], t[:, Ch:]
+    return (a * F.silu(g)).permute(0, 2, 3, 1)
+
+
+@pytest.mark.parametrize("BT,H,W,Ch,dtype", [
+    (4, 32, 32, 2880, torch.bfloat16),    # cfg2
+    (1, 128, 128, 5600, torch.bfloat16),  # cfg3
+    (2, 30, 52, 160, torch.bfloat16),     # cfg5 frame grid, ragged strips
+    (1, 5, 7, 6, torch.bfloat16),
+    (3, 1, 1, 2, torch.bfloat16),
+    (1, 9, 3, 130, torch.float32),
+    (1, 6, 11, 66, torch.float16),
+])
+def test_dwconv_gate_matches_oracle(cuda, BT, H, W, Ch, dtype):
+    g = torch.Generator().manual_seed(H * W + Ch)
+    u = torch.randn(BT, H, W, 2 * Ch, generator=g).to(dtype)
+    w = (torch.randn(2 * Ch, 1, 3, 3, generator=g) * 0.3).to(dtype)
+    b = (torch.randn(2 * Ch, generator=g) * 0.3).to(dtype)
+    ref = _dw_ref(u, w, b, Ch)
+    for round_ref in (False, True):
+        y = ops.dwconv3x3_silu_gate(u.to(cuda), w.to(cuda), b.to(cuda), round_like_reference=round_ref)
+        assert y.shape == (BT, H, W, Ch) and y.dtype == dtype
+        tol = 1e-5 if dtype == torch.float32 else 1e-2
+        assert rel_l2(y.cpu(), ref) <= tol
+        if dtype == torch.bfloat16:
+            err = (y.cpu().double() - ref).abs()
+            assert (err <= 2e-2 + 2 ** -6 * ref.abs()).all()
+    y = ops.dwconv3x3_silu_gate(u.to(cuda), w.to(cuda), None)
+    assert rel_l2(y.cpu(), _dw_ref(u, w, None, Ch)) <= (1e-5 if dtype == torch.float32 else 1e-2)
+
+
+def test_dwconv_against_c_bruteforce(cuda):
+    g = torch.Generator().manual_seed(1)
+    BT, H, W, Ch = 2, 4, 5, 10
+    u = torch.randn(BT, H, W, 2 * Ch, generator=g)
+    w = torch.randn(2 * Ch, 3, 3, generator=g) * 0.3
+    b = torch.randn(2 * Ch, generator=g) * 0.3
+    ref = torch.from_numpy(cbrute.dwconv_gate(u.numpy(), w.numpy(), b.numpy()))
+    y = ops.dwconv3x3_silu_gate(u.to(cuda), w.view(2 * Ch, 1, 3, 3).to(cuda), b.to(cuda), round_like_reference=False)
+    assert rel_l2(y.cpu(), ref) <= 1e-5
+
+
+def test_dwconv_reference_rounding_is_bitwise_on_exact_inputs(cuda):
+    """With small-integer inputs and weights every fp32 partial sum is exact, so the
+    kernel in round-like-reference mode must equal the stock bf16 op chain bit for bit."""
+    g = torch.Generator().manual_seed(2)
+    BT, H, W, Ch = 1, 8, 9, 64
+    u = torch.randint(-3, 4, (BT, H, W, 2 * Ch), generator=g).bfloat16()
+    w = torch.randint(-2, 3, (2 * Ch, 1, 3, 3), generator=g).bfloat16()
+    b = torch.randint(-2, 3, (2 * Ch,), generator=g).bfloat16()
+    t = F.conv2d(u.float().permute(0, 3, 1, 2), w.float(), b.float(), padding=1, groups=2 * Ch).bfloat16()
+    a, gg = t[:, :Ch], t[:, Ch:]
+    ref = (a * F.silu(gg)).permute(0, 2, 3, 1)
+    y = ops.dwconv3x3_silu_gate(u.to(cuda), w.to(cuda), b.to(cuda), round_like_reference=True).cpu()
+    # silu via exp2/rcp may differ from libm in the last fp32 bit, which can flip a bf16 rounding
+    diff = (y.float() - ref.float()).abs()
+    assert (diff <= 2 ** -7 * ref.float().abs() + 1e-30).all()
+    assert (diff == 0).float().mean().item() > 0.97
+
+
+GEMM_SHAPES = [
+    (1024, 3456, 1152),   # qkv at 600M, one image of cfg2
+    (4096, 5760, 1152),   # inverted conv, cfg2
+    (4096, 1152, 2880),   # point conv, cfg2
+    (16384, 2240, 2240),  # proj, cfg3
+    (16384, 2240, 5600),  # point conv, cfg3 (K not a multiple of 64)
+    (300, 72, 96),        # ragged everything
+    (1, 8, 32),
+    (257, 264, 160),
+]
+
+
+def _gemm_ref(a, w, bias, epilogue):
+    y = a.double() @ w.double().T
+    if bias is not None:
+        y = y + bias.double()
+    if epilogue == "bias_silu":
+        y = F.silu(y.bfloat16().double())   # the reference rounds the conv output, then applies SiLU
+    return y
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("epilogue", [None, "bias", "bias_silu"])
+def test_gemm_bf16_matches_oracle(cuda, M, N, K, epilogue):
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16() if epilogue else None
+    ref = _gemm_ref(a, w, bias, epilogue)
+    y = ops.gemm_bf16(a.to(cuda), w.to(cuda), None if bias is None else bias.to(cuda), epilogue)
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16
+    assert rel_l2(y.cpu(), ref) <= 4e-3          # bf16 output rounding alone is ~2e-3
+    err = (y.cpu().double() - ref).abs()
+    assert (err <= 2e-2 + 2 ** -7 * ref.abs()).all()
+
+
+def test_gemm_strided_views(cuda):
+    """Row strides larger than the row length (slices of bigger buffers)."""
+    g = torch.Generator().manual_seed(0)
+    big_a = torch.randn(200, 320, generator=g).bfloat16().to(cuda)
+    big_w = (torch.randn(136, 512, generator=g) * 0.1).bfloat16().to(cuda)
+    a, w = big_a[:, 64:64 + 160], big_w[:, 128:128 + 160]
+    out = torch.zeros(200, 400, dtype=torch.bfloat16, device=cuda)
+    ops.gemm_bf16(a, w, out=out[:, 8:8 + 136])
+    ref = a.double() @ w.double().T
+    assert rel_l2(out[:, 8:144].cpu(), ref.cpu()) <= 4e-3
+    assert out[:, :8].abs().max() == 0 and out[:, 144:].abs().max() == 0
+
+
+def test_gemm_exact_on_integer_inputs(cuda):
+    """Small integers: every product and partial sum is exact in fp32, the result is exact in bf16."""
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(-2, 3, (512, 320), generator=g).bfloat16()
+    w = torch.randint(-1, 2, (264, 320), generator=g).bfloat16()
+    y = ops.gemm_bf16(a.to(cuda), w.to(cuda)).cpu()
+    assert torch.equal(y.float(), a.float() @ w.float().T)
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 2240, 2240), (4096, 11200, 2240), (300, 72, 96), (16384, 2240, 5600)])
+@pytest.mark.parametrize("epilogue", [None, "bias_silu"])
+def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilogue):
+    g = torch.Generator().manual_seed(M + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(cuda)
+    w = torch.empty(N, K)
+    torch.nn.init.trunc_normal_(w, std=0.02, generator=g)
+    wq, s = O.quantize_w8(w.bfloat16())
+    wd = O.dequantize_w8(wq, s)
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16().to(cuda) if epilogue else None
+    y8 = ops.gemm_w8a16(a, wq.to(cuda), s.to(cuda), bias, epilogue)
+    y16 = ops.gemm_bf16(a, wd.to(cuda), bias, epilogue)
+    # in-register dequantisation reproduces (q.float()*s).bfloat16() exactly -> same kernel arithmetic
+    assert torch.equal(y8, y16)
+    ref = _gemm_ref(a.cpu(), wd, None if bias is None else bias.cpu(), epilogue)
+    assert rel_l2(y8.cpu(), ref) <= 4e-3
