@@ -1,0 +1,264 @@
+#!/usr/bin/env python3
+"""Benchmark of the SanaMSBlock hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A *step* is one denoising step of the Sana-1.6B DiT blocks at 4096x4096:
+20 random-init SanaMSBlocks chained on one batch (B=1, N=128x128=16384 tokens,
+C=2240, 70 heads x 32, Mix-FFN hidden 5600, 300 text tokens), bf16, inputs
+resident in HBM.  ``value`` is the block forward latency in ms (step / 20).
+
+The JSON line also carries, measured in the same run with HIP events on the
+launch stream:
+  roofline       the dominant kernel (the inverted-conv GEMM) against the
+                 MI355X dense bf16 MFMA peak,
+  kernels        every hand-written kernel of the block against its roofline
+                 (HBM 8 TB/s for the attention pair and the depthwise kernel,
+                 2.5 PFLOP/s for the four GEMMs),
+  images_per_s   B / (20 x block latency) at the 1024px shape (B=16, N=1024),
+                 bf16 and W8A16: DiT blocks of ONE denoising step only,
+  cpu_baseline   the oracle block (stock PyTorch, fp32) on the host cores, one
+                 block of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+DEPTH, C, HEADS_X, MLP_RATIO, N_TEXT = 20, 2240, 20, 2.5, 300   # Sana-1.6B (depth 20, width 2240, 20 cross-attn heads)
+HID = int(C * MLP_RATIO)
+
+
+def make_state(seed: int, dtype=torch.bfloat16) -> dict:
+    """Random init of one block: trunc-normal(std 0.02) weights, zero biases,
+    scale_shift_table = randn(6, C) / sqrt(C)."""
+    g = torch.Generator().manual_seed(seed)
+
+    def tn(*shape):
+        w = torch.empty(*shape)
+        torch.nn.init.trunc_normal_(w, std=0.02, generator=g)
+        return w.to(dtype)
+
+    z = lambda *s: torch.zeros(*s, dtype=dtype)
+    return {
+        "scale_shift_table": (torch.randn(6, C, generator=g) / C ** 0.5).to(dtype),
+        "attn.qkv.weight": tn(3 * C, C), "attn.proj.weight": tn(C, C), "attn.proj.bias": z(C),
+        "cross_attn.q_linear.weight": tn(C, C), "cross_attn.q_linear.bias": z(C),
+        "cross_attn.kv_linear.weight": tn(2 * C, C), "cross_attn.kv_linear.bias": z(2 * C),
+        "cross_attn.proj.weight": tn(C, C), "cross_attn.proj.bias": z(C),
+        "mlp.inverted_conv.conv.weight": tn(2 * HID, C, 1, 1), "mlp.inverted_conv.conv.bias": z(2 * HID),
+        "mlp.depth_conv.conv.weight": tn(2 * HID, 1, 3, 3), "mlp.depth_conv.conv.bias": z(2 * HID),
+        "mlp.point_conv.conv.weight": tn(C, HID, 1, 1),
+    }
+
+
+def make_inputs(B: int, N: int, seed: int = 1000):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, N, C, generator=g)
+    y = torch.randn(B, N_TEXT, C, generator=g)
+    t = torch.randn(B, 6 * C, generator=g) * 0.02
+    return x, y, t
+
+
+def event_time_us(fn, iters: int, warmup: int) -> float:
+    """Average duration of one call, HIP events on the stream the kernels are launched on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def kernel_rooflines(dev, iters=50, warmup=10):
+    """Each hand-written kernel alone at the cfg3 shape (B=1, N=16384)."""
+    from sana_amd import ops
+
+    B, N, M = 1, 16384, 16384
+    g = torch.Generator().manual_seed(7)
+    rows = []
+
+    def add(name, bound, work, t_us, note):
+        if bound == "hbm":
+            ach, peak, unit = work / t_us / 1e3, HBM_PEAK_GBS, "GB/s"
+        else:
+            ach, peak, unit = work / t_us / 1e6, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+        rows.append({"kernel": name, "bound": bound, "us": round(t_us, 2), "achieved": round(ach, 1), "peak": peak,
+                     "unit": unit, "frac": round(ach / peak, 4), "work": work, "note": note})
+
+    qkv = torch.randn(B, N, 3, C, generator=g).bfloat16().to(dev)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    state = ops.linattn_state(k, v)
+    out = torch.empty(B, N, C, dtype=torch.bfloat16, device=dev)
+    la_bytes = 2 * M * C * 2 + B * (C // 32) * 33 * 32 * 4
+    add("linattn_state", "hbm", la_bytes, event_time_us(lambda: ops.linattn_state(k, v), iters, warmup),
+        "2*M*C*2 B (K,V read) + state write")
+    add("linattn_apply", "hbm", la_bytes,
+        event_time_us(lambda: ops.linattn_apply(q, state, 1e-8, out=out), iters, warmup),
+        "M*C*2 B (Q read) + M*C*2 B (out write) + state read")
+    u = torch.randn(B, 128, 128, 2 * HID, generator=g).bfloat16().to(dev)
+    dw = (torch.randn(2 * HID, 1, 3, 3, generator=g) * 0.3).bfloat16().to(dev)
+    db = torch.zeros(2 * HID, dtype=torch.bfloat16, device=dev)
+    add("dwconv3x3_silu_gate", "hbm", M * 2 * HID * 2 + M * HID * 2 + 2 * HID * 10 * 2,
+        event_time_us(lambda: ops.dwconv3x3_silu_gate(u, dw, db, True), iters, warmup),
+        "M*2H*2 B read + M*H*2 B write + weights")
+    del u
+    for name, Nn, Kk, epi in (("gemm_qkv", 3 * C, C, None), ("gemm_proj", C, C, "bias"),
+                              ("gemm_inverted", 2 * HID, C, "bias_silu"), ("gemm_point", C, HID, None)):
+        a = torch.randn(M, Kk, generator=g).bfloat16().to(dev)
+        w = (torch.randn(Nn, Kk, generator=g) * 0.02).bfloat16().to(dev)
+        bias = torch.zeros(Nn, dtype=torch.bfloat16, device=dev) if epi else None
+        o = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
+        t_us = event_time_us(lambda: ops.gemm_bf16(a, w, bias, epi, out=o), 20, 5)
+        add(name, "mfma", 2 * M * Nn * Kk, t_us, f"2*M*K*N, M={M} N={Nn} K={Kk}")
+        t_lib = event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 20, 5)
+        rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt on the same shape, for scale only
+        del a, w, o
+    # plain device copy as a bandwidth yardstick of this box
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    t_us = event_time_us(lambda: dst.copy_(src), 20, 5)
+    copy_gbs = 2 * src.numel() / t_us / 1e3
+    return rows, round(copy_gbs, 1)
+
+
+def images_per_s(dev, w8: bool, steps: int, warmup: int) -> float:
+    """1024px shape of Sana-1.6B: B=16, N=1024; DiT blocks of one denoising step only."""
+    import sana_amd as S
+
+    B, HW = 16, (32, 32)
+    blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
+    blk.load_state_dict(make_state(0))
+    blk = blk.to(dev)
+    if w8:
+        blk.quantize_w8_()
+    x, y, t = (a.bfloat16().to(dev) for a in make_inputs(B, HW[0] * HW[1]))
+    with torch.no_grad():
+        t_us = event_time_us(lambda: blk(x, y, t, HW=HW), steps, warmup)
+    return B / (DEPTH * t_us * 1e-6)
+
+
+def cpu_baseline(iters: int = 2):
+    """The oracle (stock PyTorch restatement of the reference block) on the host
+    cores: one block of the cfg3 workload in fp32 (bf16 GEMM/conv on CPU is not a
+    fair or stable baseline), same seeded weights and inputs."""
+    from oracle import sana_oracle as O
+
+    threads = torch.get_num_threads()
+    blk = O.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv")
+    blk.load_state_dict(make_state(0, torch.float32))
+    blk.attn.fp32_attention = True
+    x, y, t = make_inputs(1, 16384)
+    with torch.no_grad():
+        blk(x, y, t, HW=(128, 128))
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            blk(x, y, t, HW=(128, 128))
+        dt = (time.perf_counter() - t0) / iters
+    model = ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": round(dt * 1e3, 2), "unit": "ms per block forward", "cores": threads, "kind": "port",
+            "sample": f"1 of the 20 blocks at the same shape (B=1, N=16384, C=2240), fp32, {iters} timed "
+                      f"iterations after 1 warm-up; os.cpu_count()={os.cpu_count()}, cpu='{model}'"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
+        sys.exit(2)
+    import sana_amd as S
+
+    dev = torch.device("cuda:0")
+    B, HW = 1, (128, 128)
+    N = HW[0] * HW[1]
+    blocks = []
+    for i in range(DEPTH):
+        blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
+        blk.load_state_dict(make_state(i))
+        blocks.append(blk.to(dev))
+    x, y, t = (a.bfloat16().to(dev) for a in make_inputs(B, N))
+
+    def step():
+        h = x
+        for blk in blocks:
+            h = blk(h, y, t, None, HW, None)
+        return h
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = step()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        assert torch.isfinite(out.float()).all()
+        ms_per_step = wall * 1e3 / args.steps
+        block_ms = ms_per_step / DEPTH
+
+        kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev)
+        ips_bf16 = images_per_s(dev, False, 20, 5)
+        ips_w8 = images_per_s(dev, True, 20, 5)
+    del blocks
+    torch.cuda.empty_cache()
+
+    dom = next((r for r in kernels if r["kernel"] == "gemm_inverted"), None)
+    roofline = None
+    if dom:
+        roofline = {"kernel": "gemm_kernel<bf16, bias+silu> (inverted 1x1 conv, M=16384 N=11200 K=2240)",
+                    "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"], "unit": "TFLOP/s",
+                    "frac": dom["frac"], "traffic": None}
+    line = {
+        "metric": "Sana-1.6B SanaMSBlock forward latency @16384 tokens (4096px latent)",
+        "value": round(block_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3: Sana-1.6B, 20 SanaMSBlocks chained = one denoising step, B=1, N=128x128=16384, "
+                               "C=2240, 70x32 heads, Mix-FFN hidden 5600, 300 text tokens, random init"},
+        "images_per_s_1024px": {"bf16": round(ips_bf16, 2), "w8a16": round(ips_w8, 2),
+                                "note": "B=16, N=1024: B / (20 x block latency); DiT blocks of one denoising step only "
+                                        "(no text encoder, VAE, embedders, step count or CFG doubling)"},
+        "roofline": roofline,
+        "kernels": kernels,
+        "copy_GBps_this_box": copy_gbs,
+        "peaks": {"hbm_GBps": HBM_PEAK_GBS, "mfma_bf16_TFLOPs": MFMA_BF16_PEAK_TFLOPS},
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -452,7 +452,7 @@ class SanaMSBlock(nn.Module):
     ffn_type="glumbconv" (the configuration of every shipped Sana config)."""
 
     def __init__(self, hidden_size, num_heads, mlp_ratio=4.0, drop_path=0.0, qk_norm=False,
-                 attn_type="linear", ffn_type="glumbconv", mlp_acts=("silu", "silu", None),
+                 attn_type="flash", ffn_type="mlp", mlp_acts=("silu", "silu", None),
                  linear_head_dim=32, cross_norm=False, cross_attn_type="flash", **block_kwargs):
         super().__init__()
         if attn_type != "linear" or ffn_type != "glumbconv":

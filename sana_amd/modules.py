@@ -1,0 +1,409 @@
+"""Drop-in modules for the SanaMSBlock hot path over the gfx950 kernels.
+
+Same constructor arguments, forward signatures, attribute names and
+``state_dict`` keys as the reference classes they stand in for:
+
+  ``LiteLA``               diffusion/model/nets/sana_blocks.py:211-301
+  ``ChunkCausalAttention`` diffusion/model/nets/sana_blocks.py:391-495 (no-RoPE form)
+  ``GLUMBConv``            diffusion/model/nets/basic_modules.py:111-199
+  ``SanaMSBlock``          diffusion/model/nets/sana_multi_scale.py:54-157
+
+Forward only (inference).  The modules run on a GPU through ``libsana_hip.so``;
+there is no CPU path and no silent fallback: a configuration the kernels do
+not cover raises ``NotImplementedError`` at construction or call time.
+Cross-attention, LayerNorm and the adaLN modulation use stock PyTorch-ROCm ops.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops
+from ._lib import SanaHipError
+
+HEAD_DIM = ops.HEAD_DIM
+
+
+def _no_grad_only(*tensors):
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise SanaHipError("the HIP path is forward-only: call it under torch.no_grad() / inference_mode()")
+
+
+# ------------------------------------------------------------------ linear layers
+
+
+class HipLinear(nn.Linear):
+    """``nn.Linear`` whose bf16 GPU forward is the hand-written MFMA GEMM.
+
+    Keys ``weight`` / ``bias`` as in ``nn.Linear``.  After :meth:`quantize_w8_`
+    the bf16 weight is dropped and replaced by ``weight_q`` (int8 [out, in]) and
+    ``weight_scale`` (fp32 [out]); the forward then runs the W8A16 GEMM.
+    Other dtypes (fp16 / fp32 models) use the stock library GEMM.
+    """
+
+    def quantize_w8_(self) -> "HipLinear":
+        wq, scale = quantize_w8(self.weight.data)
+        self.register_buffer("weight_q", wq.contiguous())
+        self.register_buffer("weight_scale", scale.contiguous())
+        self.weight = None
+        return self
+
+    @property
+    def is_quantized(self) -> bool:
+        return getattr(self, "weight_q", None) is not None
+
+    def forward(self, x: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
+        return hip_linear(x, self.weight, self.bias, epilogue,
+                          getattr(self, "weight_q", None), getattr(self, "weight_scale", None))
+
+
+def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None):
+    """y = epilogue(x @ W^T + b) over the last dim of x.  epilogue: None | "silu"."""
+    _no_grad_only(x, weight, bias)
+    lead = x.shape[:-1]
+    K = x.shape[-1]
+    if x.dtype == torch.bfloat16 and x.is_cuda:
+        x2 = x.reshape(-1, K)
+        if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+            x2 = x2.contiguous()
+        epi = {None: "bias" if bias is not None else None, "silu": "bias_silu"}[epilogue]
+        if epilogue == "silu" and bias is None:
+            bias = torch.zeros(weight_q.shape[0] if weight_q is not None else weight.shape[0],
+                               dtype=torch.bfloat16, device=x.device)
+        if weight_q is not None:
+            y = ops.gemm_w8a16(x2, weight_q, weight_scale, bias, epi)
+        else:
+            y = ops.gemm_bf16(x2, weight.reshape(weight.shape[0], -1), bias, epi)
+        return y.view(*lead, y.shape[-1])
+    if not x.is_cuda:
+        raise SanaHipError("the HIP path needs device tensors (no CPU path exists)")
+    if weight_q is not None:
+        raise SanaHipError("W8A16 needs bf16 activations")
+    # fp16 / fp32 models: plain library GEMM (hipBLASLt), activation as a stock op
+    y = F.linear(x, weight.reshape(weight.shape[0], -1), bias)
+    return F.silu(y) if epilogue == "silu" else y
+
+
+def quantize_w8(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Symmetric per-output-channel int8 quantiser of the W8A16 configuration:
+    s_o = absmax_i |W[o, i]| / 127 (fp32), Wq = clamp(round(W / s), -127, 127).
+    Returns (int8 [out, in], fp32 [out]).  Not part of the reference (it has no
+    W8A16 code); the dequantised weight is (Wq.float() * s).bfloat16()."""
+    w = weight.detach().float().flatten(1)
+    scale = w.abs().amax(dim=1) / 127.0
+    scale = torch.where(scale > 0, scale, torch.ones_like(scale))
+    wq = torch.clamp(torch.round(w / scale[:, None]), -127, 127).to(torch.int8)
+    return wq, scale
+
+
+# ------------------------------------------------------------------ linear attention
+
+
+class RMSNorm(nn.Module):
+    """diffusion/model/norms.py:182-231 (stock ops; only used with qk_norm=True)."""
+
+    def __init__(self, dim: int, scale_factor: float = 1.0, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim) * scale_factor)
+
+    def forward(self, x):
+        xf = x.float()
+        return (self.weight * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps))).type_as(x)
+
+
+def _rotary_real_tokens_(t: torch.Tensor, cos_sin) -> None:
+    """In-place real-valued RoPE on a token-major [B, N, C] view: the
+    ``use_real_unbind_dim=-2`` form LiteLA.forward uses (sana_blocks.py:282-284,
+    1572-1582).  cos, sin: [N, d] with d = head_dim; pairs are channels (2m, 2m+1)."""
+    cos, sin = cos_sin
+    B, N, C = t.shape
+    d = cos.shape[-1]
+    x = t.reshape(B, N, C // d, d)
+    cos = cos.to(t.device)[None, :, None, :]
+    sin = sin.to(t.device)[None, :, None, :]
+    xr, xi = x.reshape(B, N, C // d, d // 2, 2).unbind(-1)
+    x_rot = torch.stack([-xi, xr], dim=-1).reshape(B, N, C // d, d)
+    t.copy_((x.float() * cos + x_rot.float() * sin).to(t.dtype).reshape(B, N, C))
+
+
+def _as_token_major(t: torch.Tensor, token_dim: int) -> torch.Tensor:
+    """(B, h, d, N) [token_dim=3] or (B, h, N, d) [token_dim=2] -> [B, N, h*d] with
+    unit channel stride, without a copy when the memory already is token-major."""
+    B, h = t.shape[0], t.shape[1]
+    tm = t.permute(0, 3, 1, 2) if token_dim == 3 else t.permute(0, 2, 1, 3)  # (B, N, h, d)
+    N, d = tm.shape[1], tm.shape[3]
+    if tm.stride(3) == 1 and tm.stride(2) == d and tm.stride(1) % 8 == 0 and tm.data_ptr() % 16 == 0:
+        return tm.as_strided((B, N, h * d), (tm.stride(0), tm.stride(1), 1))
+    return tm.reshape(B, N, h * d).contiguous()
+
+
+class LiteLA(nn.Module):
+    """ReLU linear attention (reference: sana_blocks.py:211-301).
+
+    ``qkv`` / ``proj`` carry the parameters the reference inherits from timm's
+    ``Attention`` base; ``q_norm`` / ``k_norm`` are Identity or RMSNorm over the
+    full channel dim.  The attention core always accumulates in fp32 (the
+    reference's ``fp32_attention`` mode); the attribute is accepted and ignored.
+    """
+
+    PAD_VAL = 1
+
+    def __init__(self, in_dim: int, out_dim: int, heads: Optional[int] = None, heads_ratio: float = 1.0,
+                 dim: int = 32, eps: float = 1e-15, use_bias: bool = False, qk_norm: bool = False,
+                 norm_eps: float = 1e-5):
+        super().__init__()
+        heads = heads or int(out_dim // dim * heads_ratio)
+        if in_dim != out_dim:
+            raise NotImplementedError("LiteLA: in_dim != out_dim is not used by any Sana block")
+        self.in_dim, self.out_dim, self.heads = in_dim, out_dim, heads
+        self.dim = out_dim // heads
+        if self.dim != HEAD_DIM:
+            raise NotImplementedError(f"the gfx950 attention kernels are built for head_dim {HEAD_DIM}, got {self.dim}")
+        self.eps = eps
+        self.num_heads = heads
+        self.scale = self.dim ** -0.5
+        self.qkv = HipLinear(in_dim, in_dim * 3, bias=use_bias)
+        self.attn_drop = nn.Dropout(0.0)
+        self.proj = HipLinear(in_dim, in_dim)
+        self.proj_drop = nn.Dropout(0.0)
+        self.kernel_func = nn.ReLU(inplace=False)
+        if qk_norm:
+            self.q_norm = RMSNorm(in_dim, 1.0, norm_eps)
+            self.k_norm = RMSNorm(in_dim, 1.0, norm_eps)
+        else:
+            self.q_norm = nn.Identity()
+            self.k_norm = nn.Identity()
+
+    # -- second public entry point of the reference (used by the PAG processors,
+    #    sana_blocks.py:588-620): q, v (B, h, d, N); k (B, h, N, d); returns fp32 (B, h, d, N)
+    def attn_matmul(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        _no_grad_only(q, k, v)
+        B, h, d, N = q.shape
+        qt = _as_token_major(q, 3)
+        kt = _as_token_major(k, 2)
+        vt = _as_token_major(v, 3)
+        if kt.stride() != vt.stride():
+            kt, vt = kt.contiguous(), vt.contiguous()
+        out = ops.relu_linear_attention(qt, kt, vt, self.eps, out_dtype=torch.float32)  # ReLU is applied in-kernel
+        return out.view(B, N, h, d).permute(0, 2, 3, 1)
+
+    def _qkv_tokens(self, x: torch.Tensor, rotary_emb=None) -> torch.Tensor:
+        """qkv GEMM, optional qk-norm and RoPE -> fused [B, N, 3, C] buffer."""
+        B, N, C = x.shape
+        qkv = self.qkv(x).view(B, N, 3, C)
+        if not isinstance(self.q_norm, nn.Identity):
+            qkv[:, :, 0].copy_(self.q_norm(qkv[:, :, 0]))
+            qkv[:, :, 1].copy_(self.k_norm(qkv[:, :, 1]))
+        if rotary_emb is not None:
+            _rotary_real_tokens_(qkv[:, :, 0], rotary_emb)
+            _rotary_real_tokens_(qkv[:, :, 1], rotary_emb)
+        return qkv
+
+    def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_id=None,
+                block_mask=None) -> torch.Tensor:
+        _no_grad_only(x)
+        qkv = self._qkv_tokens(x, rotary_emb)
+        out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps)
+        return self.proj(out)
+
+    def quantize_w8_(self) -> "LiteLA":
+        self.qkv.quantize_w8_()
+        self.proj.quantize_w8_()
+        return self
+
+    def __repr__(self):
+        return f"EPS{self.eps}-" + super().__repr__()
+
+
+class ChunkCausalAttention(LiteLA):
+    """Chunk-causal ReLU linear attention (reference: sana_blocks.py:391-495):
+    every chunk of whole frames attends to the running sum of the states of all
+    earlier chunks plus its own.  ``HW = (frames, h, w)``; ``chunk_index`` lists
+    the first frame of each chunk.  This build covers the form without rotary
+    embedding (``rotary_emb=None``, the reference's unit rotation)."""
+
+    def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None,
+                chunk_index: Optional[List[int]] = None) -> torch.Tensor:
+        _no_grad_only(x)
+        if rotary_emb is not None:
+            raise NotImplementedError("ChunkCausalAttention: the rotary (ReLU -> RoPE) variant is not built yet")
+        if HW is None or len(HW) != 3:
+            raise ValueError("ChunkCausalAttention needs HW = (frames, h, w)")
+        f, hh, ww = HW
+        B, N, C = x.shape
+        if f * hh * ww != N:
+            raise ValueError(f"HW={HW} does not match N={N}")
+        starts = list(chunk_index) if chunk_index is not None else [0]
+        qkv = self._qkv_tokens(x)
+        out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps,
+                                        chunk_tokens=[s * hh * ww for s in starts])
+        return self.proj(out)
+
+
+# ------------------------------------------------------------------ Mix-FFN
+
+
+class ConvLayer(nn.Module):
+    """Parameter holder with the reference's attribute names (basic_modules.py:32-99):
+    ``conv`` (nn.Conv2d), ``norm`` (None), ``act``.  GLUMBConv.forward reads the
+    parameters and calls the kernels; this module's own forward is the stock op."""
+
+    def __init__(self, in_dim, out_dim, kernel_size=3, groups=1, use_bias=False, act=None):
+        super().__init__()
+        self.conv = nn.Conv2d(in_dim, out_dim, kernel_size, 1, kernel_size // 2, 1, groups, use_bias)
+        self.norm = None
+        self.act = nn.SiLU(inplace=True) if act == "silu" else None
+
+    def forward(self, x):
+        x = self.conv(x)
+        return self.act(x) if self.act else x
+
+
+def _tuple3(x):
+    xs = list(x) if isinstance(x, (list, tuple)) else [x]
+    while len(xs) < 3:
+        xs.insert(len(xs) - 1, xs[-1])
+    return tuple(xs)
+
+
+class GLUMBConv(nn.Module):
+    """Mix-FFN (reference: basic_modules.py:111-199): 1x1 conv C->2H + SiLU,
+    depthwise 3x3, gate a * SiLU(g), 1x1 conv H->C.  ``HW`` is (H, W) or
+    (T, H, W) (3x3 per frame).  Channels-last throughout: the two 1x1 convs are
+    MFMA GEMMs over tokens, the middle is one fused kernel."""
+
+    def __init__(self, in_features: int, hidden_features: int, out_feature=None, kernel_size=3, stride=1,
+                 padding=None, use_bias=False, norm=(None, None, None), act=("silu", "silu", None), dilation=1):
+        super().__init__()
+        out_feature = out_feature or in_features
+        use_bias, norm, act = _tuple3(use_bias), _tuple3(norm), _tuple3(act)
+        if kernel_size != 3 or stride != 1 or dilation != 1 or padding not in (None, 1):
+            raise NotImplementedError("GLUMBConv HIP path: kernel_size=3, stride=1, dilation=1 only")
+        if any(n is not None for n in norm):
+            raise NotImplementedError("GLUMBConv HIP path: norm must be (None, None, None)")
+        if tuple(act) != ("silu", "silu", None):
+            raise NotImplementedError("GLUMBConv HIP path: act must be ('silu', 'silu', None)")
+        self.glu_act = nn.SiLU(inplace=False)
+        self.inverted_conv = ConvLayer(in_features, hidden_features * 2, 1, use_bias=use_bias[0], act="silu")
+        self.depth_conv = ConvLayer(hidden_features * 2, hidden_features * 2, 3, groups=hidden_features * 2,
+                                    use_bias=use_bias[1], act=None)
+        self.point_conv = ConvLayer(hidden_features, out_feature, 1, use_bias=use_bias[2], act=None)
+        self.round_like_reference = True
+
+    def forward(self, x: torch.Tensor, HW=None) -> torch.Tensor:
+        _no_grad_only(x)
+        B, N, C = x.shape
+        if HW is None:
+            raise ValueError("GLUMBConv needs HW (the reference fails on HW=None too: basic_modules.py:193)")
+        if len(HW) == 2:
+            frames, (H, W) = B, HW
+        else:
+            T, H, W = HW
+            frames = B * T
+        if frames * H * W != B * N:
+            raise ValueError(f"HW={HW} does not match N={N}")
+        ic, dc, pc = self.inverted_conv.conv, self.depth_conv.conv, self.point_conv.conv
+        u = hip_linear(x, ic.weight, ic.bias, "silu", getattr(ic, "weight_q", None), getattr(ic, "weight_scale", None))
+        y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
+                                    round_like_reference=self.round_like_reference)
+        out = hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
+                         getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None))
+        return out
+
+    def quantize_w8_(self) -> "GLUMBConv":
+        for conv in (self.inverted_conv.conv, self.point_conv.conv):
+            wq, scale = quantize_w8(conv.weight.data)
+            conv.register_buffer("weight_q", wq.contiguous())
+            conv.register_buffer("weight_scale", scale.contiguous())
+            conv.weight = None
+        return self
+
+
+# ------------------------------------------------------------------ the block
+
+
+def t2i_modulate(x, shift, scale):
+    return x * (1 + scale) + shift
+
+
+class MultiHeadCrossAttention(nn.Module):
+    """Cross-attention to the text tokens on stock ops (reference:
+    sana_blocks.py:48-98, the scaled_dot_product_attention branch)."""
+
+    def __init__(self, d_model, num_heads, attn_drop=0.0, proj_drop=0.0, qk_norm=False, **block_kwargs):
+        super().__init__()
+        assert d_model % num_heads == 0, "d_model must be divisible by num_heads"
+        self.d_model, self.num_heads, self.head_dim = d_model, num_heads, d_model // num_heads
+        self.q_linear = nn.Linear(d_model, d_model)
+        self.kv_linear = nn.Linear(d_model, d_model * 2)
+        self.attn_drop = nn.Dropout(attn_drop)
+        self.proj = nn.Linear(d_model, d_model)
+        self.proj_drop = nn.Dropout(proj_drop)
+        if qk_norm:
+            self.q_norm = RMSNorm(d_model, 1.0, 1e-6)
+            self.k_norm = RMSNorm(d_model, 1.0, 1e-6)
+        else:
+            self.q_norm = nn.Identity()
+            self.k_norm = nn.Identity()
+
+    def forward(self, x, cond, mask=None):
+        B, N, C = x.shape
+        q = self.q_linear(x)
+        kv = self.kv_linear(cond).view(B, -1, 2, C)
+        k, v = kv.unbind(2)
+        q = self.q_norm(q).view(B, -1, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_norm(k).view(B, -1, self.num_heads, self.head_dim).transpose(1, 2)
+        v = v.view(B, -1, self.num_heads, self.head_dim).transpose(1, 2)
+        if mask is not None and mask.ndim == 2:
+            mask = (1 - mask.to(q.dtype)) * -10000.0
+            mask = mask[:, None, None].repeat(1, self.num_heads, 1, 1)
+        x = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, dropout_p=0.0, is_causal=False)
+        x = x.transpose(1, 2).reshape(B, -1, C)
+        return self.proj_drop(self.proj(x))
+
+
+class SanaMSBlock(nn.Module):
+    """Sana DiT block with adaLN-single conditioning (reference:
+    sana_multi_scale.py:54-157) for ``attn_type="linear"``, ``ffn_type="glumbconv"``."""
+
+    def __init__(self, hidden_size, num_heads, mlp_ratio=4.0, drop_path=0.0, qk_norm=False, attn_type="flash",
+                 ffn_type="mlp", mlp_acts=("silu", "silu", None), linear_head_dim=32, cross_norm=False,
+                 cross_attn_type="flash", **block_kwargs):
+        super().__init__()
+        if attn_type != "linear" or ffn_type != "glumbconv":
+            raise NotImplementedError("this block is the attn_type='linear' / ffn_type='glumbconv' hot path only")
+        if cross_attn_type not in ("flash", "linear"):
+            raise NotImplementedError(f"cross_attn_type={cross_attn_type!r}")
+        if drop_path > 0.0:
+            raise NotImplementedError("drop_path > 0 is a training-time option; this block is forward-only")
+        self.hidden_size = hidden_size
+        self.norm1 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        self.attn = LiteLA(hidden_size, hidden_size, heads=hidden_size // linear_head_dim, eps=1e-8, qk_norm=qk_norm)
+        self.cross_attn = MultiHeadCrossAttention(hidden_size, num_heads, qk_norm=cross_norm, **block_kwargs)
+        self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        self.mlp = GLUMBConv(in_features=hidden_size, hidden_features=int(hidden_size * mlp_ratio),
+                             use_bias=(True, True, False), norm=(None, None, None), act=mlp_acts)
+        self.drop_path = nn.Identity()
+        self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
+
+    def forward(self, x, y, t, mask=None, HW=None, image_rotary_emb=None, **kwargs):
+        B, N, C = x.shape
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+            self.scale_shift_table[None] + t.reshape(B, 6, -1)
+        ).chunk(6, dim=1)
+        x = x + self.drop_path(
+            gate_msa * self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), HW=HW, rotary_emb=image_rotary_emb))
+        x = x + self.cross_attn(x, y, mask)
+        x = x + self.drop_path(gate_mlp * self.mlp(t2i_modulate(self.norm2(x), shift_mlp, scale_mlp), HW=HW))
+        return x
+
+    def quantize_w8_(self) -> "SanaMSBlock":
+        """W8A16: int8 per-output-channel weights for qkv, proj and the two 1x1
+        convs.  The stock cross-attention linears stay bf16."""
+        self.attn.quantize_w8_()
+        self.mlp.quantize_w8_()
+        return self

@@ -1,0 +1,77 @@
+"""Host-side contract of the drop-in modules (no GPU): constructor signatures,
+attribute names and state_dict keys equal the oracle's restatement of the
+reference, checkpoints load both ways, unsupported options fail loudly."""
+import inspect
+
+import pytest
+import torch
+
+import sana_amd as S
+from oracle import sana_oracle as O
+
+
+@pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention"])
+def test_constructor_and_forward_signatures_match(name):
+    a, b = getattr(S, name), getattr(O, name)
+    pa = list(inspect.signature(a.__init__).parameters)
+    pb = list(inspect.signature(b.__init__).parameters)
+    assert pa == pb
+    fa = [p for p in inspect.signature(a.forward).parameters]
+    fb = [p for p in inspect.signature(b.forward).parameters]
+    assert fa == fb
+
+
+def test_block_state_dict_round_trip():
+    ob = O.init_block_(O.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv", linear_head_dim=32), 0)
+    hb = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv", linear_head_dim=32)
+    assert list(ob.state_dict()) == list(hb.state_dict())
+    for k, v in ob.state_dict().items():
+        assert hb.state_dict()[k].shape == v.shape, k
+    hb.load_state_dict(ob.state_dict(), strict=True)
+    ob.load_state_dict(hb.state_dict(), strict=True)
+    assert hb.attn.eps == 1e-8 and hb.attn.dim == 32 and hb.attn.heads == 2
+    assert isinstance(hb.attn.kernel_func, torch.nn.ReLU)
+
+
+def test_qk_norm_keys():
+    a = S.LiteLA(64, 64, dim=32, qk_norm=True)
+    b = O.LiteLA(64, 64, dim=32, qk_norm=True)
+    assert sorted(a.state_dict()) == sorted(b.state_dict())
+
+
+def test_unsupported_options_fail_loudly():
+    with pytest.raises(NotImplementedError):
+        S.LiteLA(224, 224, dim=112)
+    with pytest.raises(NotImplementedError):
+        S.GLUMBConv(64, 160, dilation=2)
+    with pytest.raises(NotImplementedError):
+        S.GLUMBConv(64, 160, norm=("bn2d", None, None))
+    with pytest.raises(NotImplementedError):
+        S.SanaMSBlock(64, 4, attn_type="flash")
+
+
+def test_no_cpu_path_and_no_autograd():
+    m = S.GLUMBConv(64, 160, use_bias=(True, True, False)).bfloat16()
+    with torch.no_grad(), pytest.raises(S.SanaHipError):
+        m(torch.zeros(1, 16, 64, dtype=torch.bfloat16), HW=(4, 4))
+    a = S.LiteLA(64, 64, dim=32).bfloat16()
+    with pytest.raises(S.SanaHipError):
+        a(torch.zeros(1, 16, 64, dtype=torch.bfloat16, requires_grad=True))
+
+
+def test_quantiser_matches_oracle_definition():
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(24, 40, generator=g).bfloat16()
+    wq, s = S.quantize_w8(w)
+    wq2, s2 = O.quantize_w8(w)
+    assert torch.equal(wq, wq2) and torch.equal(s, s2)
+
+
+def test_w8_state_keys():
+    blk = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").bfloat16().quantize_w8_()
+    keys = set(blk.state_dict())
+    for base in ("attn.qkv", "attn.proj", "mlp.inverted_conv.conv", "mlp.point_conv.conv"):
+        assert base + ".weight" not in keys
+        assert base + ".weight_q" in keys and base + ".weight_scale" in keys
+    assert blk.state_dict()["attn.qkv.weight_q"].dtype == torch.int8
+    assert "cross_attn.q_linear.weight" in keys and "mlp.depth_conv.conv.weight" in keys

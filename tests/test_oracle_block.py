@@ -19,7 +19,7 @@ def _block(C=64, heads=4, seed=0, dtype=torch.float64):
 
 
 def test_block_keys_and_defaults():
-    blk = O.SanaMSBlock(64, 4, mlp_ratio=2.5)
+    blk = O.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv")
     keys = set(blk.state_dict())
     assert keys == {
         "scale_shift_table", "attn.qkv.weight", "attn.proj.weight", "attn.proj.bias",
