@@ -144,7 +144,7 @@ int sana_hip_dwconv3x3_silu_gate(const void* u, const void* w, const void* bias,
  *   W     [N][K] row-major with row stride ldw  (nn.Linear / 1x1-conv weight layout)
  *   bias  [N] bf16 or NULL (must be non-NULL for SANA_EPI_BIAS*)
  *   C     [M][N] row-major with row stride ldc
- * K must be a multiple of 32; lda, ldw, ldc multiples of 8.
+ * K and N must be multiples of 8 (16-byte rows); lda, ldw, ldc multiples of 8.
  */
 int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
@@ -155,7 +155,7 @@ int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
  * value as torch's (q.float() * scale).bfloat16() — before the MFMA, so the
  * result equals sana_hip_gemm_bf16 on the dequantised weight.  No reference
  * counterpart (the reference has no W8A16 code); the quantiser is defined by the
- * benchmark configuration. */
+ * benchmark configuration.  K and ldw must be multiples of 16. */
 int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias,
                         void* C, int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                         int epilogue, void* stream);

@@ -493,10 +493,11 @@ def quantize_w8(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Symmetric per-output-channel int8: s_o = absmax_i |W[o, i]| / 127,
     Wq = clamp(round(W / s), -127, 127).  ``weight`` is [out, in, ...];
     returns (int8 [out, in...], fp32 scale [out])."""
-    w = weight.detach().float().flatten(1)
-    scale = w.abs().amax(dim=1) / 127.0
+    # fp64 intermediates make the result independent of the device's fp32 division
+    w = weight.detach().double().flatten(1)
+    scale = (w.abs().amax(dim=1) / 127.0).float()
     scale = torch.where(scale > 0, scale, torch.ones_like(scale))
-    wq = torch.clamp(torch.round(w / scale[:, None]), -127, 127).to(torch.int8)
+    wq = torch.clamp(torch.round(w / scale.double()[:, None]), -127, 127).to(torch.int8)
     return wq.view_as(weight), scale
 
 

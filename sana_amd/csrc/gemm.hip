@@ -270,7 +270,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_gemm_bf16(const v
                                                                          const void* bias, void* C, int M, int N,
                                                                          int K, int64_t lda, int64_t ldw,
                                                                          int64_t ldc, int epilogue, void* stream) {
-  const int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, epilogue, 32, 8);
+  const int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, epilogue, 8, 8);
   if (rc != SANA_OK) return rc;
   return launch<false>(A, W, nullptr, bias, C, M, N, K, lda, ldw, ldc, epilogue, static_cast<hipStream_t>(stream));
 }
@@ -281,7 +281,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_gemm_w8a16(const 
                                                                           int64_t ldw, int64_t ldc, int epilogue,
                                                                           void* stream) {
   if (!scale) return SANA_ERR_ARG;
-  const int rc = check_common(A, Wq, bias, C, M, N, K, lda, ldw, ldc, epilogue, 32, 16);
+  const int rc = check_common(A, Wq, bias, C, M, N, K, lda, ldw, ldc, epilogue, 16, 16);
   if (rc != SANA_OK) return rc;
   return launch<true>(A, Wq, scale, bias, C, M, N, K, lda, ldw, ldc, epilogue, static_cast<hipStream_t>(stream));
 }

@@ -92,10 +92,11 @@ def quantize_w8(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     s_o = absmax_i |W[o, i]| / 127 (fp32), Wq = clamp(round(W / s), -127, 127).
     Returns (int8 [out, in], fp32 [out]).  Not part of the reference (it has no
     W8A16 code); the dequantised weight is (Wq.float() * s).bfloat16()."""
-    w = weight.detach().float().flatten(1)
-    scale = w.abs().amax(dim=1) / 127.0
+    # fp64 intermediates make the result independent of the device's fp32 division
+    w = weight.detach().double().flatten(1)
+    scale = (w.abs().amax(dim=1) / 127.0).float()
     scale = torch.where(scale > 0, scale, torch.ones_like(scale))
-    wq = torch.clamp(torch.round(w / scale[:, None]), -127, 127).to(torch.int8)
+    wq = torch.clamp(torch.round(w / scale.double()[:, None]), -127, 127).to(torch.int8)
     return wq, scale
 
 
@@ -186,7 +187,7 @@ class LiteLA(nn.Module):
         qt = _as_token_major(q, 3)
         kt = _as_token_major(k, 2)
         vt = _as_token_major(v, 3)
-        if kt.stride() != vt.stride():
+        if any(a != b and n > 1 for a, b, n in zip(kt.stride(), vt.stride(), kt.shape)):
             kt, vt = kt.contiguous(), vt.contiguous()
         out = ops.relu_linear_attention(qt, kt, vt, self.eps, out_dtype=torch.float32)  # ReLU is applied in-kernel
         return out.view(B, N, h, d).permute(0, 2, 3, 1)

