@@ -11,7 +11,7 @@
 //
 // Workgroup tile 256 (tokens) x 256 (channels) x 64 (k), four waves in 2x2,
 // each 128x128 = 4x4 MFMA 32x32x16 tiles (256 fp32 accumulators).  LDS is
-// double buffered (2 x 64 KB); 16-byte chunks are XOR-swizzled by (row & 7) so
+// double buffered (2 x 64 KB); 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
 // that ds_read_b128 / ds_write_b128 are bank-conflict free.  Workgroup ids are
 // remapped so that each XCD (own L2) works on a compact group of tiles.
 #include "common.h"
@@ -25,7 +25,11 @@ constexpr int BK = 64;
 constexpr int ROW_BYTES = BK * 2;            // 128
 constexpr int TILE_BYTES = 256 * ROW_BYTES;  // 32 KB per operand per stage
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * ROW_BYTES + ((chunk ^ (row & 7)) << 4); }
+// LDS reads of 16 bytes are served 16 lanes (256 bytes = all 64 banks) per clock, so 16 consecutive
+// rows of one k chunk must land in 16 different 16-byte bank groups: rows alternate between the two
+// halves of the bank space (128-byte rows), and the chunk index is XORed with (row / 2) % 8.
+__device__ __forceinline__ int swz_key(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * ROW_BYTES + ((chunk ^ swz_key(row)) << 4); }
 
 // LDS row of weight row n (within the 256-row tile): permute inside each 32-row block
 __device__ __forceinline__ int wrow_to_lds(int n) {
@@ -221,32 +225,247 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
   }
 }
 
+
+// ============================================================================
+// Fast path: 512 threads (8 waves, two per SIMD so one wave's LDS/barrier waits
+// hide behind the other's MFMAs), same 256x256x64 tile, each wave 128 channels x
+// 64 tokens = 4x2 MFMA tiles (128 accumulators).  Global -> LDS goes straight
+// through `global_load_lds_dwordx4` (no VGPR staging, no ds_write): the data of
+// lane l lands at byte 16*l of a 1-KB block = 8 tile rows, so the XOR swizzle is
+// applied to the GLOBAL address each lane fetches.  Rows past M / N are clamped
+// (their results are never stored); a K tail (K % 64 in {16, 32, 48}) runs fewer
+// k-steps on the last tile, so clamped k chunks are never read.  Needs K % 16 == 0.
+// ============================================================================
+#define SANA_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define SANA_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// One k-tile of MFMAs.  FULL: all four k-steps of 16; otherwise `nsteps` (1..4, wave-uniform).
+template <bool FULL>
+__device__ __forceinline__ void mma_tile(const unsigned char* __restrict__ sa, const unsigned char* __restrict__ sw,
+                                         int a_off, int w_off, int x7, int fg, int nsteps, f32x16_t (&acc)[4][2]) {
+  u32x4_t fw[2][4], fa[2][2];
+  auto read = [&](int buf, int ks) {
+    const int col = ((2 * ks + fg) ^ x7) << 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fw[buf][i] = *reinterpret_cast<const u32x4_t*>(sw + w_off + i * 32 * ROW_BYTES + col);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) fa[buf][j] = *reinterpret_cast<const u32x4_t*>(sa + a_off + j * 32 * ROW_BYTES + col);
+  };
+  read(0, 0);
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    if (!FULL && ks >= nsteps) break;
+    if (ks + 1 < 4 && (FULL || ks + 1 < nsteps)) read((ks + 1) & 1, ks + 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[ks & 1][i]),
+                                                           __builtin_bit_cast(bf16x8_t, fa[ks & 1][j]), acc[i][j], 0,
+                                                           0, 0);
+  }
+}
+
+template <bool W8, int EPI>
+__global__ __launch_bounds__(512) void gemm_fast_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
+                                                        const float* __restrict__ scale,
+                                                        const uint16_t* __restrict__ bias, uint16_t* __restrict__ C,
+                                                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
+                                                        int tiles_t, int tiles_c) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+  const int total = tiles_t * tiles_c;
+  int pid = blockIdx.x;
+  {
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    pid = xcd * base + min(xcd, rem) + local;
+  }
+  constexpr int GROUP = 8;
+  const int group_sz = GROUP * tiles_c;
+  const int gid = pid / group_sz;
+  const int first_t = gid * GROUP;
+  const int gt = min(tiles_t - first_t, GROUP);
+  const int tile_t = first_t + (pid % group_sz) % gt;
+  const int tile_c = (pid % group_sz) / gt;
+  const int m0 = tile_t * BT, n0 = tile_c * BC;
+
+  // ---- direct global -> LDS loads.  Wave w fills 1-KB blocks w, w+8, w+16, w+24 of each tile.
+  const int l_row = lane >> 3;  // row inside the block; logical k chunk whose swizzled home is 16*lane:
+  int l_chunk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) l_chunk[i] = (lane & 7) ^ swz_key(8 * (wave + 8 * i) + l_row);
+  const uint16_t* a_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 8 * (wave + 8 * i) + l_row;
+    a_src[i] = A + (int64_t)min(m0 + row, M - 1) * lda;
+  }
+  const uint16_t* w_src[4];
+  if (!W8) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int lrow = 8 * (wave + 8 * i) + l_row;  // LDS row; holds weight row blk + 16*g + 4*q + s
+      const int r = lrow & 31;
+      const int n = (lrow & ~31) + 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+      w_src[i] = static_cast<const uint16_t*>(Wv) + (int64_t)min(n0 + n, N - 1) * ldw;
+    }
+  }
+  // W8: 256 rows x 4 chunks of 16 int8 through registers; thread -> chunk tid%4, rows tid/4 + 128*i
+  u32x4_t rw[2];
+  float wscale[2], woff[2];
+  const int8_t* q_src[2];
+  const int q_chunk = tid & 3;
+  if (W8) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int n = min(n0 + (tid >> 2) + 128 * i, N - 1);
+      q_src[i] = static_cast<const int8_t*>(Wv) + (int64_t)n * ldw;
+      wscale[i] = scale[n];
+      woff[i] = -128.f * wscale[i];
+    }
+  }
+  auto issue = [&](int stage, int k0) {
+    unsigned char* sa = smem + stage * 2 * TILE_BYTES;
+    unsigned char* sw = sa + TILE_BYTES;
+    int k[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) k[i] = min(k0 + 8 * l_chunk[i], K - 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds(SANA_GPTR(a_src[i] + k[i]), SANA_LPTR(sa + (wave + 8 * i) * 1024), 16, 0, 0);
+    if (!W8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        __builtin_amdgcn_global_load_lds(SANA_GPTR(w_src[i] + k[i]), SANA_LPTR(sw + (wave + 8 * i) * 1024), 16, 0,
+                                         0);
+    } else {
+      const int kq = min(k0 + 16 * q_chunk, K - 16);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) rw[i] = *reinterpret_cast<const u32x4_t*>(q_src[i] + kq);
+    }
+  };
+  auto store_w8 = [&](int stage) {
+    unsigned char* sw = smem + stage * 2 * TILE_BYTES + TILE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int lrow = wrow_to_lds((tid >> 2) + 128 * i);
+      u32x4_t q = rw[i];
+      q.x ^= 0x80808080u;
+      q.y ^= 0x80808080u;
+      q.z ^= 0x80808080u;
+      q.w ^= 0x80808080u;
+      u32x4_t lo, hi;
+      lo.x = dequant2(q.x, 0, wscale[i], woff[i]);
+      lo.y = dequant2(q.x, 1, wscale[i], woff[i]);
+      lo.z = dequant2(q.y, 0, wscale[i], woff[i]);
+      lo.w = dequant2(q.y, 1, wscale[i], woff[i]);
+      hi.x = dequant2(q.z, 0, wscale[i], woff[i]);
+      hi.y = dequant2(q.z, 1, wscale[i], woff[i]);
+      hi.z = dequant2(q.w, 0, wscale[i], woff[i]);
+      hi.w = dequant2(q.w, 1, wscale[i], woff[i]);
+      *reinterpret_cast<u32x4_t*>(sw + swz(lrow, 2 * q_chunk)) = lo;
+      *reinterpret_cast<u32x4_t*>(sw + swz(lrow, 2 * q_chunk + 1)) = hi;
+    }
+  };
+
+  // ---- MFMA tiling: wave (wc, wt): channels [wc*128, +128) x tokens [wt*64, +64)
+  const int wc = wave & 1, wt = wave >> 1;
+  const int fr = lane & 31, fg = lane >> 5;
+  const int x7 = swz_key(fr);  // tile-row bases are multiples of 32
+  const int w_off = (wc * 128 + fr) * ROW_BYTES, a_off = (wt * 64 + fr) * ROW_BYTES;
+  f32x16_t acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int KT = (K + BK - 1) / BK;
+  const int tail_steps = (K - (KT - 1) * BK) / 16;  // 1..4 k-steps of 16 on the last tile
+  issue(0, 0);
+  if (W8) store_w8(0);
+  __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): direct-to-LDS data has landed
+  __syncthreads();
+  for (int kt = 0; kt + 1 < KT; ++kt) {
+    const int cur = kt & 1;
+    issue(cur ^ 1, (kt + 1) * BK);
+    const unsigned char* sa = smem + cur * 2 * TILE_BYTES;
+    mma_tile<true>(sa, sa + TILE_BYTES, a_off, w_off, x7, fg, 4, acc);
+    if (W8) store_w8(cur ^ 1);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+  }
+  {
+    const unsigned char* sa = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
+    mma_tile<false>(sa, sa + TILE_BYTES, a_off, w_off, x7, fg, tail_steps, acc);
+  }
+
+  // ---- epilogue.  acc[i][j][r]: token m0 + wt*64 + 32*j + lane%32,
+  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + wc * 128 + 32 * i + 16 * fg;
+    float bv[16];
+    if (EPI != SANA_EPI_NONE) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bv[r] = (n + r < N) ? bf16_bits_to_f32(bias[n + r]) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + wt * 64 + 32 * j + fr;
+      if (m >= M) continue;
+      uint16_t* cp = C + (int64_t)m * ldc + n;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (n + 8 * half < N) {
+          float v[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            float x = acc[i][j][8 * half + r];
+            if (EPI != SANA_EPI_NONE) x += bv[8 * half + r];
+            if (EPI == SANA_EPI_BIAS_SILU) x = silu_f32(round_bf16(x));
+            v[r] = x;
+          }
+          u32x4_t o;
+          o.x = pack_bf16(v[0], v[1]);
+          o.y = pack_bf16(v[2], v[3]);
+          o.z = pack_bf16(v[4], v[5]);
+          o.w = pack_bf16(v[6], v[7]);
+          *reinterpret_cast<u32x4_t*>(cp + 8 * half) = o;
+        }
+      }
+    }
+  }
+}
+
 template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const void* bias, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + BC - 1) / BC;
   const int64_t total = (int64_t)tiles_t * tiles_c;
   if (total > (1 << 30)) return SANA_ERR_SHAPE;
-  dim3 grid((unsigned)total), block(256);
   const uint16_t* a = static_cast<const uint16_t*>(A);
   const uint16_t* b = static_cast<const uint16_t*>(bias);
   uint16_t* c = static_cast<uint16_t*>(C);
+  const bool fast = (K % 16 == 0);  // the generic kernel also takes K % 8 == 0
+  dim3 grid((unsigned)total), block(fast ? 512 : 256);
+#define SANA_LAUNCH(EPI)                                                                                          \
+  if (fast)                                                                                                       \
+    hipLaunchKernelGGL((gemm_fast_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw, ldc,  \
+                       tiles_t, tiles_c);                                                                         \
+  else                                                                                                            \
+    hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw, ldc,       \
+                       tiles_t, tiles_c)
   switch (epilogue) {
-    case SANA_EPI_NONE:
-      hipLaunchKernelGGL((gemm_kernel<W8, SANA_EPI_NONE>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw,
-                         ldc, tiles_t, tiles_c);
-      break;
-    case SANA_EPI_BIAS:
-      hipLaunchKernelGGL((gemm_kernel<W8, SANA_EPI_BIAS>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw,
-                         ldc, tiles_t, tiles_c);
-      break;
-    case SANA_EPI_BIAS_SILU:
-      hipLaunchKernelGGL((gemm_kernel<W8, SANA_EPI_BIAS_SILU>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda,
-                         ldw, ldc, tiles_t, tiles_c);
-      break;
-    default:
-      return SANA_ERR_ARG;
+    case SANA_EPI_NONE: SANA_LAUNCH(SANA_EPI_NONE); break;
+    case SANA_EPI_BIAS: SANA_LAUNCH(SANA_EPI_BIAS); break;
+    case SANA_EPI_BIAS_SILU: SANA_LAUNCH(SANA_EPI_BIAS_SILU); break;
+    default: return SANA_ERR_ARG;
   }
+#undef SANA_LAUNCH
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
