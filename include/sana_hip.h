@@ -160,6 +160,35 @@ int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, con
                         void* C, int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                         int epilogue, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Fused seams around the two modules (the reference runs them as separate
+ * elementwise torch ops inside SanaMSBlock.forward,
+ * diffusion/model/nets/sana_multi_scale.py:148-155, sana_blocks.py:44-45).
+ *
+ * GEMM + gated residual:  C = residual + gate[row / rows_per_gate] * (A W^T + bias)
+ *   replaces `x + gate_msa * attn(...)` / `x + gate_mlp * mlp(...)` (:151-155)
+ *   together with the module's last linear (proj / point_conv).  bf16 only.
+ *   W is bf16 [N][K] when w8_scale is NULL, else int8 [N][K] with fp32 scales.
+ *   gate: bf16 rows of N values, gate_stride elements apart, one row per
+ *   rows_per_gate consecutive rows of C (= tokens per batch element);
+ *   residual: bf16 [M][N] with row stride ldr (may alias C).  bias may be NULL.
+ *   The linear output, the gate product and the sum are each rounded to bf16,
+ *   as the reference's three ops do.
+ */
+int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_scale, const void* bias,
+                                const void* gate, const void* residual, void* C,
+                                int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc,
+                                int rows_per_gate, int64_t gate_stride, void* stream);
+
+/* LayerNorm without affine (eps inside the rsqrt) + adaLN modulation:
+ *   out[m][:] = LN(x[m][:]) * (1 + scale[m / rows_per_mod][:]) + shift[m / rows_per_mod][:]
+ *   replaces `t2i_modulate(self.norm1(x), shift, scale)` (sana_multi_scale.py:152,155).
+ *   x, out: bf16 [M][C] with row strides ldx / ldo; scale, shift: bf16 rows of C
+ *   values, mod_stride elements apart.  C % 8 == 0, C <= 8192.  bf16 only. */
+int sana_hip_layernorm_modulate(const void* x, const void* scale, const void* shift, void* out,
+                                int64_t M, int C, int64_t ldx, int64_t ldo,
+                                int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

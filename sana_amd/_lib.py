@@ -33,6 +33,11 @@ SIGNATURES = {
                                    c_int64, c_int64, c_int64, c_int, c_void_p]),
     "sana_hip_gemm_w8a16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "sana_hip_gemm_gate_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64,
+                                            c_int, c_int64, c_void_p]),
+    "sana_hip_layernorm_modulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
+                                            c_int64, c_int64, c_int, c_int64, c_float, c_int, c_void_p]),
 }
 
 _lib = None

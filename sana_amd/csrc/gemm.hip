@@ -46,10 +46,57 @@ __device__ __forceinline__ uint32_t dequant2(uint32_t q4, int which, float s, fl
   return pack_bf16(fmaf(f0, s, off), fmaf(f1, s, off));
 }
 
+// Epilogue operands.  SANA_EPI_GATE_RES: C = res + gate[row / rows_per_gate] * (acc + bias), i.e. the
+// gated residual update of the block (x + gate * module(x)), with the reference's three roundings
+// (linear output, gate product, residual sum) reproduced in registers.
+struct EpiArgs {
+  const uint16_t* bias;  // [N] or null
+  const uint16_t* gate;  // [*, N] rows gate_stride apart, one row per rows_per_gate rows of C
+  const uint16_t* res;   // [M, N] with row stride ldr
+  int64_t ldr, gate_stride;
+  int rows_per_gate;
+};
+#define SANA_EPI_GATE_RES 3
+
+// 8 outputs of one row: accumulator (+bias) -> io dtype, per the epilogue kind (everything except
+// the gated residual, which needs the row's residual and gate and is applied at store time).
+template <int EPI>
+__device__ __forceinline__ u32x4_t epi_pack8(const float* a, const float* bv) {
+  float v[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    float x = a[r];
+    if (EPI != SANA_EPI_NONE) x += bv[r];
+    if (EPI == SANA_EPI_BIAS_SILU) x = silu_f32(round_bf16(x));  // the reference rounds before the activation
+    v[r] = x;
+  }
+  u32x4_t o;
+  o.x = pack_bf16(v[0], v[1]);
+  o.y = pack_bf16(v[2], v[3]);
+  o.z = pack_bf16(v[4], v[5]);
+  o.w = pack_bf16(v[6], v[7]);
+  return o;
+}
+__device__ __forceinline__ uint32_t gate_res2(uint32_t y, uint32_t g, uint32_t r) {
+  const float t0 = round_bf16(bf16_lo(g) * bf16_lo(y)), t1 = round_bf16(bf16_hi(g) * bf16_hi(y));
+  return pack_bf16(bf16_lo(r) + t0, bf16_hi(r) + t1);
+}
+// y: 8 linear outputs (already rounded to bf16) of row m, columns n..n+7
+__device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m, int n) {
+  const u32x4_t g = *reinterpret_cast<const u32x4_t*>(e.gate + (int64_t)(m / e.rows_per_gate) * e.gate_stride + n);
+  const u32x4_t r = *reinterpret_cast<const u32x4_t*>(e.res + (int64_t)m * e.ldr + n);
+  u32x4_t o;
+  o.x = gate_res2(y.x, g.x, r.x);
+  o.y = gate_res2(y.y, g.y, r.y);
+  o.z = gate_res2(y.z, g.z, r.z);
+  o.w = gate_res2(y.w, g.w, r.w);
+  return o;
+}
+
 template <bool W8, int EPI>
 __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
-                                                   const float* __restrict__ scale,
-                                                   const uint16_t* __restrict__ bias, uint16_t* __restrict__ C,
+                                                   const float* __restrict__ scale, const EpiArgs ep,
+                                                   uint16_t* __restrict__ C,
                                                    int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                                                    int tiles_t, int tiles_c) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
@@ -189,35 +236,28 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 
   // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 32*j + lane%32,
   // channel n0 + wc*128 + 32*i + 16*(lane/32) + r
+  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int n = n0 + wc * 128 + 32 * i + 16 * fg;
     float bv[16];
-    if (EPI != SANA_EPI_NONE) {
+    if (HAS_BIAS) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) bv[r] = (n + r < N) ? bf16_bits_to_f32(bias[n + r]) : 0.f;
+      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int m = m0 + wt * 128 + 32 * j + fr;
       if (m >= M) continue;
-      float v[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = acc[i][j][r];
-        if (EPI != SANA_EPI_NONE) x += bv[r];
-        if (EPI == SANA_EPI_BIAS_SILU) x = silu_f32(round_bf16(x));  // the reference rounds before the activation
-        v[r] = x;
-      }
       uint16_t* cp = C + (int64_t)m * ldc + n;
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         if (n + 8 * half < N) {  // N % 8 == 0: a chunk is either fully inside or outside
-          u32x4_t o;
-          o.x = pack_bf16(v[8 * half + 0], v[8 * half + 1]);
-          o.y = pack_bf16(v[8 * half + 2], v[8 * half + 3]);
-          o.z = pack_bf16(v[8 * half + 4], v[8 * half + 5]);
-          o.w = pack_bf16(v[8 * half + 6], v[8 * half + 7]);
+          float a8[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
+          u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
+          if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n + 8 * half);
           *reinterpret_cast<u32x4_t*>(cp + 8 * half) = o;
         }
       }
@@ -268,8 +308,8 @@ __device__ __forceinline__ void mma_tile(const unsigned char* __restrict__ sa, c
 
 template <bool W8, int EPI>
 __global__ __launch_bounds__(512) void gemm_fast_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
-                                                        const float* __restrict__ scale,
-                                                        const uint16_t* __restrict__ bias, uint16_t* __restrict__ C,
+                                                        const float* __restrict__ scale, const EpiArgs ep,
+                                                        uint16_t* __restrict__ C,
                                                         int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                                                         int tiles_t, int tiles_c) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
@@ -404,65 +444,75 @@ __global__ __launch_bounds__(512) void gemm_fast_kernel(const uint16_t* __restri
   }
 
   // ---- epilogue.  acc[i][j][r]: token m0 + wt*64 + 32*j + lane%32,
-  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r
+  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r.  In that layout a lane owns 32-byte pieces of 32
+  // different rows; the sub-tile goes through wave-private LDS ([64 tokens][256 bytes], 16-byte chunks
+  // XOR-swizzled by token % 16) and comes back row-contiguous, so each store instruction writes four
+  // full 256-byte row segments and the residual / gate reads of the fused update are coalesced too.
+  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
+  __syncthreads();  // every wave is done with the operand tiles
+  unsigned char* stg = smem + wave * 16384;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int n = n0 + wc * 128 + 32 * i + 16 * fg;
+    const int nl = 32 * i + 16 * fg;  // channel inside the wave's 128
     float bv[16];
-    if (EPI != SANA_EPI_NONE) {
+    if (HAS_BIAS) {
+      const int n = n0 + wc * 128 + nl;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) bv[r] = (n + r < N) ? bf16_bits_to_f32(bias[n + r]) : 0.f;
+      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int m = m0 + wt * 64 + 32 * j + fr;
-      if (m >= M) continue;
-      uint16_t* cp = C + (int64_t)m * ldc + n;
+      const int tok = 32 * j + fr;
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        if (n + 8 * half < N) {
-          float v[8];
+        float a8[8];
 #pragma unroll
-          for (int r = 0; r < 8; ++r) {
-            float x = acc[i][j][8 * half + r];
-            if (EPI != SANA_EPI_NONE) x += bv[8 * half + r];
-            if (EPI == SANA_EPI_BIAS_SILU) x = silu_f32(round_bf16(x));
-            v[r] = x;
-          }
-          u32x4_t o;
-          o.x = pack_bf16(v[0], v[1]);
-          o.y = pack_bf16(v[2], v[3]);
-          o.z = pack_bf16(v[4], v[5]);
-          o.w = pack_bf16(v[6], v[7]);
-          *reinterpret_cast<u32x4_t*>(cp + 8 * half) = o;
-        }
+        for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
+        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
+        const int chunk = (nl >> 3) + half;
+        *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+  {
+    const int chunk = lane & 15, rsub = lane >> 4;
+    const int n = n0 + wc * 128 + chunk * 8;
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+      const int row = it * 4 + rsub;
+      const int m = m0 + wt * 64 + row;
+      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((chunk ^ (row & 15)) << 4));
+      if (m < M && n < N) {
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
+        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
       }
     }
   }
 }
 
 template <bool W8>
-int launch(const void* A, const void* W, const float* scale, const void* bias, void* C, int M, int N, int K,
+int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + BC - 1) / BC;
   const int64_t total = (int64_t)tiles_t * tiles_c;
   if (total > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
-  const uint16_t* b = static_cast<const uint16_t*>(bias);
   uint16_t* c = static_cast<uint16_t*>(C);
   const bool fast = (K % 16 == 0);  // the generic kernel also takes K % 8 == 0
   dim3 grid((unsigned)total), block(fast ? 512 : 256);
 #define SANA_LAUNCH(EPI)                                                                                          \
   if (fast)                                                                                                       \
-    hipLaunchKernelGGL((gemm_fast_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw, ldc,  \
+    hipLaunchKernelGGL((gemm_fast_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
                        tiles_t, tiles_c);                                                                         \
   else                                                                                                            \
-    hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, b, c, M, N, K, lda, ldw, ldc,       \
+    hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc,      \
                        tiles_t, tiles_c)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH(SANA_EPI_NONE); break;
     case SANA_EPI_BIAS: SANA_LAUNCH(SANA_EPI_BIAS); break;
     case SANA_EPI_BIAS_SILU: SANA_LAUNCH(SANA_EPI_BIAS_SILU); break;
+    case SANA_EPI_GATE_RES: SANA_LAUNCH(SANA_EPI_GATE_RES); break;
     default: return SANA_ERR_ARG;
   }
 #undef SANA_LAUNCH
@@ -472,12 +522,25 @@ int launch(const void* A, const void* W, const float* scale, const void* bias, v
 int check_common(const void* A, const void* W, const void* bias, const void* C, int M, int N, int K, int64_t lda,
                  int64_t ldw, int64_t ldc, int epilogue, int kmult, int ldw_mult) {
   if (!A || !W || !C || M <= 0 || N <= 0 || K <= 0) return SANA_ERR_ARG;
-  if (epilogue != SANA_EPI_NONE && !bias) return SANA_ERR_ARG;
-  if (epilogue < SANA_EPI_NONE || epilogue > SANA_EPI_BIAS_SILU) return SANA_ERR_ARG;
+  if ((epilogue == SANA_EPI_BIAS || epilogue == SANA_EPI_BIAS_SILU) && !bias) return SANA_ERR_ARG;
+  if (epilogue < SANA_EPI_NONE || epilogue > SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   if (K % kmult || N % 8) return SANA_ERR_SHAPE;
   if (lda < K || ldw < K || ldc < N) return SANA_ERR_ARG;
   if (lda % 8 || ldw % ldw_mult || ldc % 8 || !aligned16(A) || !aligned16(W) || !aligned16(C)) return SANA_ERR_ALIGN;
   return SANA_OK;
+}
+
+int check_gate_res(const void* gate, const void* residual, int M, int N, int64_t ldr, int rows_per_gate,
+                   int64_t gate_stride) {
+  if (!gate || !residual || rows_per_gate <= 0) return SANA_ERR_ARG;
+  if (ldr < N || gate_stride < 0) return SANA_ERR_ARG;
+  if (ldr % 8 || gate_stride % 8 || !aligned16(gate) || !aligned16(residual)) return SANA_ERR_ALIGN;
+  return SANA_OK;
+}
+
+EpiArgs plain_epi(const void* bias) {
+  EpiArgs e = {static_cast<const uint16_t*>(bias), nullptr, nullptr, 0, 0, 1};
+  return e;
 }
 
 }  // namespace
@@ -485,22 +548,39 @@ int check_common(const void* A, const void* W, const void* bias, const void* C, 
 
 using namespace sana;
 
-extern "C" __attribute__((visibility("default"))) int sana_hip_gemm_bf16(const void* A, const void* W,
-                                                                         const void* bias, void* C, int M, int N,
-                                                                         int K, int64_t lda, int64_t ldw,
-                                                                         int64_t ldc, int epilogue, void* stream) {
+#define SANA_API extern "C" __attribute__((visibility("default")))
+
+SANA_API int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,
+                                int64_t lda, int64_t ldw, int64_t ldc, int epilogue, void* stream) {
+  if (epilogue == SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   const int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, epilogue, 8, 8);
   if (rc != SANA_OK) return rc;
-  return launch<false>(A, W, nullptr, bias, C, M, N, K, lda, ldw, ldc, epilogue, static_cast<hipStream_t>(stream));
+  return launch<false>(A, W, nullptr, plain_epi(bias), C, M, N, K, lda, ldw, ldc, epilogue,
+                       static_cast<hipStream_t>(stream));
 }
 
-extern "C" __attribute__((visibility("default"))) int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq,
-                                                                          const float* scale, const void* bias,
-                                                                          void* C, int M, int N, int K, int64_t lda,
-                                                                          int64_t ldw, int64_t ldc, int epilogue,
-                                                                          void* stream) {
-  if (!scale) return SANA_ERR_ARG;
+SANA_API int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias, void* C,
+                                 int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
+                                 void* stream) {
+  if (!scale || epilogue == SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   const int rc = check_common(A, Wq, bias, C, M, N, K, lda, ldw, ldc, epilogue, 16, 16);
   if (rc != SANA_OK) return rc;
-  return launch<true>(A, Wq, scale, bias, C, M, N, K, lda, ldw, ldc, epilogue, static_cast<hipStream_t>(stream));
+  return launch<true>(A, Wq, scale, plain_epi(bias), C, M, N, K, lda, ldw, ldc, epilogue,
+                      static_cast<hipStream_t>(stream));
+}
+
+SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_scale, const void* bias,
+                                         const void* gate, const void* residual, void* C, int M, int N, int K,
+                                         int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc, int rows_per_gate,
+                                         int64_t gate_stride, void* stream) {
+  const bool w8 = w8_scale != nullptr;
+  int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, w8 ? 16 : 8, w8 ? 16 : 8);
+  if (rc != SANA_OK) return rc;
+  rc = check_gate_res(gate, residual, M, N, ldr, rows_per_gate, gate_stride);
+  if (rc != SANA_OK) return rc;
+  const EpiArgs e = {static_cast<const uint16_t*>(bias), static_cast<const uint16_t*>(gate),
+                     static_cast<const uint16_t*>(residual), ldr, gate_stride, rows_per_gate};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return w8 ? launch<true>(A, W, w8_scale, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s)
+            : launch<false>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s);
 }

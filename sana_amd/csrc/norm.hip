@@ -1,0 +1,116 @@
+// LayerNorm (no affine) fused with the adaLN-single modulation, for gfx950:
+//
+//   out[b, n, :] = LN(x[b, n, :]) * (1 + scale[b, :]) + shift[b, :]
+//
+// HBM bound: one read and one write of the activation (2 * M * C * 2 bytes).
+// One wave per token row; the row lives in registers as raw 16-byte chunks
+// (lane l holds chunks l, l+64, ...), so it is read from memory once: mean and
+// the centred variance are two register passes with wave reductions, the third
+// pass normalises, modulates and stores.  The four roundings of the stock op
+// chain (layer_norm -> 1+scale -> product -> +shift, each a bf16 tensor) are
+// reproduced in registers.
+#include "common.h"
+
+namespace sana {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// NCH: 16-byte chunks per lane (C <= 512 * NCH)
+template <int NCH>
+__global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __restrict__ x,
+                                                          const uint16_t* __restrict__ scale,
+                                                          const uint16_t* __restrict__ shift,
+                                                          uint16_t* __restrict__ out, int64_t M, int C,
+                                                          int64_t ldx, int64_t ldo, int rows_per_mod,
+                                                          int64_t mod_stride, float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= M) return;  // no barriers in this kernel
+  const int nchunks = C >> 3;
+  const uint16_t* xr = x + row * ldx;
+  u32x4_t raw[NCH];
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int ch = lane + 64 * i;
+    raw[i] = ch < nchunks ? *reinterpret_cast<const u32x4_t*>(xr + 8 * ch) : zero4;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s += bf16_lo(raw[i][e]) + bf16_hi(raw[i][e]);
+  const float mean = wave_sum(s) / (float)C;
+  float v = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    if (lane + 64 * i < nchunks) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float a = bf16_lo(raw[i][e]) - mean, b = bf16_hi(raw[i][e]) - mean;
+        v = fmaf(a, a, v);
+        v = fmaf(b, b, v);
+      }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(v) / (float)C + eps);
+  const int64_t mod = (row / rows_per_mod) * mod_stride;
+  uint16_t* orow = out + row * ldo;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int ch = lane + 64 * i;
+    if (ch < nchunks) {
+      const u32x4_t sc = *reinterpret_cast<const u32x4_t*>(scale + mod + 8 * ch);
+      const u32x4_t sh = *reinterpret_cast<const u32x4_t*>(shift + mod + 8 * ch);
+      u32x4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t ln = pack_bf16((bf16_lo(raw[i][e]) - mean) * rstd, (bf16_hi(raw[i][e]) - mean) * rstd);
+        const uint32_t s1 = pack_bf16(1.0f + bf16_lo(sc[e]), 1.0f + bf16_hi(sc[e]));
+        const uint32_t t = pack_bf16(bf16_lo(ln) * bf16_lo(s1), bf16_hi(ln) * bf16_hi(s1));
+        o[e] = pack_bf16(bf16_lo(t) + bf16_lo(sh[e]), bf16_hi(t) + bf16_hi(sh[e]));
+      }
+      *reinterpret_cast<u32x4_t*>(orow + 8 * ch) = o;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace sana
+
+using namespace sana;
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_layernorm_modulate(
+    const void* x, const void* scale, const void* shift, void* out, int64_t M, int C, int64_t ldx, int64_t ldo,
+    int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream) {
+  if (!x || !scale || !shift || !out || M <= 0 || C <= 0 || rows_per_mod <= 0) return SANA_ERR_ARG;
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (C % 8 || C > 8192) return SANA_ERR_SHAPE;
+  if (ldx < C || ldo < C || mod_stride < 0) return SANA_ERR_ARG;
+  if (ldx % 8 || ldo % 8 || mod_stride % 8 || !aligned16(x) || !aligned16(out) || !aligned16(scale) ||
+      !aligned16(shift))
+    return SANA_ERR_ALIGN;
+  if ((M + 3) / 4 > 0x7fffffff) return SANA_ERR_SHAPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)((M + 3) / 4)), block(256);
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  const uint16_t* sc = static_cast<const uint16_t*>(scale);
+  const uint16_t* sh = static_cast<const uint16_t*>(shift);
+  uint16_t* op = static_cast<uint16_t*>(out);
+  const int nch = (C / 8 + 63) / 64;
+#define SANA_LN(NCH) \
+  hipLaunchKernelGGL((ln_modulate_kernel<NCH>), grid, block, 0, s, xp, sc, sh, op, M, C, ldx, ldo, rows_per_mod, \
+                     mod_stride, eps)
+  if (nch <= 2) SANA_LN(2);
+  else if (nch <= 3) SANA_LN(3);
+  else if (nch <= 5) SANA_LN(5);
+  else if (nch <= 8) SANA_LN(8);
+  else SANA_LN(16);
+#undef SANA_LN
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}

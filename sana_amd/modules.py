@@ -55,16 +55,22 @@ class HipLinear(nn.Linear):
     def is_quantized(self) -> bool:
         return getattr(self, "weight_q", None) is not None
 
-    def forward(self, x: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, epilogue: Optional[str] = None, gate=None, residual=None) -> torch.Tensor:
         return hip_linear(x, self.weight, self.bias, epilogue,
-                          getattr(self, "weight_q", None), getattr(self, "weight_scale", None))
+                          getattr(self, "weight_q", None), getattr(self, "weight_scale", None), gate, residual)
 
 
-def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None):
-    """y = epilogue(x @ W^T + b) over the last dim of x.  epilogue: None | "silu"."""
+def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None, gate=None, residual=None):
+    """y = epilogue(x @ W^T + b) over the last dim of x.  epilogue: None | "silu".
+    With ``gate`` [B, 1, C] and ``residual`` [B, N, C]: residual + gate * y (one fused kernel in bf16)."""
     _no_grad_only(x, weight, bias)
     lead = x.shape[:-1]
     K = x.shape[-1]
+    if gate is not None:
+        if x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 3 and epilogue is None:
+            w = weight_q if weight_q is not None else weight
+            return ops.gemm_gate_residual(x, w, bias, gate, residual, weight_scale if weight_q is not None else None)
+        return residual + gate * hip_linear(x, weight, bias, epilogue, weight_q, weight_scale)
     if x.dtype == torch.bfloat16 and x.is_cuda:
         x2 = x.reshape(-1, K)
         if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
@@ -206,10 +212,14 @@ class LiteLA(nn.Module):
 
     def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_id=None,
                 block_mask=None) -> torch.Tensor:
+        return self.forward_gated(x, None, None, rotary_emb=rotary_emb)
+
+    def forward_gated(self, x, gate, residual, rotary_emb=None) -> torch.Tensor:
+        """forward(x), or residual + gate * forward(x) with the update fused into the proj GEMM."""
         _no_grad_only(x)
         qkv = self._qkv_tokens(x, rotary_emb)
         out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps)
-        return self.proj(out)
+        return self.proj(out, gate=gate, residual=residual)
 
     def quantize_w8_(self) -> "LiteLA":
         self.qkv.quantize_w8_()
@@ -296,6 +306,10 @@ class GLUMBConv(nn.Module):
         self.round_like_reference = True
 
     def forward(self, x: torch.Tensor, HW=None) -> torch.Tensor:
+        return self.forward_gated(x, HW, None, None)
+
+    def forward_gated(self, x, HW, gate, residual) -> torch.Tensor:
+        """forward(x, HW), or residual + gate * forward(x, HW) fused into the point-conv GEMM."""
         _no_grad_only(x)
         B, N, C = x.shape
         if HW is None:
@@ -312,7 +326,7 @@ class GLUMBConv(nn.Module):
         y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
                                     round_like_reference=self.round_like_reference)
         out = hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
-                         getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None))
+                         getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual)
         return out
 
     def quantize_w8_(self) -> "GLUMBConv":
@@ -433,6 +447,13 @@ class SanaMSBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
             self.scale_shift_table[None] + t.reshape(B, 6, -1)
         ).chunk(6, dim=1)
+        if x.is_cuda and x.dtype == torch.bfloat16 and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
+            # fused seams: LayerNorm + modulate in one kernel, gate * out + residual in the GEMM epilogue
+            h = ops.layernorm_modulate(x, scale_msa, shift_msa, self.norm1.eps)
+            x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
+            x = x + self.cross_attn(x, y, mask)
+            h = ops.layernorm_modulate(x, scale_mlp, shift_mlp, self.norm2.eps)
+            return self.mlp.forward_gated(h, HW, gate_mlp, x)
         x = x + self.drop_path(
             gate_msa * self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), HW=HW, rotary_emb=image_rotary_emb))
         x = x + self.cross_attn(x, y, mask)

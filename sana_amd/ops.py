@@ -219,3 +219,52 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
                                            M, N, K, lda, ldw, ldc, epi, _stream())
     _lib.check(code, "sana_hip_gemm_w8a16")
     return out
+
+
+# --------------------------------------------------------------------------- fused seams of the block
+
+def _mod_rows(t: torch.Tensor, B: int, C: int, what: str) -> Tuple[torch.Tensor, int]:
+    """Per-batch row vectors [B, 1, C] / [B, C] with unit inner stride -> (tensor, batch stride)."""
+    if t.dim() == 3 and t.shape[1] == 1:
+        t = t[:, 0]
+    if t.dim() != 2 or t.shape != (B, C) or t.stride(1) != 1:
+        raise SanaHipError(f"{what} must be [B, C] (or [B, 1, C]) with unit inner stride, got {tuple(t.shape)}")
+    return t, (t.stride(0) if B > 1 else 0)
+
+
+def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], gate: torch.Tensor,
+                       residual: torch.Tensor, weight_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """residual + gate * (a @ weight.T + bias) with a: [B, N, K], residual: [B, N, C], gate: [B, 1, C].
+    weight is bf16 [C, K], or int8 with ``weight_scale`` (W8A16)."""
+    _need_cuda(a, weight, bias, gate, residual, weight_scale)
+    B, Ntok, K = a.shape
+    C = weight.shape[0]
+    if a.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or gate.dtype != torch.bfloat16:
+        raise SanaHipError("gemm_gate_residual is bf16 only")
+    a2, lda = _rows(a.reshape(B * Ntok, K), "a")
+    w2, ldw = _rows(weight.reshape(C, -1), "weight")
+    r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
+    g2, gstride = _mod_rows(gate, B, C, "gate")
+    out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=a.device)
+    code = _lib.load().sana_hip_gemm_gate_residual(
+        a2.data_ptr(), w2.data_ptr(), weight_scale.data_ptr() if weight_scale is not None else None,
+        bias.data_ptr() if bias is not None else None, g2.data_ptr(), r2.data_ptr(), out.data_ptr(),
+        B * Ntok, C, K, lda, ldw, ldr, C, Ntok, gstride, _stream())
+    _lib.check(code, "sana_hip_gemm_gate_residual")
+    return out.view(B, Ntok, C)
+
+
+def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """LN(x) * (1 + scale) + shift over the last dim; x: [B, N, C] bf16, scale/shift: [B, 1, C]."""
+    _need_cuda(x, scale, shift)
+    B, Ntok, C = x.shape
+    x2, ldx = _rows(x.reshape(B * Ntok, C), "x")
+    sc, s1 = _mod_rows(scale, B, C, "scale")
+    sh, s2 = _mod_rows(shift, B, C, "shift")
+    if s1 != s2:
+        raise SanaHipError("scale and shift must share their batch stride")
+    out = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
+    code = _lib.load().sana_hip_layernorm_modulate(x2.data_ptr(), sc.data_ptr(), sh.data_ptr(), out.data_ptr(),
+                                                   B * Ntok, C, ldx, C, Ntok, s1, float(eps), _dt(x), _stream())
+    _lib.check(code, "sana_hip_layernorm_modulate")
+    return out.view(B, Ntok, C)

@@ -156,3 +156,48 @@ def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilog
     assert torch.equal(y8, y16)
     ref = _gemm_ref(a.cpu(), wd, None if bias is None else bias.cpu(), epilogue)
     assert rel_l2(y8.cpu(), ref) <= 4e-3
+
+
+# ---------------------------------------------------------------- fused seams of the block
+
+
+@pytest.mark.parametrize("B,Ntok,C,K,w8", [(1, 16384, 2240, 2240, False), (2, 1024, 2240, 5600, False),
+                                          (3, 100, 96, 240, False), (2, 1024, 2240, 5600, True)])
+def test_gemm_gate_residual_matches_stock_op_chain(cuda, B, Ntok, C, K, w8):
+    g = torch.Generator().manual_seed(B + K)
+    a = torch.randn(B, Ntok, K, generator=g).bfloat16().to(cuda)
+    w = (torch.randn(C, K, generator=g) * 0.03).bfloat16()
+    bias = (torch.randn(C, generator=g) * 0.1).bfloat16().to(cuda)
+    mod = (torch.randn(B, 6, C, generator=g) * 0.5).bfloat16().to(cuda)   # gate is a strided view, as in the block
+    gate = mod[:, 2:3]
+    res = torch.randn(B, Ntok, C, generator=g).bfloat16().to(cuda)
+    if w8:
+        wq, s = O.quantize_w8(w)
+        w = O.dequantize_w8(wq, s)
+        out = ops.gemm_gate_residual(a, wq.to(cuda), bias, gate, res, s.to(cuda))
+    else:
+        out = ops.gemm_gate_residual(a, w.to(cuda), bias, gate, res)
+    # the reference's op chain in bf16: linear -> gate * y -> x + (.)
+    y = ops.gemm_bf16(a.view(-1, K), w.to(cuda), bias, "bias").view(B, Ntok, C)
+    chain = res + gate * y
+    assert torch.equal(out, chain)
+    ref = res.double() + gate.double() * (a.double() @ w.double().to(cuda).T + bias.double())
+    assert rel_l2(out, ref) <= 4e-3
+
+
+@pytest.mark.parametrize("B,Ntok,C", [(1, 16384, 2240), (4, 1024, 1152), (2, 77, 96), (1, 5, 4096)])
+def test_layernorm_modulate_matches_stock_op_chain(cuda, B, Ntok, C):
+    g = torch.Generator().manual_seed(C)
+    x = (torch.randn(B, Ntok, C, generator=g) * 2 + 0.3).bfloat16().to(cuda)
+    mod = (torch.randn(B, 6, C, generator=g) * 0.3).bfloat16().to(cuda)
+    shift, scale = mod[:, 0:1], mod[:, 1:2]
+    out = ops.layernorm_modulate(x, scale, shift, 1e-6)
+    ref64 = F.layer_norm(x.double(), (C,), eps=1e-6) * (1 + scale.double()) + shift.double()
+    assert rel_l2(out, ref64) <= 4e-3
+    chain = F.layer_norm(x, (C,), eps=1e-6) * (1 + scale) + shift      # stock bf16 chain (four roundings)
+    diff = (out.float() - chain.float()).abs()
+    # same rounding points: equal except where the fp32 statistics differ in the last bit; a flipped
+    # rounding of the product is one bf16 ulp of the product, which the final sum may partly cancel
+    mag = chain.float().abs() + shift.float().abs()
+    assert (diff > 2 ** -6 * mag + 1e-6).sum().item() == 0
+    assert (diff == 0).float().mean().item() > 0.98
