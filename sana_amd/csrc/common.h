@@ -77,6 +77,20 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32_bf16(u32x4_t a, u32x4_t b, f32x
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// acc + lo(x) + hi(x) for two packed 16-bit floats: one dot2 against (1, 1), fp32 accumulate
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <typename T>
+__device__ __forceinline__ float add_pk16(uint32_t x, float acc);
+template <>
+__device__ __forceinline__ float add_pk16<BF16>(uint32_t x, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc,
+                                         false);
+}
+template <>
+__device__ __forceinline__ float add_pk16<F16>(uint32_t x, float acc) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, x), __builtin_bit_cast(f16x2_t, 0x3c003c00u), acc, false);
+}
+
 __device__ __forceinline__ float silu_f32(float g) {
   // g * sigmoid(g) = g / (1 + exp(-g)); exp via the hardware exp2
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g));

@@ -10,7 +10,8 @@
 //            waves take interleaved 32-token tiles.  A tile is loaded with
 //            16-byte coalesced loads, written to wave-private LDS and read back
 //            transposed (token-contiguous per channel) as MFMA 32x32x16
-//            operands: S += V^T K and ksum += 1^T K.  Waves are summed in LDS.
+//            operands: S += V^T K; the ones-row (ksum) is a packed dot2 against (1, 1)
+//            on the K operand registers.  Waves are summed in LDS.
 //   phase 2  one wave = (pair of heads, token range); the fp32 state is split
 //            into three bf16 terms (hi + mid + lo = all 24 mantissa bits) and
 //            applied with MFMA 16x16x32; rows 32..47 of the A operand all carry
@@ -19,6 +20,14 @@
 #include <type_traits>
 
 #include "common.h"
+
+// tuning knobs of the bf16 apply kernel: tokens per workgroup, 16-token steps in flight per wave
+#ifndef SANA_LA_APPLY_TOKENS
+#define SANA_LA_APPLY_TOKENS 128
+#endif
+#ifndef SANA_LA_APPLY_U
+#define SANA_LA_APPLY_U 4
+#endif
 
 namespace sana {
 namespace {
@@ -77,17 +86,14 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
   const uint16_t* kbase = K + (int64_t)b * stride_b + ld_ch;
   const uint16_t* vbase = V + (int64_t)b * stride_b + ld_ch;
 
-  f32x16_t accS[2], accK[2];
+  f32x16_t accS[2];
+  float accK[2] = {0.f, 0.f};  // sum over this lane's tokens of relu(K)[tok][j]
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     accS[0][i] = 0.f;
     accS[1][i] = 0.f;
-    accK[0][i] = 0.f;
-    accK[1][i] = 0.f;
   }
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  const uint32_t one2 = std::is_same<T, BF16>::value ? 0x3f803f80u : 0x3c003c00u;
-  const u32x4_t ones = {one2, one2, one2, one2};
 
   u32x4_t kreg[4], vreg[4];
   auto issue_loads = [&](int tile) {
@@ -131,8 +137,9 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
           fk[r2] = klo | (khi << 16);
           fv[r2] = vlo | (vhi << 16);
         }
-        accS[hh] = mfma_32x32x16<T>(fv, fk, accS[hh]);    // S[i][j] += sum_tok V[tok][i] K[tok][j]
-        accK[hh] = mfma_32x32x16<T>(ones, fk, accK[hh]);  // every row: sum_tok K[tok][j]
+        accS[hh] = mfma_32x32x16<T>(fv, fk, accS[hh]);  // S[i][j] += sum_tok V[tok][i] K[tok][j]
+#pragma unroll
+        for (int r2 = 0; r2 < 4; ++r2) accK[hh] = add_pk16<T>(fk[r2], accK[hh]);  // the "1" row of [V|1]
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites
@@ -149,7 +156,8 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
       const int row = 8 * (r >> 2) + 4 * g + (r & 3);
       red[hh * STATE_ELEMS + row * D + j] = accS[hh][r];
     }
-    if (g == 0) red[hh * STATE_ELEMS + D * D + j] = accK[hh][0];
+    const float ks = accK[hh] + __shfl_xor(accK[hh], 32, 64);  // the two token halves of channel j
+    if (g == 0) red[hh * STATE_ELEMS + D * D + j] = ks;
   }
   __syncthreads();
   const float* all = reinterpret_cast<const float*>(smem);
@@ -224,9 +232,16 @@ __global__ __launch_bounds__(256) void linattn_reduce_scan_kernel(const float* _
   const int e = (int)(gid - bh * STATE_ELEMS);
   float run = 0.f;
   for (int c = 0; c < n_chunks; ++c) {
-    const int64_t slot0 = (bh * n_chunks + c) * nsplit;
-    float s = partial[slot0 * STATE_ELEMS + e];
-    for (int sp = 1; sp < nsplit; ++sp) s += partial[(slot0 + sp) * STATE_ELEMS + e];
+    const float* p0 = partial + ((bh * n_chunks + c) * nsplit) * STATE_ELEMS + e;
+    // batches of sixteen independent loads (all in flight together), added in split order
+    float s = 0.f;
+    for (int sp0 = 0; sp0 < nsplit; sp0 += 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = (sp0 + u < nsplit) ? p0[(int64_t)(sp0 + u) * STATE_ELEMS] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) s += v[u];
+    }
     if (causal) {
       run += s;
       s = run;
@@ -300,7 +315,7 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
 
   const uint16_t* qp = Q + (int64_t)b * q_stride_b + p * 64 + 8 * g;
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  constexpr int U = 4;  // 16-token steps in flight
+  constexpr int U = SANA_LA_APPLY_U;  // 16-token steps in flight
   for (int t = t0; t < t1; t += 16 * U) {
     u32x4_t qf[U][2];
 #pragma unroll
@@ -424,8 +439,8 @@ __global__ __launch_bounds__(256) void linattn_apply32_kernel(
 // ---------------------------------------------------------------------------- host side
 
 int pick_nsplit(int items, int max_chunk_tokens, int min_tokens) {
-  // aim for >= 512 workgroups, but keep >= min_tokens tokens per split
-  int ns = (512 + items - 1) / items;
+  // aim for >= 1024 workgroups (four per CU), but keep >= min_tokens tokens per split
+  int ns = (1024 + items - 1) / items;
   const int cap = (max_chunk_tokens + min_tokens - 1) / min_tokens;
   if (ns > cap) ns = cap;
   if (ns < 1) ns = 1;
@@ -550,7 +565,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(con
       (o_stride_n * osz) % 16 || (o_stride_b * osz) % 16)
     return SANA_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int wg_tokens = io_dtype == SANA_DT_BF16 ? 256 : 64;
+  const int wg_tokens = io_dtype == SANA_DT_BF16 ? SANA_LA_APPLY_TOKENS : 64;
   const unsigned gx = (unsigned)((max_chunk_tokens + wg_tokens - 1) / wg_tokens);
   if (io_dtype == SANA_DT_BF16) {
     const int pairs = (h + 1) / 2;
