@@ -491,6 +491,196 @@ __global__ __launch_bounds__(512) void gemm_fast_kernel(const uint16_t* __restri
   }
 }
 
+// ============================================================================
+// bf16 path: 256 threads, one wave per SIMD with the whole register file (256
+// accumulators + 256 VGPRs), each wave a 128x128 sub-tile = 4x4 MFMA tiles, so a
+// fragment read from LDS feeds four MFMAs.  With a single wave per SIMD nothing
+// else hides a stalled memory instruction, so the main loop is one hand-ordered
+// stream (pinned with sched_barrier): a k-tile is 64 MFMA slots and every slot
+// carries at most one LDS or global instruction:
+//   * even slots of k-steps 0-2 read the fragments of the next k-step;
+//   * slot 3q+1 stores staging quad q (k-tile kt+1) into the other LDS stage and
+//     slot 3q+2 reloads the same registers with k-tile kt+2, so every global load
+//     has a whole k-tile (about 1 us) to land and one 64-register set is enough;
+//   * the only barrier sits in k-step 3 after the last store; the slots behind it
+//     read k-step 0 of the next tile.
+// Rows past M / N and k chunks past K are clamped to valid addresses: clamped
+// rows only feed outputs that are never stored, and the last k-tile runs just the
+// k-steps that exist.  Needs K % 16 == 0 and K >= 64.
+// ============================================================================
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Wb,
+                                                    const EpiArgs ep, uint16_t* __restrict__ C, int M, int N, int K,
+                                                    int64_t lda, int64_t ldw, int64_t ldc, int tiles_t, int tiles_c) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int total = tiles_t * tiles_c;
+  int pid = blockIdx.x;
+  {
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    pid = xcd * base + min(xcd, rem) + local;
+  }
+  constexpr int GROUP = 8;
+  const int group_sz = GROUP * tiles_c;
+  const int gid = pid / group_sz;
+  const int first_t = gid * GROUP;
+  const int gt = min(tiles_t - first_t, GROUP);
+  const int tile_t = first_t + (pid % group_sz) % gt;
+  const int tile_c = (pid % group_sz) / gt;
+  const int m0 = tile_t * BT, n0 = tile_c * BC;
+
+  // global -> VGPR -> LDS: thread -> k chunk tid%8, rows tid/8 + 32*q (q < 8), for A and for W
+  const int g_chunk = tid & 7, g_row = tid >> 3;
+  const int a_last = min(BT, M - m0) - 1, w_last = min(BC, N - n0) - 1;  // last valid row of each tile
+  const uint16_t* Abase = A + (int64_t)m0 * lda + 8 * g_chunk;
+  const uint16_t* Wbase = Wb + (int64_t)n0 * ldw + 8 * g_chunk;
+  const uint32_t ulda = (uint32_t)lda, uldw = (uint32_t)ldw;
+  const int a_dst0 = swz(g_row, g_chunk);                            // rows +32*q keep the key: +4096 bytes each
+  const int w_dst0 = TILE_BYTES + swz(wrow_to_lds(g_row), g_chunk);  // the row permutation stays inside 32-row blocks
+  u32x4_t rs[16];  // the k-tile in flight: A quads 0..7, W quads 8..15
+
+  const int wc = wave & 1, wt = wave >> 1;
+  const int fr = lane & 31, fg = lane >> 5;
+  const int x7 = swz_key(fr);
+  const int w_off = TILE_BYTES + (wc * 128 + fr) * ROW_BYTES, a_off = (wt * 128 + fr) * ROW_BYTES;
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  u32x4_t fw[2][4], fa[2][4];
+
+#define SANA_G4_PIN() __builtin_amdgcn_sched_barrier(0)
+  auto gload = [&](int q, int k0) {
+    const uint32_t k = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
+    // row offsets are recomputed (two VALU ops) rather than held in 16 registers
+    if (q < 8) rs[q] = *reinterpret_cast<const u32x4_t*>(Abase + ((uint32_t)min(g_row + 32 * q, a_last) * ulda + k));
+    else rs[q] = *reinterpret_cast<const u32x4_t*>(Wbase + ((uint32_t)min(g_row + 32 * (q - 8), w_last) * uldw + k));
+  };
+  auto lstore = [&](int q, int stage) {
+    unsigned char* base = smem + stage * 2 * TILE_BYTES;
+    if (q < 8) *reinterpret_cast<u32x4_t*>(base + a_dst0 + 4096 * q) = rs[q];
+    else *reinterpret_cast<u32x4_t*>(base + w_dst0 + 4096 * (q - 8)) = rs[q];
+  };
+  auto fread = [&](const unsigned char* st, int buf, int ks, int q) {  // q < 4: W fragment, else A fragment
+    const int col = ((2 * ks + fg) ^ x7) << 4;
+    if (q < 4) fw[buf][q] = *reinterpret_cast<const u32x4_t*>(st + w_off + q * 32 * ROW_BYTES + col);
+    else fa[buf][q - 4] = *reinterpret_cast<const u32x4_t*>(st + a_off + (q - 4) * 32 * ROW_BYTES + col);
+  };
+  auto mfma = [&](int buf, int t) {
+    const int i = t >> 2, j = t & 3;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[buf][i]),
+                                                       __builtin_bit_cast(bf16x8_t, fa[buf][j]), acc[i][j], 0, 0, 0);
+  };
+
+  const int KT = (K + BK - 1) / BK;
+  // prologue: k-tile 0 -> stage 0, k-tile 1 in flight
+#pragma unroll
+  for (int q = 0; q < 16; ++q) gload(q, 0);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) lstore(q, 0);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) gload(q, BK);
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 8; ++q) fread(smem, 0, 0, q);
+
+  for (int kt = 0; kt < KT - 1; ++kt) {
+    const int cur = kt & 1;
+    const unsigned char* st = smem + cur * 2 * TILE_BYTES;
+    const unsigned char* stn = smem + (cur ^ 1) * 2 * TILE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int slot = ks * 16 + t;
+        mfma(ks & 1, t);
+        SANA_G4_PIN();
+        if (ks < 3) {
+          if (t % 2 == 0) fread(st, (ks + 1) & 1, ks + 1, t / 2);
+        } else if (t == 7) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own LDS stores done; no fence: loads stay in flight
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+        } else if (t >= 8) {
+          fread(stn, 0, 0, t - 8);
+        }
+        if (slot % 3 == 1 && slot / 3 < 16) lstore(slot / 3, cur ^ 1);
+        if (slot % 3 == 2 && slot / 3 < 16) gload(slot / 3, (kt + 2) * BK);
+        SANA_G4_PIN();
+      }
+    }
+  }
+#undef SANA_G4_PIN
+  {  // last k-tile: no successor, and K % 64 may leave fewer than four k-steps
+    const unsigned char* st = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
+    const int steps = (K - (KT - 1) * BK) / 16;
+    for (int ks = 0; ks < steps; ++ks) {
+      const int col = ((2 * ks + fg) ^ x7) << 4;
+      u32x4_t w4[4], a4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w4[i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 32 * ROW_BYTES + col);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a4[j] = *reinterpret_cast<const u32x4_t*>(st + a_off + j * 32 * ROW_BYTES + col);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, w4[i]),
+                                                             __builtin_bit_cast(bf16x8_t, a4[j]), acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 32*j + lane%32,
+  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r.  The wave's sub-tile goes through its own 32 KB of
+  // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
+  // row-contiguous: each store instruction then writes four full 256-byte row segments.
+  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
+  __syncthreads();  // every wave is done with the operand tiles
+  unsigned char* stg = smem + wave * 32768;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int nl = 32 * i + 16 * fg;  // channel inside the wave's 128
+    float bv[16];
+    if (HAS_BIAS) {
+      const int n = n0 + wc * 128 + nl;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int tok = 32 * j + fr;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        float a8[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
+        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
+        const int chunk = (nl >> 3) + half;
+        *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+  {
+    const int chunk = lane & 15, rsub = lane >> 4;
+    const int n = n0 + wc * 128 + chunk * 8;
+#pragma unroll 4
+    for (int it = 0; it < 32; ++it) {
+      const int row = it * 4 + rsub;
+      const int m = m0 + wt * 128 + row;
+      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((chunk ^ (row & 15)) << 4));
+      if (m < M && n < N) {
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
+        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
+      }
+    }
+  }
+}
+
 template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
@@ -500,6 +690,21 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
   const bool fast = (K % 16 == 0);  // the generic kernel also takes K % 8 == 0
+  if (!W8 && K % 16 == 0 && K >= 64) {
+    dim3 grid4((unsigned)total), block4(256);
+    const uint16_t* wb = static_cast<const uint16_t*>(W);
+#define SANA_LAUNCH4(EPI) \
+  hipLaunchKernelGGL((gemm4_kernel<EPI>), grid4, block4, 0, s, a, wb, ep, c, M, N, K, lda, ldw, ldc, tiles_t, tiles_c)
+    switch (epilogue) {
+      case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
+      case SANA_EPI_BIAS: SANA_LAUNCH4(SANA_EPI_BIAS); break;
+      case SANA_EPI_BIAS_SILU: SANA_LAUNCH4(SANA_EPI_BIAS_SILU); break;
+      case SANA_EPI_GATE_RES: SANA_LAUNCH4(SANA_EPI_GATE_RES); break;
+      default: return SANA_ERR_ARG;
+    }
+#undef SANA_LAUNCH4
+    return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+  }
   dim3 grid((unsigned)total), block(fast ? 512 : 256);
 #define SANA_LAUNCH(EPI)                                                                                          \
   if (fast)                                                                                                       \
