@@ -64,17 +64,44 @@ template <int EPI>
 __device__ __forceinline__ u32x4_t epi_pack8(const float* a, const float* bv) {
   float v[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    float x = a[r];
-    if (EPI != SANA_EPI_NONE) x += bv[r];
-    if (EPI == SANA_EPI_BIAS_SILU) x = silu_f32(round_bf16(x));  // the reference rounds before the activation
-    v[r] = x;
-  }
+  for (int r = 0; r < 8; ++r) v[r] = EPI != SANA_EPI_NONE ? a[r] + bv[r] : a[r];
   u32x4_t o;
   o.x = pack_bf16(v[0], v[1]);
   o.y = pack_bf16(v[2], v[3]);
   o.z = pack_bf16(v[4], v[5]);
   o.w = pack_bf16(v[6], v[7]);
+  if (EPI == SANA_EPI_BIAS_SILU) {
+    // The reference rounds the linear output to bf16 before the activation.  x * rcp(1 + 2^(-x log2 e)),
+    // written stage by stage over the eight values (and pinned that way): one value at a time is a
+    // chain of dependent instructions with two slow transcendentals, which a lone wave per SIMD
+    // cannot hide.
+    float x[8], t[8];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      x[2 * p] = bf16_lo(o[p]);
+      x[2 * p + 1] = bf16_hi(o[p]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = -1.44269504088896341f * x[r];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = __builtin_amdgcn_exp2f(t[r]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = 1.0f + t[r];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) t[r] = __builtin_amdgcn_rcpf(t[r]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) x[r] *= t[r];
+    __builtin_amdgcn_sched_barrier(0);
+    o.x = pack_bf16(x[0], x[1]);
+    o.y = pack_bf16(x[2], x[3]);
+    o.z = pack_bf16(x[4], x[5]);
+    o.w = pack_bf16(x[6], x[7]);
+  }
   return o;
 }
 __device__ __forceinline__ uint32_t gate_res2(uint32_t y, uint32_t g, uint32_t r) {
@@ -637,45 +664,46 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 32*j + lane%32,
   // channel n0 + wc*128 + 32*i + 16*(lane/32) + r.  The wave's sub-tile goes through its own 32 KB of
   // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
-  // row-contiguous: each store instruction then writes four full 256-byte row segments.
+  // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
+  // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
   __syncthreads();  // every wave is done with the operand tiles
   unsigned char* stg = smem + wave * 32768;
+  float bv[4][16];
+  if (HAS_BIAS) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int nl = 32 * i + 16 * fg;  // channel inside the wave's 128
-    float bv[16];
-    if (HAS_BIAS) {
-      const int n = n0 + wc * 128 + nl;
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + wc * 128 + 32 * i + 16 * fg;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
+      for (int r = 0; r < 16; ++r) bv[i][r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
     }
+  }
+  const int o_chunk = lane & 15, o_rsub = lane >> 4;
+  const int o_n = n0 + wc * 128 + o_chunk * 8;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int tok = 32 * j + fr;
+  for (int j = 0; j < 4; ++j) {
+    const int tok = 32 * j + fr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float a8[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
-        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
-        const int chunk = (nl >> 3) + half;
+        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[i] + 8 * half);
+        const int chunk = 4 * i + 2 * fg + half;
         *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
       }
     }
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
-  {
-    const int chunk = lane & 15, rsub = lane >> 4;
-    const int n = n0 + wc * 128 + chunk * 8;
-#pragma unroll 4
-    for (int it = 0; it < 32; ++it) {
-      const int row = it * 4 + rsub;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int row = 32 * j + it * 4 + o_rsub;
       const int m = m0 + wt * 128 + row;
-      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((chunk ^ (row & 15)) << 4));
-      if (m < M && n < N) {
-        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
-        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
+      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
+      if (m < M && o_n < N) {
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, o_n);
+        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + o_n) = o;
       }
     }
   }
