@@ -294,251 +294,30 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 
 
 // ============================================================================
-// Fast path: 512 threads (8 waves, two per SIMD so one wave's LDS/barrier waits
-// hide behind the other's MFMAs), same 256x256x64 tile, each wave 128 channels x
-// 64 tokens = 4x2 MFMA tiles (128 accumulators).  Global -> LDS goes straight
-// through `global_load_lds_dwordx4` (no VGPR staging, no ds_write): the data of
-// lane l lands at byte 16*l of a 1-KB block = 8 tile rows, so the XOR swizzle is
-// applied to the GLOBAL address each lane fetches.  Rows past M / N are clamped
-// (their results are never stored); a K tail (K % 64 in {16, 32, 48}) runs fewer
-// k-steps on the last tile, so clamped k chunks are never read.  Needs K % 16 == 0.
-// ============================================================================
-#define SANA_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
-#define SANA_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
-
-// One k-tile of MFMAs.  FULL: all four k-steps of 16; otherwise `nsteps` (1..4, wave-uniform).
-template <bool FULL>
-__device__ __forceinline__ void mma_tile(const unsigned char* __restrict__ sa, const unsigned char* __restrict__ sw,
-                                         int a_off, int w_off, int x7, int fg, int nsteps, f32x16_t (&acc)[4][2]) {
-  u32x4_t fw[2][4], fa[2][2];
-  auto read = [&](int buf, int ks) {
-    const int col = ((2 * ks + fg) ^ x7) << 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) fw[buf][i] = *reinterpret_cast<const u32x4_t*>(sw + w_off + i * 32 * ROW_BYTES + col);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) fa[buf][j] = *reinterpret_cast<const u32x4_t*>(sa + a_off + j * 32 * ROW_BYTES + col);
-  };
-  read(0, 0);
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    if (!FULL && ks >= nsteps) break;
-    if (ks + 1 < 4 && (FULL || ks + 1 < nsteps)) read((ks + 1) & 1, ks + 1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[ks & 1][i]),
-                                                           __builtin_bit_cast(bf16x8_t, fa[ks & 1][j]), acc[i][j], 0,
-                                                           0, 0);
-  }
-}
-
-template <bool W8, int EPI>
-__global__ __launch_bounds__(512) void gemm_fast_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
-                                                        const float* __restrict__ scale, const EpiArgs ep,
-                                                        uint16_t* __restrict__ C,
-                                                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
-                                                        int tiles_t, int tiles_c) {
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-
-  const int total = tiles_t * tiles_c;
-  int pid = blockIdx.x;
-  {
-    const int xcd = pid & 7, local = pid >> 3;
-    const int base = total >> 3, rem = total & 7;
-    pid = xcd * base + min(xcd, rem) + local;
-  }
-  constexpr int GROUP = 8;
-  const int group_sz = GROUP * tiles_c;
-  const int gid = pid / group_sz;
-  const int first_t = gid * GROUP;
-  const int gt = min(tiles_t - first_t, GROUP);
-  const int tile_t = first_t + (pid % group_sz) % gt;
-  const int tile_c = (pid % group_sz) / gt;
-  const int m0 = tile_t * BT, n0 = tile_c * BC;
-
-  // ---- direct global -> LDS loads.  Wave w fills 1-KB blocks w, w+8, w+16, w+24 of each tile.
-  const int l_row = lane >> 3;  // row inside the block; logical k chunk whose swizzled home is 16*lane:
-  int l_chunk[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) l_chunk[i] = (lane & 7) ^ swz_key(8 * (wave + 8 * i) + l_row);
-  const uint16_t* a_src[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 8 * (wave + 8 * i) + l_row;
-    a_src[i] = A + (int64_t)min(m0 + row, M - 1) * lda;
-  }
-  const uint16_t* w_src[4];
-  if (!W8) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int lrow = 8 * (wave + 8 * i) + l_row;  // LDS row; holds weight row blk + 16*g + 4*q + s
-      const int r = lrow & 31;
-      const int n = (lrow & ~31) + 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
-      w_src[i] = static_cast<const uint16_t*>(Wv) + (int64_t)min(n0 + n, N - 1) * ldw;
-    }
-  }
-  // W8: 256 rows x 4 chunks of 16 int8 through registers; thread -> chunk tid%4, rows tid/4 + 128*i
-  u32x4_t rw[2];
-  float wscale[2], woff[2];
-  const int8_t* q_src[2];
-  const int q_chunk = tid & 3;
-  if (W8) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int n = min(n0 + (tid >> 2) + 128 * i, N - 1);
-      q_src[i] = static_cast<const int8_t*>(Wv) + (int64_t)n * ldw;
-      wscale[i] = scale[n];
-      woff[i] = -128.f * wscale[i];
-    }
-  }
-  auto issue = [&](int stage, int k0) {
-    unsigned char* sa = smem + stage * 2 * TILE_BYTES;
-    unsigned char* sw = sa + TILE_BYTES;
-    int k[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) k[i] = min(k0 + 8 * l_chunk[i], K - 8);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_global_load_lds(SANA_GPTR(a_src[i] + k[i]), SANA_LPTR(sa + (wave + 8 * i) * 1024), 16, 0, 0);
-    if (!W8) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_global_load_lds(SANA_GPTR(w_src[i] + k[i]), SANA_LPTR(sw + (wave + 8 * i) * 1024), 16, 0,
-                                         0);
-    } else {
-      const int kq = min(k0 + 16 * q_chunk, K - 16);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) rw[i] = *reinterpret_cast<const u32x4_t*>(q_src[i] + kq);
-    }
-  };
-  auto store_w8 = [&](int stage) {
-    unsigned char* sw = smem + stage * 2 * TILE_BYTES + TILE_BYTES;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int lrow = wrow_to_lds((tid >> 2) + 128 * i);
-      u32x4_t q = rw[i];
-      q.x ^= 0x80808080u;
-      q.y ^= 0x80808080u;
-      q.z ^= 0x80808080u;
-      q.w ^= 0x80808080u;
-      u32x4_t lo, hi;
-      lo.x = dequant2(q.x, 0, wscale[i], woff[i]);
-      lo.y = dequant2(q.x, 1, wscale[i], woff[i]);
-      lo.z = dequant2(q.y, 0, wscale[i], woff[i]);
-      lo.w = dequant2(q.y, 1, wscale[i], woff[i]);
-      hi.x = dequant2(q.z, 0, wscale[i], woff[i]);
-      hi.y = dequant2(q.z, 1, wscale[i], woff[i]);
-      hi.z = dequant2(q.w, 0, wscale[i], woff[i]);
-      hi.w = dequant2(q.w, 1, wscale[i], woff[i]);
-      *reinterpret_cast<u32x4_t*>(sw + swz(lrow, 2 * q_chunk)) = lo;
-      *reinterpret_cast<u32x4_t*>(sw + swz(lrow, 2 * q_chunk + 1)) = hi;
-    }
-  };
-
-  // ---- MFMA tiling: wave (wc, wt): channels [wc*128, +128) x tokens [wt*64, +64)
-  const int wc = wave & 1, wt = wave >> 1;
-  const int fr = lane & 31, fg = lane >> 5;
-  const int x7 = swz_key(fr);  // tile-row bases are multiples of 32
-  const int w_off = (wc * 128 + fr) * ROW_BYTES, a_off = (wt * 64 + fr) * ROW_BYTES;
-  f32x16_t acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  const int KT = (K + BK - 1) / BK;
-  const int tail_steps = (K - (KT - 1) * BK) / 16;  // 1..4 k-steps of 16 on the last tile
-  issue(0, 0);
-  if (W8) store_w8(0);
-  __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): direct-to-LDS data has landed
-  __syncthreads();
-  for (int kt = 0; kt + 1 < KT; ++kt) {
-    const int cur = kt & 1;
-    issue(cur ^ 1, (kt + 1) * BK);
-    const unsigned char* sa = smem + cur * 2 * TILE_BYTES;
-    mma_tile<true>(sa, sa + TILE_BYTES, a_off, w_off, x7, fg, 4, acc);
-    if (W8) store_w8(cur ^ 1);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-  }
-  {
-    const unsigned char* sa = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
-    mma_tile<false>(sa, sa + TILE_BYTES, a_off, w_off, x7, fg, tail_steps, acc);
-  }
-
-  // ---- epilogue.  acc[i][j][r]: token m0 + wt*64 + 32*j + lane%32,
-  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r.  In that layout a lane owns 32-byte pieces of 32
-  // different rows; the sub-tile goes through wave-private LDS ([64 tokens][256 bytes], 16-byte chunks
-  // XOR-swizzled by token % 16) and comes back row-contiguous, so each store instruction writes four
-  // full 256-byte row segments and the residual / gate reads of the fused update are coalesced too.
-  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
-  __syncthreads();  // every wave is done with the operand tiles
-  unsigned char* stg = smem + wave * 16384;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int nl = 32 * i + 16 * fg;  // channel inside the wave's 128
-    float bv[16];
-    if (HAS_BIAS) {
-      const int n = n0 + wc * 128 + nl;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int tok = 32 * j + fr;
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        float a8[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
-        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
-        const int chunk = (nl >> 3) + half;
-        *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
-      }
-    }
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
-  {
-    const int chunk = lane & 15, rsub = lane >> 4;
-    const int n = n0 + wc * 128 + chunk * 8;
-#pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
-      const int row = it * 4 + rsub;
-      const int m = m0 + wt * 64 + row;
-      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((chunk ^ (row & 15)) << 4));
-      if (m < M && n < N) {
-        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
-        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
-      }
-    }
-  }
-}
-
-// ============================================================================
-// bf16 path: 256 threads, one wave per SIMD with the whole register file (256
-// accumulators + 256 VGPRs), each wave a 128x128 sub-tile = 4x4 MFMA tiles, so a
-// fragment read from LDS feeds four MFMAs.  With a single wave per SIMD nothing
+// Pipelined kernel (K % 16 == 0, K >= 64; bf16 and int8 weights): 256 threads, one
+// wave per SIMD with the whole register file (256 accumulators + 256 VGPRs), each
+// wave a 128x128 sub-tile = 4x4 MFMA tiles, so a fragment read from LDS feeds four
+// MFMAs.  With a single wave per SIMD nothing
 // else hides a stalled memory instruction, so the main loop is one hand-ordered
 // stream (pinned with sched_barrier): a k-tile is 64 MFMA slots and every slot
 // carries at most one LDS or global instruction:
 //   * even slots of k-steps 0-2 read the fragments of the next k-step;
 //   * slot 3q+1 stores staging quad q (k-tile kt+1) into the other LDS stage and
 //     slot 3q+2 reloads the same registers with k-tile kt+2, so every global load
-//     has a whole k-tile (about 1 us) to land and one 64-register set is enough;
+//     has a whole k-tile (about 1 us) to land and one 64-register set is enough
+//     (int8 weights: 16 values per quad, converted two at a time in the MFMA slots
+//     before they are stored, the quad reloaded after its last piece);
 //   * the only barrier sits in k-step 3 after the last store; the slots behind it
 //     read k-step 0 of the next tile.
 // Rows past M / N and k chunks past K are clamped to valid addresses: clamped
 // rows only feed outputs that are never stored, and the last k-tile runs just the
 // k-steps that exist.  Needs K % 16 == 0 and K >= 64.
 // ============================================================================
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Wb,
-                                                    const EpiArgs ep, uint16_t* __restrict__ C, int M, int N, int K,
-                                                    int64_t lda, int64_t ldw, int64_t ldc, int tiles_t, int tiles_c) {
+template <bool W8, int EPI>
+__global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
+                                                    const float* __restrict__ scale, const EpiArgs ep,
+                                                    uint16_t* __restrict__ C, int M, int N, int K, int64_t lda,
+                                                    int64_t ldw, int64_t ldc, int tiles_t, int tiles_c) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int total = tiles_t * tiles_c;
@@ -557,15 +336,30 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int tile_c = (pid % group_sz) / gt;
   const int m0 = tile_t * BT, n0 = tile_c * BC;
 
-  // global -> VGPR -> LDS: thread -> k chunk tid%8, rows tid/8 + 32*q (q < 8), for A and for W
+  // global -> VGPR -> LDS: thread -> k chunk tid%8, rows tid/8 + 32*q (q < 8), for A and for bf16 W.
+  // int8 W: thread -> 16-value chunk tid%4, rows tid/4 + 64*q (q < 4); dequantised on the way to LDS.
   const int g_chunk = tid & 7, g_row = tid >> 3;
   const int a_last = min(BT, M - m0) - 1, w_last = min(BC, N - n0) - 1;  // last valid row of each tile
   const uint16_t* Abase = A + (int64_t)m0 * lda + 8 * g_chunk;
-  const uint16_t* Wbase = Wb + (int64_t)n0 * ldw + 8 * g_chunk;
+  const uint16_t* Wbase = static_cast<const uint16_t*>(Wv) + (int64_t)n0 * ldw + 8 * g_chunk;
   const uint32_t ulda = (uint32_t)lda, uldw = (uint32_t)ldw;
   const int a_dst0 = swz(g_row, g_chunk);                            // rows +32*q keep the key: +4096 bytes each
   const int w_dst0 = TILE_BYTES + swz(wrow_to_lds(g_row), g_chunk);  // the row permutation stays inside 32-row blocks
-  u32x4_t rs[16];  // the k-tile in flight: A quads 0..7, W quads 8..15
+  constexpr int NQ = W8 ? 12 : 16;
+  u32x4_t rs[NQ];  // the k-tile in flight: A quads 0..7, then W quads (8 of bf16 or 4 of int8)
+  const int q_chunk = tid & 3, q_row = tid >> 2;
+  const int8_t* Qbase = static_cast<const int8_t*>(Wv) + (int64_t)n0 * ldw + 16 * q_chunk;
+  const int q_dst_lo = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk);  // rows +64*q: +8192 bytes, same key
+  const int q_dst_hi = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk + 1);
+  float wscale[4], woff[4];
+  if (W8) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      wscale[q] = scale[n0 + min(q_row + 64 * q, w_last)];
+      woff[q] = -128.f * wscale[q];
+    }
+  }
+  u32x4_t dq[2];  // dequantised halves of the int8 quad being converted
 
   const int wc = wave & 1, wt = wave >> 1;
   const int fr = lane & 31, fg = lane >> 5;
@@ -582,15 +376,31 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 
 #define SANA_G4_PIN() __builtin_amdgcn_sched_barrier(0)
   auto gload = [&](int q, int k0) {
-    const uint32_t k = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
-    // row offsets are recomputed (two VALU ops) rather than held in 16 registers
-    if (q < 8) rs[q] = *reinterpret_cast<const u32x4_t*>(Abase + ((uint32_t)min(g_row + 32 * q, a_last) * ulda + k));
-    else rs[q] = *reinterpret_cast<const u32x4_t*>(Wbase + ((uint32_t)min(g_row + 32 * (q - 8), w_last) * uldw + k));
+    // row offsets are recomputed (two VALU ops) rather than held in registers
+    if (q < 8) {
+      const uint32_t kk = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
+      rs[q] = *reinterpret_cast<const u32x4_t*>(Abase + ((uint32_t)min(g_row + 32 * q, a_last) * ulda + kk));
+    } else if (!W8) {
+      const uint32_t kk = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
+      rs[q] = *reinterpret_cast<const u32x4_t*>(Wbase + ((uint32_t)min(g_row + 32 * (q - 8), w_last) * uldw + kk));
+    } else {
+      const uint32_t kk = (uint32_t)min(k0, K - 16 - 16 * q_chunk);
+      rs[q] = *reinterpret_cast<const u32x4_t*>(Qbase + ((uint32_t)min(q_row + 64 * (q - 8), w_last) * uldw + kk));
+    }
   };
-  auto lstore = [&](int q, int stage) {
+  auto lstore = [&](int q, int stage) {  // A quads, bf16 W quads
     unsigned char* base = smem + stage * 2 * TILE_BYTES;
     if (q < 8) *reinterpret_cast<u32x4_t*>(base + a_dst0 + 4096 * q) = rs[q];
     else *reinterpret_cast<u32x4_t*>(base + w_dst0 + 4096 * (q - 8)) = rs[q];
+  };
+  // int8 quad wq (16 values), piece 0..7 = two values each: convert, and store a 16-byte half when complete
+  auto dequant_piece = [&](int wq, int piece, int stage) {
+    uint32_t word = rs[8 + wq][piece >> 1] ^ 0x80808080u;
+    dq[piece >> 2][piece & 3] = dequant2(word, piece & 1, wscale[wq], woff[wq]);
+    if ((piece & 3) == 3) {
+      unsigned char* base = smem + stage * 2 * TILE_BYTES + 8192 * wq;
+      *reinterpret_cast<u32x4_t*>(base + (piece < 4 ? q_dst_lo : q_dst_hi)) = dq[piece >> 2];
+    }
   };
   auto fread = [&](const unsigned char* st, int buf, int ks, int q) {  // q < 4: W fragment, else A fragment
     const int col = ((2 * ks + fg) ^ x7) << 4;
@@ -606,11 +416,15 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int KT = (K + BK - 1) / BK;
   // prologue: k-tile 0 -> stage 0, k-tile 1 in flight
 #pragma unroll
-  for (int q = 0; q < 16; ++q) gload(q, 0);
+  for (int q = 0; q < NQ; ++q) gload(q, 0);
 #pragma unroll
-  for (int q = 0; q < 16; ++q) lstore(q, 0);
+  for (int q = 0; q < (W8 ? 8 : 16); ++q) lstore(q, 0);
+  if (W8) {
 #pragma unroll
-  for (int q = 0; q < 16; ++q) gload(q, BK);
+    for (int n = 0; n < 32; ++n) dequant_piece(n >> 3, n & 7, 0);
+  }
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) gload(q, BK);
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < 8; ++q) fread(smem, 0, 0, q);
@@ -635,8 +449,17 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
         } else if (t >= 8) {
           fread(stn, 0, 0, t - 8);
         }
-        if (slot % 3 == 1 && slot / 3 < 16) lstore(slot / 3, cur ^ 1);
-        if (slot % 3 == 2 && slot / 3 < 16) gload(slot / 3, (kt + 2) * BK);
+        if (!W8) {
+          if (slot % 3 == 1 && slot / 3 < 16) lstore(slot / 3, cur ^ 1);
+          if (slot % 3 == 2 && slot / 3 < 16) gload(slot / 3, (kt + 2) * BK);
+        } else {
+          // A quad q: store at slot 4q, reload at 4q+1.  int8 piece n at slot n+2 (its half is stored
+          // with pieces 3 and 7), the quad is reloaded right after its last piece.
+          if (slot % 4 == 0 && slot / 4 < 8) lstore(slot / 4, cur ^ 1);
+          if (slot % 4 == 1 && slot / 4 < 8) gload(slot / 4, (kt + 2) * BK);
+          if (slot >= 2 && slot < 34) dequant_piece((slot - 2) >> 3, (slot - 2) & 7, cur ^ 1);
+          if (slot >= 10 && slot <= 34 && (slot - 10) % 8 == 0) gload(8 + (slot - 10) / 8, (kt + 2) * BK);
+        }
         SANA_G4_PIN();
       }
     }
@@ -717,12 +540,11 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
   if (total > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
-  const bool fast = (K % 16 == 0);  // the generic kernel also takes K % 8 == 0
-  if (!W8 && K % 16 == 0 && K >= 64) {
+  if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
     dim3 grid4((unsigned)total), block4(256);
-    const uint16_t* wb = static_cast<const uint16_t*>(W);
-#define SANA_LAUNCH4(EPI) \
-  hipLaunchKernelGGL((gemm4_kernel<EPI>), grid4, block4, 0, s, a, wb, ep, c, M, N, K, lda, ldw, ldc, tiles_t, tiles_c)
+#define SANA_LAUNCH4(EPI)                                                                                       \
+  hipLaunchKernelGGL((gemm4_kernel<W8, EPI>), grid4, block4, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+                     tiles_t, tiles_c)
     switch (epilogue) {
       case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
       case SANA_EPI_BIAS: SANA_LAUNCH4(SANA_EPI_BIAS); break;
@@ -733,14 +555,9 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
 #undef SANA_LAUNCH4
     return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
   }
-  dim3 grid((unsigned)total), block(fast ? 512 : 256);
-#define SANA_LAUNCH(EPI)                                                                                          \
-  if (fast)                                                                                                       \
-    hipLaunchKernelGGL((gemm_fast_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
-                       tiles_t, tiles_c);                                                                         \
-  else                                                                                                            \
-    hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc,      \
-                       tiles_t, tiles_c)
+  dim3 grid((unsigned)total), block(256);
+#define SANA_LAUNCH(EPI) \
+  hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, tiles_t, tiles_c)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH(SANA_EPI_NONE); break;
     case SANA_EPI_BIAS: SANA_LAUNCH(SANA_EPI_BIAS); break;

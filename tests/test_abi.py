@@ -56,8 +56,9 @@ def test_workspace_query():
     # 1.6B @ 16384 tokens: 70 heads -> splits of the token axis need partial states
     n = lib.sana_hip_linattn_workspace_bytes(1, 70, 32, 1, 16384, 1)
     assert n > 0 and n % (33 * 32 * 4) == 0
-    # many (batch, head) pairs at 1024 tokens: no split, no workspace
-    assert lib.sana_hip_linattn_workspace_bytes(16, 70, 32, 1, 1024, 1) == 0
+    # short sequences are never split (a split is at least 256 tokens): no workspace
+    assert lib.sana_hip_linattn_workspace_bytes(16, 70, 32, 1, 256, 1) == 0
+    assert lib.sana_hip_linattn_workspace_bytes(64, 70, 32, 4, 300, 1) == 0
 
 
 def test_ops_refuse_cpu_tensors():

@@ -89,8 +89,12 @@ GEMM_SHAPES = [
     (16384, 2240, 2240),  # proj, cfg3
     (16384, 2240, 5600),  # point conv, cfg3 (K not a multiple of 64)
     (300, 72, 96),        # ragged everything
-    (1, 8, 32),
+    (1, 8, 32),           # K < 64: the generic kernel
     (257, 264, 160),
+    (513, 40, 64),        # a single k-tile
+    (31, 24, 80),         # two k-tiles, the second with one k-step; fewer than 32 rows either side
+    (260, 520, 136),      # K % 16 != 0: the generic kernel
+    (129, 1000, 208),     # k tail of one k-step after three full tiles
 ]
 
 
@@ -140,7 +144,8 @@ def test_gemm_exact_on_integer_inputs(cuda):
     assert torch.equal(y.float(), a.float() @ w.float().T)
 
 
-@pytest.mark.parametrize("M,N,K", [(1024, 2240, 2240), (4096, 11200, 2240), (300, 72, 96), (16384, 2240, 5600)])
+@pytest.mark.parametrize("M,N,K", [(1024, 2240, 2240), (4096, 11200, 2240), (300, 72, 96), (16384, 2240, 5600),
+                                   (40, 24, 64), (513, 264, 208), (9, 8, 48)])
 @pytest.mark.parametrize("epilogue", [None, "bias_silu"])
 def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilogue):
     g = torch.Generator().manual_seed(M + K)
