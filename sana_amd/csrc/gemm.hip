@@ -296,11 +296,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 // ============================================================================
 // Pipelined kernel (K % 16 == 0, K >= 64; bf16 and int8 weights): 256 threads, one
 // wave per SIMD with the whole register file (256 accumulators + 256 VGPRs), each
-// wave a 128x128 sub-tile = 4x4 MFMA tiles, so a fragment read from LDS feeds four
-// MFMAs.  With a single wave per SIMD nothing
+// wave a sub-tile of 128 tokens x 32*NI channels = NI x 4 MFMA tiles (NI = 4: 128x128,
+// every fragment read from LDS feeds four MFMAs; NI = 3 or 2 narrows the workgroup's
+// channel tile to 192 or 128 where that fills the last round of workgroups better).  With a single wave per SIMD nothing
 // else hides a stalled memory instruction, so the main loop is one hand-ordered
-// stream (pinned with sched_barrier): a k-tile is 64 MFMA slots and every slot
-// carries at most one LDS or global instruction:
+// stream (pinned with sched_barrier): a k-tile is 16*NI MFMA slots and a slot carries
+// one or two LDS / global instructions (NI = 4, bf16):
 //   * even slots of k-steps 0-2 read the fragments of the next k-step;
 //   * slot 3q+1 stores staging quad q (k-tile kt+1) into the other LDS stage and
 //     slot 3q+2 reloads the same registers with k-tile kt+2, so every global load
@@ -313,7 +314,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 // rows only feed outputs that are never stored, and the last k-tile runs just the
 // k-steps that exist.  Needs K % 16 == 0 and K >= 64.
 // ============================================================================
-template <bool W8, int EPI>
+template <bool W8, int EPI, int NI>
 __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
                                                     const float* __restrict__ scale, const EpiArgs ep,
                                                     uint16_t* __restrict__ C, int M, int N, int K, int64_t lda,
@@ -334,27 +335,29 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int gt = min(tiles_t - first_t, GROUP);
   const int tile_t = first_t + (pid % group_sz) % gt;
   const int tile_c = (pid % group_sz) / gt;
-  const int m0 = tile_t * BT, n0 = tile_c * BC;
+  constexpr int BCN = 64 * NI;  // channels per workgroup: two waves x NI MFMA tiles of 32
+  const int m0 = tile_t * BT, n0 = tile_c * BCN;
 
-  // global -> VGPR -> LDS: thread -> k chunk tid%8, rows tid/8 + 32*q (q < 8), for A and for bf16 W.
-  // int8 W: thread -> 16-value chunk tid%4, rows tid/4 + 64*q (q < 4); dequantised on the way to LDS.
+  // global -> VGPR -> LDS: thread -> k chunk tid%8, rows tid/8 + 32*q, q < 8 for A and q < 2*NI for bf16 W.
+  // int8 W: thread -> 16-value chunk tid%4, rows tid/4 + 64*q (q < NI); dequantised on the way to LDS.
   const int g_chunk = tid & 7, g_row = tid >> 3;
-  const int a_last = min(BT, M - m0) - 1, w_last = min(BC, N - n0) - 1;  // last valid row of each tile
+  const int a_last = min(BT, M - m0) - 1, w_last = min(BCN, N - n0) - 1;  // last valid row of each tile
   const uint16_t* Abase = A + (int64_t)m0 * lda + 8 * g_chunk;
   const uint16_t* Wbase = static_cast<const uint16_t*>(Wv) + (int64_t)n0 * ldw + 8 * g_chunk;
   const uint32_t ulda = (uint32_t)lda, uldw = (uint32_t)ldw;
   const int a_dst0 = swz(g_row, g_chunk);                            // rows +32*q keep the key: +4096 bytes each
   const int w_dst0 = TILE_BYTES + swz(wrow_to_lds(g_row), g_chunk);  // the row permutation stays inside 32-row blocks
-  constexpr int NQ = W8 ? 12 : 16;
-  u32x4_t rs[NQ];  // the k-tile in flight: A quads 0..7, then W quads (8 of bf16 or 4 of int8)
+  constexpr int NWQ = W8 ? NI : 2 * NI;  // W quads per thread
+  constexpr int NQ = 8 + NWQ;
+  u32x4_t rs[NQ];  // the k-tile in flight: A quads 0..7, then the W quads
   const int q_chunk = tid & 3, q_row = tid >> 2;
   const int8_t* Qbase = static_cast<const int8_t*>(Wv) + (int64_t)n0 * ldw + 16 * q_chunk;
   const int q_dst_lo = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk);  // rows +64*q: +8192 bytes, same key
   const int q_dst_hi = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk + 1);
-  float wscale[4], woff[4];
+  float wscale[NI], woff[NI];
   if (W8) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < NI; ++q) {
       wscale[q] = scale[n0 + min(q_row + 64 * q, w_last)];
       woff[q] = -128.f * wscale[q];
     }
@@ -364,15 +367,15 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int wc = wave & 1, wt = wave >> 1;
   const int fr = lane & 31, fg = lane >> 5;
   const int x7 = swz_key(fr);
-  const int w_off = TILE_BYTES + (wc * 128 + fr) * ROW_BYTES, a_off = (wt * 128 + fr) * ROW_BYTES;
-  f32x16_t acc[4][4];
+  const int w_off = TILE_BYTES + (wc * 32 * NI + fr) * ROW_BYTES, a_off = (wt * 128 + fr) * ROW_BYTES;
+  f32x16_t acc[NI][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  u32x4_t fw[2][4], fa[2][4];
+  u32x4_t fw[2][NI], fa[2][4];
 
 #define SANA_G4_PIN() __builtin_amdgcn_sched_barrier(0)
   auto gload = [&](int q, int k0) {
@@ -402,12 +405,13 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       *reinterpret_cast<u32x4_t*>(base + (piece < 4 ? q_dst_lo : q_dst_hi)) = dq[piece >> 2];
     }
   };
-  auto fread = [&](const unsigned char* st, int buf, int ks, int q) {  // q < 4: W fragment, else A fragment
+  constexpr int NFR = NI + 4;  // fragment reads per k-step
+  auto fread = [&](const unsigned char* st, int buf, int ks, int q) {  // q < NI: W fragment, else A fragment
     const int col = ((2 * ks + fg) ^ x7) << 4;
-    if (q < 4) fw[buf][q] = *reinterpret_cast<const u32x4_t*>(st + w_off + q * 32 * ROW_BYTES + col);
-    else fa[buf][q - 4] = *reinterpret_cast<const u32x4_t*>(st + a_off + (q - 4) * 32 * ROW_BYTES + col);
+    if (q < NI) fw[buf][q] = *reinterpret_cast<const u32x4_t*>(st + w_off + q * 32 * ROW_BYTES + col);
+    else fa[buf][q - NI] = *reinterpret_cast<const u32x4_t*>(st + a_off + (q - NI) * 32 * ROW_BYTES + col);
   };
-  auto mfma = [&](int buf, int t) {
+  auto mfma = [&](int buf, int t) {  // t < 4 * NI
     const int i = t >> 2, j = t & 3;
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[buf][i]),
                                                        __builtin_bit_cast(bf16x8_t, fa[buf][j]), acc[i][j], 0, 0, 0);
@@ -418,17 +422,22 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
   for (int q = 0; q < NQ; ++q) gload(q, 0);
 #pragma unroll
-  for (int q = 0; q < (W8 ? 8 : 16); ++q) lstore(q, 0);
+  for (int q = 0; q < (W8 ? 8 : NQ); ++q) lstore(q, 0);
   if (W8) {
 #pragma unroll
-    for (int n = 0; n < 32; ++n) dequant_piece(n >> 3, n & 7, 0);
+    for (int n = 0; n < 8 * NI; ++n) dequant_piece(n >> 3, n & 7, 0);
   }
 #pragma unroll
   for (int q = 0; q < NQ; ++q) gload(q, BK);
   __syncthreads();
 #pragma unroll
-  for (int q = 0; q < 8; ++q) fread(smem, 0, 0, q);
+  for (int q = 0; q < NFR; ++q) fread(smem, 0, 0, q);
 
+  // slots per k-step, the barrier slot (the NFR slots behind it read the next tile's k-step 0), and
+  // the spacing of the staging quads in front of it
+  constexpr int SL = 4 * NI, BAR = 4 * SL - NFR - 1;
+  constexpr int QSTRIDE = (BAR - 2) / NQ;  // bf16: store quad q at slot 1 + q*QSTRIDE, reload it one slot later
+  static_assert(QSTRIDE >= 2 && 4 * 7 + 1 < BAR && 8 * NI + 2 < BAR, "staging does not fit in front of the barrier");
   for (int kt = 0; kt < KT - 1; ++kt) {
     const int cur = kt & 1;
     const unsigned char* st = smem + cur * 2 * TILE_BYTES;
@@ -436,29 +445,33 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const int slot = ks * 16 + t;
+      for (int t = 0; t < SL; ++t) {
+        const int slot = ks * SL + t;
         mfma(ks & 1, t);
         SANA_G4_PIN();
         if (ks < 3) {
-          if (t % 2 == 0) fread(st, (ks + 1) & 1, ks + 1, t / 2);
-        } else if (t == 7) {
+          // read r of the next k-step goes to slot (r * SL) / NFR of this one
+          if (((t * NFR + SL - 1) / SL) * SL / NFR == t && (t * NFR + SL - 1) / SL < NFR)
+            fread(st, (ks + 1) & 1, ks + 1, (t * NFR + SL - 1) / SL);
+        }
+        if (slot == BAR) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own LDS stores done; no fence: loads stay in flight
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
-        } else if (t >= 8) {
-          fread(stn, 0, 0, t - 8);
+        } else if (slot > BAR) {
+          fread(stn, 0, 0, slot - BAR - 1);
         }
         if (!W8) {
-          if (slot % 3 == 1 && slot / 3 < 16) lstore(slot / 3, cur ^ 1);
-          if (slot % 3 == 2 && slot / 3 < 16) gload(slot / 3, (kt + 2) * BK);
+          if (slot >= 1 && (slot - 1) % QSTRIDE == 0 && (slot - 1) / QSTRIDE < NQ) lstore((slot - 1) / QSTRIDE, cur ^ 1);
+          if (slot >= 2 && (slot - 2) % QSTRIDE == 0 && (slot - 2) / QSTRIDE < NQ)
+            gload((slot - 2) / QSTRIDE, (kt + 2) * BK);
         } else {
           // A quad q: store at slot 4q, reload at 4q+1.  int8 piece n at slot n+2 (its half is stored
           // with pieces 3 and 7), the quad is reloaded right after its last piece.
           if (slot % 4 == 0 && slot / 4 < 8) lstore(slot / 4, cur ^ 1);
           if (slot % 4 == 1 && slot / 4 < 8) gload(slot / 4, (kt + 2) * BK);
-          if (slot >= 2 && slot < 34) dequant_piece((slot - 2) >> 3, (slot - 2) & 7, cur ^ 1);
-          if (slot >= 10 && slot <= 34 && (slot - 10) % 8 == 0) gload(8 + (slot - 10) / 8, (kt + 2) * BK);
+          if (slot >= 2 && slot < 2 + 8 * NI) dequant_piece((slot - 2) >> 3, (slot - 2) & 7, cur ^ 1);
+          if (slot >= 10 && slot <= 2 + 8 * NI && (slot - 10) % 8 == 0) gload(8 + (slot - 10) / 8, (kt + 2) * BK);
         }
         SANA_G4_PIN();
       }
@@ -470,13 +483,13 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     const int steps = (K - (KT - 1) * BK) / 16;
     for (int ks = 0; ks < steps; ++ks) {
       const int col = ((2 * ks + fg) ^ x7) << 4;
-      u32x4_t w4[4], a4[4];
+      u32x4_t w4[NI], a4[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w4[i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 32 * ROW_BYTES + col);
+      for (int i = 0; i < NI; ++i) w4[i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 32 * ROW_BYTES + col);
 #pragma unroll
       for (int j = 0; j < 4; ++j) a4[j] = *reinterpret_cast<const u32x4_t*>(st + a_off + j * 32 * ROW_BYTES + col);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, w4[i]),
@@ -492,22 +505,23 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
   __syncthreads();  // every wave is done with the operand tiles
   unsigned char* stg = smem + wave * 32768;
-  float bv[4][16];
+  float bv[NI][16];
   if (HAS_BIAS) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + wc * 128 + 32 * i + 16 * fg;
+    for (int i = 0; i < NI; ++i) {
+      const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg;
 #pragma unroll
       for (int r = 0; r < 16; ++r) bv[i][r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
     }
   }
   const int o_chunk = lane & 15, o_rsub = lane >> 4;
-  const int o_n = n0 + wc * 128 + o_chunk * 8;
+  const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
+  const bool o_live = o_chunk < 4 * NI;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int tok = 32 * j + fr;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float a8[8];
@@ -524,7 +538,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       const int row = 32 * j + it * 4 + o_rsub;
       const int m = m0 + wt * 128 + row;
       u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-      if (m < M && o_n < N) {
+      if (o_live && m < M && o_n < N) {
         if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, o_n);
         *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + o_n) = o;
       }
@@ -532,32 +546,59 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   }
 }
 
+int compute_units() {
+  static int n = 0;  // same value from every thread that races here
+  if (n == 0) {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
+      cu = 256;
+    n = cu;
+  }
+  return n;
+}
+
+template <bool W8, int NI>
+int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N, int K,
+            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
+  const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + 64 * NI - 1) / (64 * NI);
+  dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
+#define SANA_LAUNCH4(EPI)                                                                                         \
+  hipLaunchKernelGGL((gemm4_kernel<W8, EPI, NI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+                     tiles_t, tiles_c)
+  switch (epilogue) {
+    case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
+    case SANA_EPI_BIAS: SANA_LAUNCH4(SANA_EPI_BIAS); break;
+    case SANA_EPI_BIAS_SILU: SANA_LAUNCH4(SANA_EPI_BIAS_SILU); break;
+    case SANA_EPI_GATE_RES: SANA_LAUNCH4(SANA_EPI_GATE_RES); break;
+    default: return SANA_ERR_ARG;
+  }
+#undef SANA_LAUNCH4
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
 template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
-  const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + BC - 1) / BC;
-  const int64_t total = (int64_t)tiles_t * tiles_c;
-  if (total > (1 << 30)) return SANA_ERR_SHAPE;
+  const int64_t tiles_t = (M + BT - 1) / BT;
+  if (tiles_t * ((N + 127) / 128) > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
   if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
-    dim3 grid4((unsigned)total), block4(256);
-#define SANA_LAUNCH4(EPI)                                                                                       \
-  hipLaunchKernelGGL((gemm4_kernel<W8, EPI>), grid4, block4, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
-                     tiles_t, tiles_c)
-    switch (epilogue) {
-      case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
-      case SANA_EPI_BIAS: SANA_LAUNCH4(SANA_EPI_BIAS); break;
-      case SANA_EPI_BIAS_SILU: SANA_LAUNCH4(SANA_EPI_BIAS_SILU); break;
-      case SANA_EPI_GATE_RES: SANA_LAUNCH4(SANA_EPI_GATE_RES); break;
-      default: return SANA_ERR_ARG;
-    }
-#undef SANA_LAUNCH4
-    return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+    // One workgroup per compute unit at a time, so the grid runs in rounds: pick the channel tile
+    // (256 or 192) whose rounds x tile size is smaller; the narrower tile re-reads a little more
+    // per MFMA, hence its 4 % handicap.
+    const int64_t cu = compute_units();
+    const int64_t t256 = tiles_t * ((N + 255) / 256), t192 = tiles_t * ((N + 191) / 192);
+    const double cost256 = (double)((t256 + cu - 1) / cu) * 4.0, cost192 = (double)((t192 + cu - 1) / cu) * 3.0 * 1.04;
+    return cost192 < cost256 ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s)
+                             : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
   }
-  dim3 grid((unsigned)total), block(256);
-#define SANA_LAUNCH(EPI) \
-  hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, tiles_t, tiles_c)
+  const int tiles_c = (N + BC - 1) / BC;
+  dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
+#define SANA_LAUNCH(EPI)                                                                                        \
+  hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+                     (int)tiles_t, tiles_c)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH(SANA_EPI_NONE); break;
     case SANA_EPI_BIAS: SANA_LAUNCH(SANA_EPI_BIAS); break;
