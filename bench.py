@@ -13,12 +13,18 @@ launch stream:
   roofline       the dominant kernel (the inverted-conv GEMM) against the
                  MI355X dense bf16 MFMA peak,
   kernels        every hand-written kernel of the block against its roofline
-                 (HBM 8 TB/s for the attention pair and the depthwise kernel,
-                 2.5 PFLOP/s for the four GEMMs),
+                 (HBM 8 TB/s for the attention pair, the depthwise kernel and
+                 the LayerNorm+modulate kernel, 2.5 PFLOP/s for the GEMMs),
   images_per_s   B / (20 x block latency) at the 1024px shape (B=16, N=1024),
                  bf16 and W8A16: DiT blocks of ONE denoising step only,
   cpu_baseline   the oracle block (stock PyTorch, fp32) on the host cores, one
                  block of the same workload.
+
+``--kernels-only`` runs just the per-kernel section (the command the rocprofv3
+summaries under profiles/ were taken with).  ``roofline.traffic`` is not
+measurable from inside the process: it is the HBM byte count of one launch of
+the dominant kernel from two ``rocprofv3 --pmc`` runs of that command
+(FETCH_SIZE, WRITE_SIZE), copied here from profiles/kernels_cfg3_hbm_traffic.txt.
 """
 from __future__ import annotations
 
@@ -33,6 +39,10 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+
+# HBM bytes per launch of the dominant kernel (inverted-conv GEMM at cfg3), from the pmc summary
+# profiles/kernels_cfg3_hbm_traffic.txt: FETCH_SIZE x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE x 1.0.
+DOMINANT_KERNEL_TRAFFIC_BYTES = None
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -72,18 +82,31 @@ def make_inputs(B: int, N: int, seed: int = 1000):
     return x, y, t
 
 
-def event_time_us(fn, iters: int, warmup: int) -> float:
-    """Average duration of one call, HIP events on the stream the kernels are launched on."""
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
+def event_time_us(fn, iters: int, warmup: int, repeats: int = 3) -> float:
+    """Average duration of one call, HIP events on the stream the kernels are launched on.  The chip
+    idles (and drops its clocks) while the host prepares the next operand set, so the warm-up runs
+    for at least 0.1 s of GPU time, and the figure is the median of ``repeats`` timed regions of
+    ``iters`` back-to-back calls each."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters
+    done, spent_ms = 0, 0.0
+    while done < warmup or spent_ms < 100.0:
+        n = max(warmup - done, 5)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        spent_ms += e0.elapsed_time(e1)
+        done += n
+    times = []
+    for _ in range(repeats):
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3 / iters)
+    return sorted(times)[len(times) // 2]
 
 
 def kernel_rooflines(dev, iters=50, warmup=10):
@@ -119,16 +142,31 @@ def kernel_rooflines(dev, iters=50, warmup=10):
         event_time_us(lambda: ops.dwconv3x3_silu_gate(u, dw, db, True), iters, warmup),
         "M*2H*2 B read + M*H*2 B write + weights")
     del u
-    for name, Nn, Kk, epi in (("gemm_qkv", 3 * C, C, None), ("gemm_proj", C, C, "bias"),
-                              ("gemm_inverted", 2 * HID, C, "bias_silu"), ("gemm_point", C, HID, None)):
+    x_ln = torch.randn(B, N, C, generator=g).bfloat16().to(dev)
+    mod = (torch.randn(B, 6, C, generator=g) * 0.5).bfloat16().to(dev)
+    add("layernorm_modulate", "hbm", 2 * M * C * 2,
+        event_time_us(lambda: ops.layernorm_modulate(x_ln, mod[:, 1:2], mod[:, 0:1], 1e-6), iters, warmup),
+        "M*C*2 B read + M*C*2 B write")
+    for name, Nn, Kk, epi in (("gemm_qkv", 3 * C, C, None), ("gemm_proj_gate_residual", C, C, "gate_res"),
+                              ("gemm_inverted", 2 * HID, C, "bias_silu"), ("gemm_point_gate_residual", C, HID, "gate_res"),
+                              ("gemm_inverted_w8a16", 2 * HID, C, "w8_bias_silu")):
         a = torch.randn(M, Kk, generator=g).bfloat16().to(dev)
         w = (torch.randn(Nn, Kk, generator=g) * 0.02).bfloat16().to(dev)
         bias = torch.zeros(Nn, dtype=torch.bfloat16, device=dev) if epi else None
         o = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
-        t_us = event_time_us(lambda: ops.gemm_bf16(a, w, bias, epi, out=o), 20, 5)
+        lib_extra = ""
+        if epi == "gate_res":     # x + gate * (a @ w.T + bias): the two gated residual seams of the block
+            fn = lambda: ops.gemm_gate_residual(a.view(B, N, Kk), w, bias, mod[:, 2:3], x_ln)
+        elif epi == "w8_bias_silu":
+            from sana_amd.modules import quantize_w8
+            wq, sc = quantize_w8(w)
+            fn = lambda: ops.gemm_w8a16(a, wq, sc, bias, "bias_silu", out=o)
+        else:
+            fn = lambda: ops.gemm_bf16(a, w, bias, epi, out=o)
+        t_us = event_time_us(fn, 20, 5)
         add(name, "mfma", 2 * M * Nn * Kk, t_us, f"2*M*K*N, M={M} N={Nn} K={Kk}")
         t_lib = event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 20, 5)
-        rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt on the same shape, for scale only
+        rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt, plain GEMM(+bias) of the same shape, for scale only
         del a, w, o
     # plain device copy as a bandwidth yardstick of this box
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -191,6 +229,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
+    ap.add_argument("--kernels-only", action="store_true", help="only the per-kernel section (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -201,6 +240,11 @@ def main():
     import sana_amd as S
 
     dev = torch.device("cuda:0")
+    if args.kernels_only:
+        with torch.no_grad():
+            kernels, copy_gbs = kernel_rooflines(dev)
+        print(json.dumps({"kernels": kernels, "copy_GBps_this_box": copy_gbs}))
+        return
     B, HW = 1, (128, 128)
     N = HW[0] * HW[1]
     blocks = []
@@ -238,9 +282,9 @@ def main():
     dom = next((r for r in kernels if r["kernel"] == "gemm_inverted"), None)
     roofline = None
     if dom:
-        roofline = {"kernel": "gemm_kernel<bf16, bias+silu> (inverted 1x1 conv, M=16384 N=11200 K=2240)",
+        roofline = {"kernel": "gemm4_kernel<bf16, bias+silu> (inverted 1x1 conv, M=16384 N=11200 K=2240)",
                     "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"], "unit": "TFLOP/s",
-                    "frac": dom["frac"], "traffic": None}
+                    "frac": dom["frac"], "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES}
     line = {
         "metric": "Sana-1.6B SanaMSBlock forward latency @16384 tokens (4096px latent)",
         "value": round(block_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -108,6 +108,15 @@ __device__ __forceinline__ uint32_t gate_res2(uint32_t y, uint32_t g, uint32_t r
   const float t0 = round_bf16(bf16_lo(g) * bf16_lo(y)), t1 = round_bf16(bf16_hi(g) * bf16_hi(y));
   return pack_bf16(bf16_lo(r) + t0, bf16_hi(r) + t1);
 }
+// y: 8 linear outputs (already rounded to bf16), g / r: the gate and residual values of the same 8 columns
+__device__ __forceinline__ u32x4_t gate_res8v(u32x4_t y, u32x4_t g, u32x4_t r) {
+  u32x4_t o;
+  o.x = gate_res2(y.x, g.x, r.x);
+  o.y = gate_res2(y.y, g.y, r.y);
+  o.z = gate_res2(y.z, g.z, r.z);
+  o.w = gate_res2(y.w, g.w, r.w);
+  return o;
+}
 // y: 8 linear outputs (already rounded to bf16) of row m, columns n..n+7
 __device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m, int n) {
   const u32x4_t g = *reinterpret_cast<const u32x4_t*>(e.gate + (int64_t)(m / e.rows_per_gate) * e.gate_stride + n);
@@ -516,10 +525,28 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   }
   const int o_chunk = lane & 15, o_rsub = lane >> 4;
   const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
-  const bool o_live = o_chunk < 4 * NI;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
+  const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
+  // Gated residual: the residual rows this lane will add are requested now, a whole epilogue ahead
+  // of their use (128 registers that the main loop no longer needs).
+  u32x4_t res[4][8];
+  if (EPI == SANA_EPI_GATE_RES) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int m = m0 + wt * 128 + 32 * j + it * 4 + o_rsub;
+        if (o_live && m < M) res[j][it] = *reinterpret_cast<const u32x4_t*>(ep.res + (int64_t)m * ep.ldr + o_n);
+      }
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int tok = 32 * j + fr;
+    // one gate row serves the whole group unless a batch boundary runs through its 32 tokens
+    const int m_first = m0 + wt * 128 + 32 * j;
+    const int g_first = m_first / ep.rows_per_gate, g_last = min(m_first + 31, M - 1) / ep.rows_per_gate;
+    u32x4_t gate = {0u, 0u, 0u, 0u};
+    if (EPI == SANA_EPI_GATE_RES && o_live && m_first < M)
+      gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
 #pragma unroll
@@ -538,8 +565,13 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       const int row = 32 * j + it * 4 + o_rsub;
       const int m = m0 + wt * 128 + row;
       u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-      if (o_live && m < M && o_n < N) {
-        if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, o_n);
+      if (o_live && m < M) {
+        if (EPI == SANA_EPI_GATE_RES) {
+          u32x4_t g = gate;
+          if (g_first != g_last && m / ep.rows_per_gate != g_first)
+            g = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
+          o = gate_res8v(o, g, res[j][it]);
+        }
         *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + o_n) = o;
       }
     }
