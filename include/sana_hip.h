@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 1
+#define SANA_HIP_ABI_VERSION 2
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -112,6 +112,48 @@ int sana_hip_linattn_apply(const void* q, const float* state, void* out,
                            int64_t o_stride_b, int64_t o_stride_n,
                            const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
                            float eps, int io_dtype, int out_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * q/k RMSNorm and rotary embedding inside the attention kernels (bf16 io)
+ *
+ * LiteLAReLURope / ChunkCausalAttention / CachedCausalAttention
+ * (sana_blocks.py:304-388, 391-495, 498-572) normalise q and k over ALL channels
+ * of a token before the head split (`self.q_norm(q)`, RMSNorm of
+ * diffusion/model/norms.py:182-231: weight * (x.float() * rsqrt(mean(x^2) + eps)),
+ * rounded to the io dtype), apply ReLU, then rotate adjacent channel pairs
+ * (2i, 2i+1) of every head by the complex factor freqs[n][i] (`apply_rotary_emb`,
+ * sana_blocks.py:359-362).  Only the numerator uses the rotated values:
+ *   vk = v @ k_rot^T,  out = vk @ q_rot,   z = 1 / (sum_n k[n] . q + eps).
+ *
+ * sana_hip_qk_rms writes the per-token statistic rsqrt(mean_c x[n][c]^2 + eps) of q
+ * and of k ([B][N] fp32 each).  The *_pre variants of the two attention phases take
+ *   rinv    [B][N] fp32 from sana_hip_qk_rms, or NULL (no norm)
+ *   weight  [h*d] bf16 RMSNorm weight (required with rinv)
+ *   rope    [N][d/2][2] fp32 (cos, sin) of freqs[n][i], shared by batch and heads, or NULL
+ * and are otherwise identical to sana_hip_linattn_state / sana_hip_linattn_apply
+ * (with all three NULL they are the same call).  SANA_ERR_DTYPE unless io is bf16.
+ */
+int sana_hip_qk_rms(const void* q, const void* k, float* q_rinv, float* k_rinv,
+                    int B, int N, int C, int64_t stride_b, int64_t stride_n,
+                    float eps, int io_dtype, void* stream);
+
+int sana_hip_linattn_state_pre(const void* k, const void* v, float* state,
+                               void* workspace, size_t workspace_bytes,
+                               int B, int N, int h, int d,
+                               int64_t stride_b, int64_t stride_n,
+                               const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+                               int causal, int io_dtype,
+                               const float* k_rinv, const void* k_weight, const float* rope,
+                               void* stream);
+
+int sana_hip_linattn_apply_pre(const void* q, const float* state, void* out,
+                               int B, int N, int h, int d,
+                               int64_t q_stride_b, int64_t q_stride_n,
+                               int64_t o_stride_b, int64_t o_stride_n,
+                               const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+                               float eps, int io_dtype, int out_dtype,
+                               const float* q_rinv, const void* q_weight, const float* rope,
+                               void* stream);
 
 /* ---------------------------------------------------------------------------
  * Depthwise 3x3 conv (zero pad 1, stride 1) + bias + SiLU gate, channels-last

@@ -27,6 +27,16 @@ SIGNATURES = {
     "sana_hip_linattn_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                        c_int64, c_int64, c_int64, c_int64,
                                        c_void_p, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    "sana_hip_qk_rms": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_int64,
+                                c_float, c_int, c_void_p]),
+    "sana_hip_linattn_state_pre": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                           c_int, c_int, c_int, c_int, c_int64, c_int64,
+                                           c_void_p, c_int, c_int, c_int, c_int,
+                                           c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sana_hip_linattn_apply_pre": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                           c_int64, c_int64, c_int64, c_int64,
+                                           c_void_p, c_int, c_int, c_float, c_int, c_int,
+                                           c_void_p, c_void_p, c_void_p, c_void_p]),
     "sana_hip_dwconv3x3_silu_gate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                              c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "sana_hip_gemm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,

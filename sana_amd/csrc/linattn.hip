@@ -51,16 +51,47 @@ __device__ __forceinline__ ChunkRange chunk_range(const int32_t* chunk_starts, i
   return r;
 }
 
+// Optional transforms of q / k on load (bf16 io): RMSNorm over all channels of the token
+// (per-token 1/rms from a statistics pass, per-channel weight), applied before the ReLU, and the
+// rotary embedding applied after it.  The rotation acts on adjacent channel pairs (2i, 2i+1) of a
+// head, i.e. on the two halves of one packed dword; only the numerator operands are rotated, the
+// ksum row / denominator use the unrotated values.
+struct QkPre {
+  const float* rinv;       // [B][N], or null
+  const uint16_t* weight;  // [h*32] bf16, with rinv
+  const float* rope;       // [N][16][2] (cos, sin) per token and pair of a head, or null
+};
+
+// bf16(w * (x * rinv)): the float chain of the reference RMSNorm, rounded once at the end
+__device__ __forceinline__ u32x4_t rms_scale8(u32x4_t x, float rinv, u32x4_t w) {
+  u32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    o[e] = pack_bf16(bf16_lo(w[e]) * (bf16_lo(x[e]) * rinv), bf16_hi(w[e]) * (bf16_hi(x[e]) * rinv));
+  return o;
+}
+// (x0 + i x1)(cos + i sin) on the four channel pairs of x; cs0 = (c, s) of pairs 0, 1; cs1 of pairs 2, 3
+__device__ __forceinline__ u32x4_t rope8(u32x4_t x, f32x4_t cs0, f32x4_t cs1) {
+  const float c[4] = {cs0[0], cs0[2], cs1[0], cs1[2]}, sn[4] = {cs0[1], cs0[3], cs1[1], cs1[3]};
+  u32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float x0 = bf16_lo(x[e]), x1 = bf16_hi(x[e]);
+    o[e] = pack_bf16(fmaf(x0, c[e], -(x1 * sn[e])), fmaf(x0, sn[e], x1 * c[e]));
+  }
+  return o;
+}
+
 // ----------------------------------------------------------------------------
 // phase 1, 16-bit io
 // grid: x = nsplit, y = n_chunks, z = B * pairs;  block 256
 // dst: when nsplit == 1 the final state, else partial[(bh*n_chunks + c)*nsplit + split][1056]
 // ----------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool PRE>
 __global__ __launch_bounds__(256) void linattn_state16_kernel(
     const uint16_t* __restrict__ K, const uint16_t* __restrict__ V, float* __restrict__ dst,
     const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int nsplit, int split_tokens,
-    int64_t stride_b, int64_t stride_n) {
+    int64_t stride_b, int64_t stride_n, const QkPre pre) {
   // staging: per wave K tile [32 tok][64 ch] + V tile, 16-bit -> 8 KB per wave.
   // reduction: per wave 2 heads x 1056 fp32 -> 8448 B per wave.  The two uses
   // never overlap in time, so they share one buffer.
@@ -96,6 +127,15 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 
   u32x4_t kreg[4], vreg[4];
+  // PRE: per-token 1/rms and this lane's four (cos, sin) pairs travel with the tile; the norm weight
+  // of the lane's 8 channels is loop-invariant; ksum is accumulated here, per lane and channel,
+  // from the unrotated values (the MFMA operands in LDS are rotated).
+  float rin[4];
+  f32x4_t cs[4][2];
+  u32x4_t kw = zero4;
+  float ks8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  if (has_norm && ch_ok) kw = *reinterpret_cast<const u32x4_t*>(pre.weight + ld_ch);
   auto issue_loads = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -103,9 +143,20 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
       if (ch_ok && tok < t1) {
         kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n);
         vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n);
+        if (has_norm) rin[i] = pre.rinv[(int64_t)b * N + tok];
+        if (has_rope) {
+          const float* rp = pre.rope + ((int64_t)tok * 16 + (lane & 3) * 4) * 2;
+          cs[i][0] = *reinterpret_cast<const f32x4_t*>(rp);
+          cs[i][1] = *reinterpret_cast<const f32x4_t*>(rp + 4);
+        }
       } else {
         kreg[i] = zero4;
         vreg[i] = zero4;
+        if (has_norm) rin[i] = 0.f;
+        if (has_rope) {
+          cs[i][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          cs[i][1] = cs[i][0];
+        }
       }
     }
   };
@@ -119,7 +170,20 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
   for (; tile < t1; tile += 4 * TILE) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4_t*>(lds_k + (ld_tok + 8 * i) * 64 + (lane & 7) * 8) = relu_pk16(kreg[i]);
+      u32x4_t kk = kreg[i];
+      if (PRE) {
+        if (has_norm) kk = rms_scale8(kk, rin[i], kw);
+        kk = relu_pk16(kk);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ks8[2 * e] += bf16_lo(kk[e]);
+          ks8[2 * e + 1] += bf16_hi(kk[e]);
+        }
+        if (has_rope) kk = rope8(kk, cs[i][0], cs[i][1]);
+      } else {
+        kk = relu_pk16(kk);
+      }
+      *reinterpret_cast<u32x4_t*>(lds_k + (ld_tok + 8 * i) * 64 + (lane & 7) * 8) = kk;
       *reinterpret_cast<u32x4_t*>(lds_v + (ld_tok + 8 * i) * 64 + (lane & 7) * 8) = vreg[i];
     }
     if (tile + 4 * TILE < t1) issue_loads(tile + 4 * TILE);
@@ -138,8 +202,10 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
           fv[r2] = vlo | (vhi << 16);
         }
         accS[hh] = mfma_32x32x16<T>(fv, fk, accS[hh]);  // S[i][j] += sum_tok V[tok][i] K[tok][j]
+        if (!PRE) {
 #pragma unroll
-        for (int r2 = 0; r2 < 4; ++r2) accK[hh] = add_pk16<T>(fk[r2], accK[hh]);  // the "1" row of [V|1]
+          for (int r2 = 0; r2 < 4; ++r2) accK[hh] = add_pk16<T>(fk[r2], accK[hh]);  // the "1" row of [V|1]
+        }
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites
@@ -156,8 +222,20 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
       const int row = 8 * (r >> 2) + 4 * g + (r & 3);
       red[hh * STATE_ELEMS + row * D + j] = accS[hh][r];
     }
-    const float ks = accK[hh] + __shfl_xor(accK[hh], 32, 64);  // the two token halves of channel j
-    if (g == 0) red[hh * STATE_ELEMS + D * D + j] = ks;
+    if (!PRE) {
+      const float ks = accK[hh] + __shfl_xor(accK[hh], 32, 64);  // the two token halves of channel j
+      if (g == 0) red[hh * STATE_ELEMS + D * D + j] = ks;
+    }
+  }
+  if (PRE) {  // lanes with the same channel chunk (lane % 8) hold different tokens: fold them
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = ks8[e];
+      x += __shfl_xor(x, 8, 64);
+      x += __shfl_xor(x, 16, 64);
+      x += __shfl_xor(x, 32, 64);
+      if (lane < 8) red[(lane >> 2) * STATE_ELEMS + D * D + (lane & 3) * 8 + e] = x;
+    }
   }
   __syncthreads();
   const float* all = reinterpret_cast<const float*>(smem);
@@ -277,11 +355,12 @@ __device__ __forceinline__ void split3(const float x[8], u32x4_t out[3]) {
   }
 }
 
-template <bool OUT_F32>
+template <bool OUT_F32, bool PRE>
 __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     const uint16_t* __restrict__ Q, const float* __restrict__ state, void* __restrict__ out,
     const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int wg_tokens,
-    int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, float eps) {
+    int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, float eps,
+    const QkPre pre) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pairs = (h + 1) >> 1;
   const int pgroups = (pairs + 3) >> 2;
@@ -315,9 +394,18 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
 
   const uint16_t* qp = Q + (int64_t)b * q_stride_b + p * 64 + 8 * g;
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  u32x4_t qw[2] = {zero4, zero4};
+  if (has_norm) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+      if (hh < nheads) qw[hh] = *reinterpret_cast<const u32x4_t*>(pre.weight + p * 64 + hh * D + 8 * g);
+  }
   constexpr int U = SANA_LA_APPLY_U;  // 16-token steps in flight
   for (int t = t0; t < t1; t += 16 * U) {
     u32x4_t qf[U][2];
+    float rin[U];
+    f32x4_t cs[U][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int tok = t + 16 * u + n;
@@ -327,20 +415,30 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
                         ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + hh * D)
                         : zero4;
       }
+      if (has_norm) rin[u] = tok < t1 ? pre.rinv[(int64_t)b * N + tok] : 0.f;
+      if (has_rope) {
+        const float* rp = pre.rope + ((int64_t)min(tok, t1 - 1) * 16 + g * 4) * 2;
+        cs[u][0] = *reinterpret_cast<const f32x4_t*>(rp);
+        cs[u][1] = *reinterpret_cast<const f32x4_t*>(rp + 4);
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int tok = t + 16 * u + n;
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
-        const u32x4_t qb = relu_pk16(qf[u][hh]);
+        u32x4_t qd = qf[u][hh];
+        if (has_norm) qd = rms_scale8(qd, rin[u], qw[hh]);
+        qd = relu_pk16(qd);                                              // denominator operand
+        const u32x4_t qb = has_rope ? rope8(qd, cs[u][0], cs[u][1]) : qd;  // numerator operand
         f32x4_t acc[3];
 #pragma unroll
         for (int rb = 0; rb < 3; ++rb) {
+          const u32x4_t bop = rb < 2 ? qb : qd;
           f32x4_t a = {0.f, 0.f, 0.f, 0.f};
-          a = mfma_16x16x32_bf16(st[hh].a[rb][2], qb, a);  // smallest term first
-          a = mfma_16x16x32_bf16(st[hh].a[rb][1], qb, a);
-          a = mfma_16x16x32_bf16(st[hh].a[rb][0], qb, a);
+          a = mfma_16x16x32_bf16(st[hh].a[rb][2], bop, a);  // smallest term first
+          a = mfma_16x16x32_bf16(st[hh].a[rb][1], bop, a);
+          a = mfma_16x16x32_bf16(st[hh].a[rb][0], bop, a);
           acc[rb] = a;
         }
         if (tok < t1 && hh < nheads) {
@@ -436,6 +534,33 @@ __global__ __launch_bounds__(256) void linattn_apply32_kernel(
   }
 }
 
+// ----------------------------------------------------------------------------
+// Per-token 1/rms of q and of k over all C channels (the statistic of the reference's
+// RMSNorm before the head split): rinv = rsqrt(mean(x^2) + eps).  One wave per (token, tensor).
+// grid: x = ceil(B*N/4), y = 2 (q, k); block 256.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void qk_rms_kernel(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                                                     float* __restrict__ rq, float* __restrict__ rk, int64_t BN,
+                                                     int N, int C, int64_t stride_b, int64_t stride_n, float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= BN) return;
+  const uint16_t* x = (blockIdx.y == 0 ? Q : K) + (row / N) * stride_b + (row % N) * stride_n;
+  float acc = 0.f;
+  for (int c0 = lane * 8; c0 < C; c0 += 512) {
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + c0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float a = bf16_lo(v[e]), b2 = bf16_hi(v[e]);
+      acc = fmaf(a, a, acc);
+      acc = fmaf(b2, b2, acc);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0) (blockIdx.y == 0 ? rq : rk)[row] = rsqrtf(acc / (float)C + eps);
+}
+
 // ---------------------------------------------------------------------------- host side
 
 int pick_nsplit(int items, int max_chunk_tokens, int min_tokens) {
@@ -485,11 +610,23 @@ extern "C" __attribute__((visibility("default"))) size_t sana_hip_linattn_worksp
   return pl.nsplit > 1 ? (size_t)B * h * n_chunks * pl.nsplit * STATE_ELEMS * sizeof(float) : 0;
 }
 
-extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(const void* k, const void* v, float* state, void* workspace,
-                                      size_t workspace_bytes, int B, int N, int h, int d, int64_t stride_b,
-                                      int64_t stride_n, const int32_t* chunk_starts, int n_chunks,
-                                      int max_chunk_tokens, int causal, int io_dtype, void* stream) {
+static int check_pre(const QkPre& pre, int io_dtype) {
+  if (!pre.rinv && !pre.rope) return SANA_OK;
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (pre.rinv && !pre.weight) return SANA_ERR_ARG;
+  if ((pre.weight && !aligned16(pre.weight)) || (pre.rope && !aligned16(pre.rope))) return SANA_ERR_ALIGN;
+  return SANA_OK;
+}
+
+static int state_impl(const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B,
+                      int N, int h, int d, int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts,
+                      int n_chunks, int max_chunk_tokens, int causal, int io_dtype, const QkPre pre, void* stream) {
   if (!k || !v || !state || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  const bool use_pre = pre.rinv || pre.rope;
+  {
+    const int rc = check_pre(pre, io_dtype);
+    if (rc != SANA_OK) return rc;
+  }
   if (d != D) return SANA_ERR_SHAPE;
   if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
   if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
@@ -516,14 +653,18 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(con
                        pl.split_tokens, stride_b, stride_n);
   } else {
     dim3 grid(pl.nsplit, n_chunks, B * ((h + 1) / 2));
-    if (io_dtype == SANA_DT_BF16)
-      hipLaunchKernelGGL(linattn_state16_kernel<BF16>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
+    if (io_dtype == SANA_DT_BF16 && use_pre)
+      hipLaunchKernelGGL((linattn_state16_kernel<BF16, true>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
                          static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
-                         pl.split_tokens, stride_b, stride_n);
+                         pl.split_tokens, stride_b, stride_n, pre);
+    else if (io_dtype == SANA_DT_BF16)
+      hipLaunchKernelGGL((linattn_state16_kernel<BF16, false>), grid, dim3(256), 0, s,
+                         static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v), dst, chunk_starts, N, h,
+                         n_chunks, pl.nsplit, pl.split_tokens, stride_b, stride_n, pre);
     else
-      hipLaunchKernelGGL(linattn_state16_kernel<F16>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
-                         static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
-                         pl.split_tokens, stride_b, stride_n);
+      hipLaunchKernelGGL((linattn_state16_kernel<F16, false>), grid, dim3(256), 0, s,
+                         static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v), dst, chunk_starts, N, h,
+                         n_chunks, pl.nsplit, pl.split_tokens, stride_b, stride_n, pre);
   }
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
   const bool scan = causal && n_chunks > 1;
@@ -536,6 +677,41 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(con
   return SANA_OK;
 }
 
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(
+    const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N, int h, int d,
+    int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens, int causal,
+    int io_dtype, void* stream) {
+  const QkPre none = {nullptr, nullptr, nullptr};
+  return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, chunk_starts, n_chunks,
+                    max_chunk_tokens, causal, io_dtype, none, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state_pre(
+    const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N, int h, int d,
+    int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens, int causal,
+    int io_dtype, const float* k_rinv, const void* k_weight, const float* rope, void* stream) {
+  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope};
+  return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, chunk_starts, n_chunks,
+                    max_chunk_tokens, causal, io_dtype, pre, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_qk_rms(const void* q, const void* k, float* q_rinv,
+                                                                      float* k_rinv, int B, int N, int C,
+                                                                      int64_t stride_b, int64_t stride_n, float eps,
+                                                                      int io_dtype, void* stream) {
+  if (!q || !k || !q_rinv || !k_rinv || B <= 0 || N <= 0 || C <= 0) return SANA_ERR_ARG;
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (C % 8) return SANA_ERR_SHAPE;
+  if (stride_n < C || stride_b < 0) return SANA_ERR_ARG;
+  if (!aligned16(q) || !aligned16(k) || (stride_n * 2) % 16 || (stride_b * 2) % 16) return SANA_ERR_ALIGN;
+  const int64_t BN = (int64_t)B * N;
+  if ((BN + 3) / 4 > 0x7fffffff) return SANA_ERR_SHAPE;
+  hipLaunchKernelGGL(qk_rms_kernel, dim3((unsigned)((BN + 3) / 4), 2), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k), q_rinv, k_rinv, BN, N, C,
+                     stride_b, stride_n, eps);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
 extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_chunk_scan(float* state, int B, int h, int d, int n_chunks, void* stream) {
   if (!state || B <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
   if (d != D) return SANA_ERR_SHAPE;
@@ -546,11 +722,16 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_chunk_sca
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
-extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(const void* q, const float* state, void* out, int B, int N, int h, int d,
-                                      int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b,
-                                      int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks,
-                                      int max_chunk_tokens, float eps, int io_dtype, int out_dtype, void* stream) {
+static int apply_impl(const void* q, const float* state, void* out, int B, int N, int h, int d, int64_t q_stride_b,
+                      int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts,
+                      int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre pre,
+                      void* stream) {
   if (!q || !state || !out || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  const bool use_pre = pre.rinv || pre.rope;
+  {
+    const int rc = check_pre(pre, io_dtype);
+    if (rc != SANA_OK) return rc;
+  }
   if (d != D) return SANA_ERR_SHAPE;
   if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
   if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
@@ -570,14 +751,18 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(con
   if (io_dtype == SANA_DT_BF16) {
     const int pairs = (h + 1) / 2;
     dim3 grid(gx, n_chunks, B * ((pairs + 3) / 4));
-    if (out_dtype == SANA_DT_F32)
-      hipLaunchKernelGGL(linattn_apply_bf16_kernel<true>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(q),
-                         state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,
-                         o_stride_n, eps);
-    else
-      hipLaunchKernelGGL(linattn_apply_bf16_kernel<false>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(q),
-                         state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,
-                         o_stride_n, eps);
+#define SANA_APPLY(F32, PRE)                                                                                   \
+  hipLaunchKernelGGL((linattn_apply_bf16_kernel<F32, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(q), \
+                     state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,     \
+                     o_stride_n, eps, pre)
+    if (out_dtype == SANA_DT_F32) {
+      if (use_pre) SANA_APPLY(true, true);
+      else SANA_APPLY(true, false);
+    } else {
+      if (use_pre) SANA_APPLY(false, true);
+      else SANA_APPLY(false, false);
+    }
+#undef SANA_APPLY
   } else {
     dim3 grid(gx, n_chunks, B * ((h + 3) / 4));
     if (io_dtype == SANA_DT_F32)
@@ -594,4 +779,23 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(con
                          n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps);
   }
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(
+    const void* q, const float* state, void* out, int B, int N, int h, int d, int64_t q_stride_b, int64_t q_stride_n,
+    int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+    float eps, int io_dtype, int out_dtype, void* stream) {
+  const QkPre none = {nullptr, nullptr, nullptr};
+  return apply_impl(q, state, out, B, N, h, d, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
+                    n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, none, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply_pre(
+    const void* q, const float* state, void* out, int B, int N, int h, int d, int64_t q_stride_b, int64_t q_stride_n,
+    int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+    float eps, int io_dtype, int out_dtype, const float* q_rinv, const void* q_weight, const float* rope,
+    void* stream) {
+  const QkPre pre = {q_rinv, static_cast<const uint16_t*>(q_weight), rope};
+  return apply_impl(q, state, out, B, N, h, d, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
+                    n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, pre, stream);
 }

@@ -217,9 +217,45 @@ class LiteLA(nn.Module):
     def forward_gated(self, x, gate, residual, rotary_emb=None) -> torch.Tensor:
         """forward(x), or residual + gate * forward(x) with the update fused into the proj GEMM."""
         _no_grad_only(x)
-        qkv = self._qkv_tokens(x, rotary_emb)
-        out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps)
+        if rotary_emb is None and x.dtype == torch.bfloat16:   # qk-norm (if any) on load inside the kernels
+            B, N, C = x.shape
+            out = self._attend(self.qkv(x).view(B, N, 3, C), None)
+        else:
+            qkv = self._qkv_tokens(x, rotary_emb)
+            out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps)
         return self.proj(out, gate=gate, residual=residual)
+
+    def _pre(self, qkv: torch.Tensor, rotary_emb):
+        """(QkPre for q, QkPre for k) for a fused [B, N, 3, C] buffer, or (None, None)."""
+        B, N = qkv.shape[:2]
+        norm = not isinstance(self.q_norm, nn.Identity)
+        if not norm and rotary_emb is None:
+            return None, None
+        if qkv.dtype != torch.bfloat16:
+            raise NotImplementedError("qk-norm / rotary embedding inside the attention kernels is bf16 only")
+        rope = None
+        if rotary_emb is not None:
+            cache = self.__dict__.get("_rope_cache")
+            key = (id(rotary_emb), rotary_emb._version, N, qkv.device)
+            if cache is None or cache[0] != key:
+                cache = (key, ops.rope_table(rotary_emb, N, qkv.device))
+                self.__dict__["_rope_cache"] = cache
+            rope = cache[1]
+        if norm:
+            if self.q_norm.eps != self.k_norm.eps:
+                raise NotImplementedError("q_norm and k_norm with different eps")
+            rq, rk = ops.qk_rms(qkv[:, :, 0], qkv[:, :, 1], self.q_norm.eps)
+            wq = self.q_norm.weight.detach().to(torch.bfloat16).contiguous()
+            wk = self.k_norm.weight.detach().to(torch.bfloat16).contiguous()
+            return ops.QkPre(rq, wq, rope), ops.QkPre(rk, wk, rope)
+        return ops.QkPre(rope=rope), ops.QkPre(rope=rope)
+
+    def _attend(self, qkv, rotary_emb, chunk_tokens=None):
+        pre_q, pre_k = self._pre(qkv, rotary_emb)
+        causal = chunk_tokens is not None and len(chunk_tokens) > 1
+        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], chunk_tokens, causal=causal, pre=pre_k)
+        return ops.linattn_apply(qkv[:, :, 0], state, self.eps, chunk_tokens, pre=pre_q)
+
 
     def quantize_w8_(self) -> "LiteLA":
         self.qkv.quantize_w8_()
@@ -230,18 +266,33 @@ class LiteLA(nn.Module):
         return f"EPS{self.eps}-" + super().__repr__()
 
 
-class ChunkCausalAttention(LiteLA):
+class LiteLAReLURope(LiteLA):
+    """ReLU linear attention with the rotary embedding applied AFTER the ReLU and to the
+    numerator only (reference: sana_blocks.py:304-388): ``vk = v @ rope(relu(k))^T``,
+    ``out = vk @ rope(relu(q))``, ``z = 1 / (sum_n relu(k_n) . relu(q) + eps)``.
+    ``rotary_emb`` is the complex factor tensor [1, 1, N, d/2] the reference passes
+    (``None`` = the unit rotation).  RMSNorm of q / k, the ReLU and the rotation all happen
+    on load inside the two attention kernels (bf16); nothing is written back to the qkv buffer."""
+
+    def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None, **kwargs) -> torch.Tensor:
+        return self.forward_gated(x, None, None, rotary_emb=rotary_emb)
+
+    def forward_gated(self, x, gate, residual, rotary_emb=None) -> torch.Tensor:
+        _no_grad_only(x)
+        B, N, C = x.shape
+        qkv = self.qkv(x).view(B, N, 3, C)
+        return self.proj(self._attend(qkv, rotary_emb), gate=gate, residual=residual)
+
+
+class ChunkCausalAttention(LiteLAReLURope):
     """Chunk-causal ReLU linear attention (reference: sana_blocks.py:391-495):
     every chunk of whole frames attends to the running sum of the states of all
     earlier chunks plus its own.  ``HW = (frames, h, w)``; ``chunk_index`` lists
-    the first frame of each chunk.  This build covers the form without rotary
-    embedding (``rotary_emb=None``, the reference's unit rotation)."""
+    the first frame of each chunk; ``rotary_emb`` as in :class:`LiteLAReLURope`."""
 
     def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None,
                 chunk_index: Optional[List[int]] = None) -> torch.Tensor:
         _no_grad_only(x)
-        if rotary_emb is not None:
-            raise NotImplementedError("ChunkCausalAttention: the rotary (ReLU -> RoPE) variant is not built yet")
         if HW is None or len(HW) != 3:
             raise ValueError("ChunkCausalAttention needs HW = (frames, h, w)")
         f, hh, ww = HW
@@ -249,10 +300,52 @@ class ChunkCausalAttention(LiteLA):
         if f * hh * ww != N:
             raise ValueError(f"HW={HW} does not match N={N}")
         starts = list(chunk_index) if chunk_index is not None else [0]
-        qkv = self._qkv_tokens(x)
-        out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps,
-                                        chunk_tokens=[s * hh * ww for s in starts])
+        qkv = self.qkv(x).view(B, N, 3, C)
+        out = self._attend(qkv, rotary_emb, chunk_tokens=[s * hh * ww for s in starts])
         return self.proj(out)
+
+
+class CachedCausalAttention(LiteLAReLURope):
+    """Streaming form of the chunk-causal attention (reference: sana_blocks.py:498-572): the call
+    sees one chunk, computes that chunk's own state, optionally saves it UN-accumulated into
+    ``kv_cache[0:2]`` (``vk`` [B, h, d, d] and ``k_sum`` [B, h, 1, d], here fp32), adds the
+    accumulated past the caller supplies in the same two slots, and returns ``(out, kv_cache)``.
+    The caller accumulates saved states across chunks (:func:`accumulate_kv_cache`, the host-side
+    loop of diffusion/longsana/pipeline/sana_inference_pipeline.py:242-263)."""
+
+    def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None,
+                save_kv_cache: bool = False, kv_cache: Optional[list] = None, **kwargs):
+        _no_grad_only(x)
+        B, N, C = x.shape
+        qkv = self.qkv(x).view(B, N, 3, C)
+        pre_q, pre_k = self._pre(qkv, rotary_emb)
+        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], pre=pre_k)   # [B, h, 1, 33, 32]: this chunk only
+        if kv_cache is not None:
+            past_vk, past_ks = kv_cache[0], kv_cache[1]
+            if save_kv_cache:
+                kv_cache[0] = state[:, :, 0, :HEAD_DIM].clone()
+                kv_cache[1] = state[:, :, 0, HEAD_DIM:].clone()
+            if past_vk is not None and past_ks is not None:
+                state[:, :, 0, :HEAD_DIM] += past_vk.to(state)
+                state[:, :, 0, HEAD_DIM:] += past_ks.to(state)
+        out = self.proj(ops.linattn_apply(qkv[:, :, 0], state, self.eps, pre=pre_q))
+        if kv_cache is not None:
+            return out, kv_cache
+        return out
+
+
+def accumulate_kv_cache(accumulated: Optional[list], saved: list) -> list:
+    """Running sum of the attention states a :class:`CachedCausalAttention` saved, as the streaming
+    pipeline keeps it between chunks (sana_inference_pipeline.py:242-263): slots 0 and 1 add up,
+    any further slot (the temporal-conv tail) is replaced by the newest value."""
+    if accumulated is None:
+        return [None if t is None else t.clone() for t in saved]
+    out = list(accumulated)
+    for i, t in enumerate(saved):
+        if t is None:
+            continue
+        out[i] = t.clone() if (i >= 2 or out[i] is None) else out[i] + t
+    return out
 
 
 # ------------------------------------------------------------------ Mix-FFN

@@ -68,7 +68,67 @@ def _token_major_view(t: torch.Tensor, what: str) -> Tuple[int, int]:
     return (t.stride(0) if t.shape[0] > 1 else 0), t.stride(1)
 
 
-def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False) -> torch.Tensor:
+class QkPre:
+    """Transforms applied to q or k on load inside the attention kernels (bf16 io):
+    RMSNorm over all channels (``rinv`` [B, N] fp32 from :func:`qk_rms` and the bf16
+    ``weight`` [C]) before the ReLU, rotary embedding (``rope`` [N, 16, 2] fp32 from
+    :func:`rope_table`) after it, on the numerator operands only."""
+
+    __slots__ = ("rinv", "weight", "rope")
+
+    def __init__(self, rinv=None, weight=None, rope=None):
+        if (rinv is None) != (weight is None):
+            raise SanaHipError("rinv and weight go together")
+        self.rinv, self.weight, self.rope = rinv, weight, rope
+
+    def check(self, x: torch.Tensor) -> Tuple[Optional[int], Optional[int], Optional[int]]:
+        B, N, C = x.shape
+        _need_cuda(self.rinv, self.weight, self.rope)
+        if x.dtype != torch.bfloat16:
+            raise SanaHipError("qk-norm / rotary embedding inside the kernels is bf16 only")
+        if self.rinv is not None:
+            if self.rinv.dtype != torch.float32 or tuple(self.rinv.shape) != (B, N) or not self.rinv.is_contiguous():
+                raise SanaHipError(f"rinv must be contiguous fp32 {(B, N)}")
+            if self.weight.dtype != torch.bfloat16 or self.weight.numel() != C or not self.weight.is_contiguous():
+                raise SanaHipError(f"norm weight must be contiguous bf16 [{C}]")
+        if self.rope is not None:
+            if self.rope.dtype != torch.float32 or tuple(self.rope.shape) != (N, HEAD_DIM // 2, 2) or \
+                    not self.rope.is_contiguous():
+                raise SanaHipError(f"rope must be contiguous fp32 {(N, HEAD_DIM // 2, 2)}")
+        ptr = lambda t: None if t is None else t.data_ptr()
+        return ptr(self.rinv), ptr(self.weight), ptr(self.rope)
+
+
+def qk_rms(q: torch.Tensor, k: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-token rsqrt(mean_c x^2 + eps) of q and of k: [B, N, C] bf16 views with equal strides -> two fp32 [B, N]."""
+    _need_cuda(q, k)
+    same = all(a == b or n == 1 for a, b, n in zip(q.stride(), k.stride(), q.shape))
+    if q.shape != k.shape or q.dtype != k.dtype or not same:
+        raise SanaHipError("q and k must share shape, dtype and strides")
+    B, N, C = q.shape
+    sb, sn = _token_major_view(q, "q")
+    rq = torch.empty(B, N, dtype=torch.float32, device=q.device)
+    rk = torch.empty(B, N, dtype=torch.float32, device=q.device)
+    code = _lib.load().sana_hip_qk_rms(q.data_ptr(), k.data_ptr(), rq.data_ptr(), rk.data_ptr(), B, N, C, sb, sn,
+                                       float(eps), _dt(q), _stream())
+    _lib.check(code, "sana_hip_qk_rms")
+    return rq, rk
+
+
+def rope_table(freqs: torch.Tensor, N: int, device) -> torch.Tensor:
+    """Complex rotary factors [..., N, 16] (any leading singleton dims, as the reference passes
+    ``rotary_emb`` [1, 1, N, d/2]) -> fp32 (cos, sin) table [N, 16, 2] on ``device``."""
+    if not torch.is_complex(freqs):
+        raise SanaHipError("rotary_emb must be a complex tensor of unit factors")
+    f = freqs.reshape(-1, freqs.shape[-1])
+    if tuple(f.shape) != (N, HEAD_DIM // 2):
+        raise SanaHipError(f"rotary_emb must broadcast over batch and heads: expected [.., {N}, {HEAD_DIM // 2}], "
+                           f"got {tuple(freqs.shape)}")
+    return torch.view_as_real(f.to(torch.complex64)).to(device=device, dtype=torch.float32).contiguous()
+
+
+def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False,
+                  pre: Optional[QkPre] = None) -> torch.Tensor:
     """Phase 1.  k, v: [B, N, C] token-major views (C = h*32).  Returns the fp32
     state [B, h, n_chunks, 33, 32] (inclusive prefix over chunks when causal)."""
     _need_cuda(k, v)
@@ -85,10 +145,13 @@ def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: b
     state = torch.empty(B, h, n_chunks, HEAD_DIM + 1, HEAD_DIM, dtype=torch.float32, device=k.device)
     nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, HEAD_DIM, n_chunks, longest, _dt(k))
     ws = _workspace(k.device, nbytes)
-    code = lib.sana_hip_linattn_state(
-        k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
-        B, N, h, HEAD_DIM, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
-        1 if causal else 0, _dt(k), _stream())
+    args = (k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
+            B, N, h, HEAD_DIM, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
+            1 if causal else 0, _dt(k))
+    if pre is None:
+        code = lib.sana_hip_linattn_state(*args, _stream())
+    else:
+        code = lib.sana_hip_linattn_state_pre(*args, *pre.check(k), _stream())
     _lib.check(code, "sana_hip_linattn_state")
     return state
 
@@ -105,7 +168,8 @@ def linattn_chunk_scan_(state: torch.Tensor) -> torch.Tensor:
 
 
 def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens=None,
-                  out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
+                  pre: Optional[QkPre] = None) -> torch.Tensor:
     """Phase 2.  q: [B, N, C] token-major view; state from :func:`linattn_state`.
     Returns [B, N, C] in ``out_dtype`` (q's dtype or fp32)."""
     _need_cuda(q, state)
@@ -122,10 +186,12 @@ def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens
     elif out.shape != q.shape or out.dtype != out_dtype:
         raise SanaHipError("out has the wrong shape or dtype")
     osb, osn = _token_major_view(out, "out")
-    code = _lib.load().sana_hip_linattn_apply(
-        q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, HEAD_DIM, qsb, qsn, osb, osn,
-        tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype],
-        _stream())
+    args = (q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, HEAD_DIM, qsb, qsn, osb, osn,
+            tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype])
+    if pre is None:
+        code = _lib.load().sana_hip_linattn_apply(*args, _stream())
+    else:
+        code = _lib.load().sana_hip_linattn_apply_pre(*args, *pre.check(q), _stream())
     _lib.check(code, "sana_hip_linattn_apply")
     return out
 

@@ -1,0 +1,141 @@
+"""GPU parity of the attention variants with q/k RMSNorm and rotary embedding applied inside the
+kernels (LiteLAReLURope, ChunkCausalAttention with rotary_emb, CachedCausalAttention) against the
+oracle's restatement of the reference modules, same state_dict, same seeded inputs."""
+import copy
+
+import pytest
+import torch
+
+import sana_amd as S
+from oracle import sana_oracle as O
+from sana_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+
+def check(out, ref, what=""):
+    """north-star tolerance for bf16 attention outputs: max-abs 2e-2, rel-L2 1e-2 (against fp64)."""
+    mx = (out.double().cpu() - ref.double()).abs().max().item()
+    rl = rel_l2(out.cpu(), ref)
+    assert mx <= 2e-2 and rl <= 1e-2, f"{what}: max-abs {mx:.3e} rel-L2 {rl:.3e}"
+
+
+def freqs(N, seed=0):
+    """Unit complex rotary factors [1, 1, N, 16], as the reference passes rotary_emb."""
+    theta = torch.rand(N, 16, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * 6.283
+    return torch.polar(torch.ones_like(theta), theta)[None, None]
+
+
+def make(cls_name, C, qk_norm, seed):
+    heads = C // 32
+    om = getattr(O, cls_name)(C, C, heads=heads, eps=1e-8, qk_norm=qk_norm)
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for n, p in om.named_parameters():
+            if "norm" in n:
+                p.copy_(1.0 + 0.3 * torch.randn(p.shape, generator=g))
+            elif n.endswith("bias"):
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+            else:
+                p.copy_(torch.randn(p.shape, generator=g) * (2.0 / C) ** 0.5)
+    om = om.bfloat16()
+    hm = getattr(S, cls_name)(C, C, heads=heads, eps=1e-8, qk_norm=qk_norm).bfloat16()
+    hm.load_state_dict(om.state_dict(), strict=True)
+    return om, hm
+
+
+def ref64(module, x, **kw):
+    m = copy.deepcopy(module).double()
+    return m(x.double(), **kw)
+
+
+@pytest.mark.parametrize("B,N,C", [(2, 1024, 1152), (1, 16384, 2240)])
+def test_qk_rms_statistic(cuda, B, N, C):
+    g = torch.Generator().manual_seed(N + C)
+    qkv = (torch.randn(B, N, 3, C, generator=g) * 1.7).bfloat16().to(cuda)
+    rq, rk = ops.qk_rms(qkv[:, :, 0], qkv[:, :, 1], 1e-5)
+    for r, x in ((rq, qkv[:, :, 0]), (rk, qkv[:, :, 1])):
+        ref = torch.rsqrt(x.double().pow(2).mean(-1) + 1e-5)
+        assert r.shape == (B, N) and r.dtype == torch.float32
+        assert ((r.double() - ref).abs() / ref).max().item() <= 2e-6
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+@pytest.mark.parametrize("rot", [False, True])
+@pytest.mark.parametrize("B,N,C", [(2, 640, 1152), (1, 77, 96), (1, 4096, 2240)])
+def test_litela_relu_rope(cuda, B, N, C, qk_norm, rot):
+    om, hm = make("LiteLAReLURope", C, qk_norm, seed=N)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(1)).bfloat16()
+    f = freqs(N) if rot else None
+    with torch.no_grad():
+        ref = ref64(om, x, rotary_emb=f)
+        out = hm(x.to(cuda), rotary_emb=None if f is None else f.to(cuda))
+    assert out.dtype == torch.bfloat16 and out.shape == (B, N, C)
+    check(out, ref, f"LiteLAReLURope norm={qk_norm} rope={rot}")
+
+
+def test_rotation_is_numerator_only_and_unit_rotation_is_identity(cuda):
+    """theta = 0 must reproduce the call without rotary_emb bit for bit; a rotation by pi flips the sign of
+    every rotated q and k, which cancels in the numerator (vk . q_rot) and never touches the denominator."""
+    B, N, C = 1, 512, 256
+    om, hm = make("LiteLAReLURope", C, False, seed=9)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(2)).bfloat16().to(cuda)
+    one = torch.ones(1, 1, N, 16, dtype=torch.complex128)
+    with torch.no_grad():
+        base = hm(x)
+        assert torch.equal(hm(x, rotary_emb=one.to(cuda)), base)
+        assert torch.equal(hm(x, rotary_emb=(-one).to(cuda)), base)
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+def test_chunk_causal_with_rope(cuda, qk_norm):
+    B, (f, h, w), C = 1, (5, 6, 8), 160
+    N = f * h * w
+    om, hm = make("ChunkCausalAttention", C, qk_norm, seed=4)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(3)).bfloat16()
+    fr = freqs(N, 5)
+    with torch.no_grad():
+        ref = ref64(om, x, HW=(f, h, w), rotary_emb=fr, chunk_index=[0, 1, 3])
+        out = hm(x.to(cuda), HW=(f, h, w), rotary_emb=fr.to(cuda), chunk_index=[0, 1, 3])
+    check(out, ref, "ChunkCausalAttention + rope")
+
+
+def test_cached_stream_equals_chunk_causal(cuda):
+    """Feeding chunks one at a time through CachedCausalAttention, with the caller accumulating the
+    saved states, reproduces the chunk-causal module on the whole sequence; and each step matches
+    the oracle's cached module given the same accumulated past."""
+    B, (f, h, w), C = 2, (6, 4, 8), 128
+    hw = h * w
+    N = f * hw
+    om, hm = make("CachedCausalAttention", C, True, seed=6)
+    whole = S.ChunkCausalAttention(C, C, heads=C // 32, eps=1e-8, qk_norm=True).bfloat16()
+    whole.load_state_dict(om.state_dict(), strict=True)
+    hm, whole = hm.to(cuda), whole.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(7)).bfloat16()
+    fr = freqs(N, 8)
+    starts = [0, 2, 3, 6]
+    with torch.no_grad():
+        full = whole(x.to(cuda), HW=(f, h, w), rotary_emb=fr.to(cuda), chunk_index=starts[:-1])
+        acc, acc_ref = None, None
+        o64 = copy.deepcopy(om).double()
+        for a, b in zip(starts[:-1], starts[1:]):
+            xs, fs = x[:, a * hw:b * hw], fr[:, :, a * hw:b * hw]
+            cache = [None, None] if acc is None else [acc[0], acc[1]]
+            out, cache = hm(xs.to(cuda), rotary_emb=fs.to(cuda), save_kv_cache=True, kv_cache=cache)
+            assert cache[0].shape == (B, C // 32, 32, 32) and cache[1].shape == (B, C // 32, 1, 32)
+            acc = S.accumulate_kv_cache(acc, cache)
+            # the streamed chunk equals the same tokens of the whole-sequence chunk-causal call
+            assert (out.float() - full[:, a * hw:b * hw].float()).abs().max().item() <= 2e-2
+            # and the oracle's cached module, given its own accumulated past
+            cache_ref = [None, None] if acc_ref is None else [acc_ref[0], acc_ref[1]]
+            ref, cache_ref = o64(xs.double(), rotary_emb=fs, save_kv_cache=True, kv_cache=cache_ref)
+            acc_ref = cache_ref if acc_ref is None else [acc_ref[0] + cache_ref[0], acc_ref[1] + cache_ref[1]]
+            check(out, ref, f"cached chunk {a}:{b}")
+            assert rel_l2(cache[0].cpu(), cache_ref[0]) <= 1e-2 and rel_l2(cache[1].cpu(), cache_ref[1]) <= 1e-2

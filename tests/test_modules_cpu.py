@@ -10,7 +10,8 @@ import sana_amd as S
 from oracle import sana_oracle as O
 
 
-@pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention"])
+@pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention", "LiteLAReLURope",
+                                  "CachedCausalAttention"])
 def test_constructor_and_forward_signatures_match(name):
     a, b = getattr(S, name), getattr(O, name)
     pa = list(inspect.signature(a.__init__).parameters)
