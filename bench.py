@@ -135,6 +135,35 @@ def kernel_rooflines(dev, iters=50, warmup=10):
     add("linattn_apply", "hbm", la_bytes,
         event_time_us(lambda: ops.linattn_apply(q, state, 1e-8, out=out), iters, warmup),
         "M*C*2 B (Q read) + M*C*2 B (out write) + state read")
+    # the same two phases with q/k RMSNorm and the rotary embedding applied on load (LiteLAReLURope), plus
+    # the statistics pass they need; and the chunk-causal video shape (21 frames x 30x52 tokens, one chunk per frame)
+    wn = (1 + 0.1 * torch.randn(C, generator=g)).bfloat16().to(dev)
+    theta = torch.rand(N, 16, generator=g, dtype=torch.float64) * 6.283
+    rope = ops.rope_table(torch.polar(torch.ones_like(theta), theta), N, dev)
+    rq, rk = ops.qk_rms(q, k, 1e-5)
+    add("qk_rms", "hbm", 2 * M * C * 2 + 2 * M * 4, event_time_us(lambda: ops.qk_rms(q, k, 1e-5), iters, warmup),
+        "2*M*C*2 B (Q,K read) + 2*M*4 B")
+    pre_k, pre_q = ops.QkPre(rk, wn, rope), ops.QkPre(rq, wn, rope)
+    rope_bytes = M * 16 * 2 * 4 + M * 4
+    add("linattn_state_norm_rope", "hbm", la_bytes + rope_bytes,
+        event_time_us(lambda: ops.linattn_state(k, v, pre=pre_k), iters, warmup),
+        "as linattn_state + rope table (128 B/token) + 1/rms (4 B/token)")
+    add("linattn_apply_norm_rope", "hbm", la_bytes + rope_bytes,
+        event_time_us(lambda: ops.linattn_apply(q, state, 1e-8, out=out, pre=pre_q), iters, warmup),
+        "as linattn_apply + rope table + 1/rms")
+    Nv, hw = 21 * 30 * 52, 30 * 52
+    qkv5 = torch.randn(1, Nv, 3, C, generator=g).bfloat16().to(dev)
+    starts = [f * hw for f in range(21)]
+    st5 = ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts, causal=True)
+    out5 = torch.empty(1, Nv, C, dtype=torch.bfloat16, device=dev)
+    la5 = 2 * Nv * C * 2 + 21 * (C // 32) * 33 * 32 * 4
+    add("linattn_state_chunk_causal_cfg5", "hbm", la5,
+        event_time_us(lambda: ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts, causal=True), iters, warmup),
+        "cfg5: N=32760, 21 chunks; K,V read + 21 states")
+    add("linattn_apply_chunk_causal_cfg5", "hbm", la5,
+        event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st5, 1e-8, starts, out=out5), iters, warmup),
+        "cfg5: Q read + out write + 21 states")
+    del qkv5, out5
     u = torch.randn(B, 128, 128, 2 * HID, generator=g).bfloat16().to(dev)
     dw = (torch.randn(2 * HID, 1, 3, 3, generator=g) * 0.3).bfloat16().to(dev)
     db = torch.zeros(2 * HID, dtype=torch.bfloat16, device=dev)
