@@ -408,6 +408,91 @@ class GLUMBConv(nn.Module):
         return x
 
 
+class GLUMBConvTemp(GLUMBConv):
+    """diffusion/model/nets/basic_modules.py:200-264 (single GPU: no halo exchange).  The Mix-FFN per
+    frame, then a residual temporal conv (kernel (t, 1), full channel mixing, zero-initialised)."""
+
+    def __init__(self, in_features, hidden_features, out_feature=None, kernel_size=3, stride=1, padding=None,
+                 use_bias=False, norm=(None, None, None), act=("silu", "silu", None), t_kernel_size=3):
+        super().__init__(in_features, hidden_features, out_feature=out_feature, kernel_size=kernel_size,
+                         stride=stride, padding=padding, use_bias=use_bias, norm=norm, act=act)
+        out_feature = out_feature or in_features
+        self.t_conv = nn.Conv2d(out_feature, out_feature, kernel_size=(t_kernel_size, 1), stride=1,
+                                padding=(t_kernel_size // 2, 0), bias=False)
+        nn.init.zeros_(self.t_conv.weight)
+
+    def _spatial_bcthw(self, x, HW):
+        """:238-246: tokens -> (B, C, T, H*W) after the per-frame Mix-FFN."""
+        B, N, C = x.shape
+        assert len(HW) == 3, "HW must be a tuple of (T, H, W)"
+        T, H, W = HW
+        x = x.reshape(B * T, H, W, C).permute(0, 3, 1, 2)
+        x = self._apply_spatial_autochunked(x)
+        return x.view(B, T, C, H * W).permute(0, 2, 1, 3)
+
+    def forward(self, x, HW=None, **kwargs):
+        B, N, C = x.shape
+        x_reshaped = self._spatial_bcthw(x, HW)
+        frame_mask = kwargs.get("frame_valid_mask", None)
+        if frame_mask is not None:
+            frame_mask = frame_mask.reshape(B, HW[0]).to(x_reshaped)
+            x_reshaped = x_reshaped * frame_mask[:, None, :, None]
+        x_out = x_reshaped + self.t_conv(x_reshaped)
+        if frame_mask is not None:
+            x_out = x_out * frame_mask[:, None, :, None]
+        return x_out.permute(0, 2, 3, 1).reshape(B, N, C)
+
+
+class ChunkGLUMBConvTemp(GLUMBConvTemp):
+    """basic_modules.py:267-354 (single GPU).  The temporal conv sees, for every chunk of frames, the
+    tail of the previous chunk on the left and zeros on the right."""
+
+    def forward(self, x, HW=None, chunk_index=None, **kwargs):
+        if chunk_index is None:
+            chunk_index = [0]
+        B, N, C = x.shape
+        T = HW[0]
+        x_reshaped = self._spatial_bcthw(x, HW)
+        frame_mask = kwargs.get("frame_valid_mask")
+        if frame_mask is not None:
+            frame_mask = frame_mask.reshape(B, T).to(x_reshaped)
+            x_reshaped = x_reshaped * frame_mask[:, None, :, None]
+        pad = self.t_conv.kernel_size[0] // 2
+        bounds = sorted({0, *(int(i) for i in chunk_index if 0 < int(i) < T), T})
+        outs = []
+        for a, b in zip(bounds[:-1], bounds[1:]):
+            left = x_reshaped[:, :, a - pad:a] if a > 0 else x_reshaped.new_zeros(B, C, 0, x_reshaped.shape[-1])
+            seg = torch.cat([left, x_reshaped[:, :, a:b], x_reshaped.new_zeros(B, C, pad, x_reshaped.shape[-1])], dim=2)
+            o = self.t_conv(seg)   # its own zero padding adds `pad` rows either side
+            outs.append(o[:, :, left.shape[2]:left.shape[2] + (b - a)])
+        x_out = x_reshaped + torch.cat(outs, dim=2)
+        if frame_mask is not None:
+            x_out = x_out * frame_mask[:, None, :, None]
+        return x_out.permute(0, 2, 3, 1).reshape(B, N, C)
+
+
+class CachedGLUMBConvTemp(GLUMBConvTemp):
+    """basic_modules.py:357-399.  Streaming form: the left context of the temporal conv comes from
+    the last slot of ``kv_cache`` (the previous chunk's last frames, saved un-convolved)."""
+
+    def forward(self, x, HW=None, save_kv_cache=False, kv_cache=None, **kwargs):
+        B, N, C = x.shape
+        x_reshaped = self._spatial_bcthw(x, HW)
+        pad = self.t_conv.kernel_size[0] // 2
+        x_in, padded = x_reshaped, 0
+        if kv_cache is not None:
+            if kv_cache[-1] is not None:
+                x_in = torch.cat([kv_cache[-1][:, :, -pad:], x_reshaped], dim=2)
+                padded = x_in.shape[2] - x_reshaped.shape[2]
+            if save_kv_cache:
+                kv_cache[-1] = x_reshaped[:, :, -pad:, :].detach().clone()
+        x_out = x_reshaped + self.t_conv(x_in)[:, :, padded:]
+        x_out = x_out.permute(0, 2, 3, 1).reshape(B, N, C)
+        if kv_cache is not None:
+            return x_out, kv_cache
+        return x_out
+
+
 # --------------------------------------------------------------------------
 # A14: cross attention (SDPA branch), A7: the block
 # --------------------------------------------------------------------------

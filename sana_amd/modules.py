@@ -431,6 +431,97 @@ class GLUMBConv(nn.Module):
         return self
 
 
+class GLUMBConvTemp(GLUMBConv):
+    """Mix-FFN per frame plus a residual temporal conv (reference: basic_modules.py:200-264):
+    ``x + t_conv(x)`` with ``t_conv`` a (t, 1) convolution over frames that mixes all channels,
+    zero-initialised.  The per-frame part runs the HIP kernels; the temporal conv stays a stock op
+    (it is outside the hot path), applied to a channels-last view of the token-major buffer."""
+
+    def __init__(self, in_features: int, hidden_features: int, out_feature=None, kernel_size=3, stride=1,
+                 padding=None, use_bias=False, norm=(None, None, None), act=("silu", "silu", None), t_kernel_size=3):
+        super().__init__(in_features, hidden_features, out_feature=out_feature, kernel_size=kernel_size,
+                         stride=stride, padding=padding, use_bias=use_bias, norm=norm, act=act)
+        out_feature = out_feature or in_features
+        self.t_conv = nn.Conv2d(out_feature, out_feature, kernel_size=(t_kernel_size, 1), stride=1,
+                                padding=(t_kernel_size // 2, 0), bias=False)
+        nn.init.zeros_(self.t_conv.weight)
+
+    def _spatial_bcthw(self, x: torch.Tensor, HW) -> torch.Tensor:
+        """tokens [B, N, C] -> the Mix-FFN output as a (B, C, T, H*W) view of its token-major buffer."""
+        if HW is None or len(HW) != 3:
+            raise ValueError("HW must be a tuple of (T, H, W)")
+        B, N, C = x.shape
+        T, H, W = HW
+        y = super().forward_gated(x, HW, None, None)          # [B, N, C_out], token-major
+        return y.view(B, T, H * W, y.shape[-1]).permute(0, 3, 1, 2)
+
+    @staticmethod
+    def _tokens(x_bcthw: torch.Tensor) -> torch.Tensor:
+        B, C, T, P = x_bcthw.shape
+        return x_bcthw.permute(0, 2, 3, 1).reshape(B, T * P, C)
+
+    def forward(self, x: torch.Tensor, HW=None, **kwargs) -> torch.Tensor:
+        B = x.shape[0]
+        xr = self._spatial_bcthw(x, HW)
+        frame_mask = kwargs.get("frame_valid_mask", None)
+        if frame_mask is not None:
+            frame_mask = frame_mask.reshape(B, HW[0]).to(xr)
+            xr = xr * frame_mask[:, None, :, None]
+        out = xr + self.t_conv(xr)
+        if frame_mask is not None:
+            out = out * frame_mask[:, None, :, None]
+        return self._tokens(out)
+
+
+class ChunkGLUMBConvTemp(GLUMBConvTemp):
+    """Chunked temporal conv (reference: basic_modules.py:267-354, single GPU): every chunk of frames
+    sees the tail of the previous chunk on its left and zeros on its right."""
+
+    def forward(self, x: torch.Tensor, HW=None, chunk_index=None, **kwargs) -> torch.Tensor:
+        if chunk_index is None:
+            chunk_index = [0]
+        B = x.shape[0]
+        xr = self._spatial_bcthw(x, HW)
+        T = HW[0]
+        frame_mask = kwargs.get("frame_valid_mask")
+        if frame_mask is not None:
+            frame_mask = frame_mask.reshape(B, T).to(xr)
+            xr = xr * frame_mask[:, None, :, None]
+        pad = self.t_conv.kernel_size[0] // 2
+        bounds = sorted({0, *(int(i) for i in chunk_index if 0 < int(i) < T), T})
+        zeros = xr.new_zeros(B, xr.shape[1], pad, xr.shape[3])
+        outs = []
+        for a, b in zip(bounds[:-1], bounds[1:]):
+            lo = max(a - pad, 0) if a > 0 else a
+            seg = torch.cat([xr[:, :, lo:b], zeros], dim=2)
+            outs.append(self.t_conv(seg)[:, :, a - lo:a - lo + (b - a)])
+        out = xr + torch.cat(outs, dim=2)
+        if frame_mask is not None:
+            out = out * frame_mask[:, None, :, None]
+        return self._tokens(out)
+
+
+class CachedGLUMBConvTemp(GLUMBConvTemp):
+    """Streaming temporal conv (reference: basic_modules.py:357-399): the left context is the last
+    slot of ``kv_cache`` (the previous chunk's last frames, saved un-convolved when
+    ``save_kv_cache``); returns ``(out, kv_cache)`` when a cache list is passed."""
+
+    def forward(self, x: torch.Tensor, HW=None, save_kv_cache=False, kv_cache=None, **kwargs):
+        xr = self._spatial_bcthw(x, HW)
+        pad = self.t_conv.kernel_size[0] // 2
+        x_in, padded = xr, 0
+        if kv_cache is not None:
+            if kv_cache[-1] is not None:
+                x_in = torch.cat([kv_cache[-1][:, :, -pad:].to(xr), xr], dim=2)
+                padded = x_in.shape[2] - xr.shape[2]
+            if save_kv_cache:
+                kv_cache[-1] = xr[:, :, -pad:, :].detach().clone()
+        out = self._tokens(xr + self.t_conv(x_in)[:, :, padded:])
+        if kv_cache is not None:
+            return out, kv_cache
+        return out
+
+
 # ------------------------------------------------------------------ the block
 
 

@@ -167,3 +167,43 @@ def test_fp16_model_uses_library_gemm_and_hip_attention(cuda):
         ref = ob.double()(x.double(), y.double(), t.double(), HW=HW)
         out = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
     assert rel_l2(out.cpu(), ref) <= 2e-3
+
+
+def _temp_pair(name, C, Hd, seed):
+    om = getattr(O, name)(C, Hd, use_bias=(True, True, False))
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for n, p in om.named_parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * (0.05 if n.endswith("bias") else 0.25 / p[0].numel() ** 0.5 * 2))
+    om = om.bfloat16()
+    hm = getattr(S, name)(C, Hd, use_bias=(True, True, False)).bfloat16()
+    assert list(hm.state_dict()) == list(om.state_dict())
+    hm.load_state_dict(om.state_dict(), strict=True)
+    return om, hm
+
+
+def test_temporal_mix_ffn_variants(cuda):
+    """GLUMBConvTemp / ChunkGLUMBConvTemp against the fp64 oracle, and the cached stream against the chunked call."""
+    C, Hd, (T, H, W), B = 96, 240, (6, 5, 7), 2
+    P = H * W
+    x = torch.randn(B, T * P, C, generator=torch.Generator().manual_seed(11)).bfloat16()
+    with torch.no_grad():
+        om, hm = _temp_pair("GLUMBConvTemp", C, Hd, 1)
+        hm = hm.to(cuda)
+        check(hm(x.to(cuda), HW=(T, H, W)), _ref64(om, x, HW=(T, H, W)), "GLUMBConvTemp")
+        mask = torch.ones(B, T)
+        mask[:, 4:] = 0
+        check(hm(x.to(cuda), HW=(T, H, W), frame_valid_mask=mask.to(cuda)),
+              _ref64(om, x, HW=(T, H, W), frame_valid_mask=mask), "GLUMBConvTemp masked")
+        om, hm = _temp_pair("ChunkGLUMBConvTemp", C, Hd, 2)
+        hm = hm.to(cuda)
+        full = hm(x.to(cuda), HW=(T, H, W), chunk_index=[0, 1, 4])
+        check(full, _ref64(om, x, HW=(T, H, W), chunk_index=[0, 1, 4]), "ChunkGLUMBConvTemp")
+        cm = S.CachedGLUMBConvTemp(C, Hd, use_bias=(True, True, False)).bfloat16()
+        cm.load_state_dict(om.state_dict(), strict=True)
+        cm = cm.to(cuda)
+        cache, outs = [None, None, None], []
+        for a, b in ((0, 1), (1, 4), (4, 6)):
+            o, cache = cm(x[:, a * P:b * P].to(cuda), HW=(b - a, H, W), save_kv_cache=True, kv_cache=cache)
+            outs.append(o)
+        assert (torch.cat(outs, 1).float() - full.float()).abs().max().item() <= 2 ** -6

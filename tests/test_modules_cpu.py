@@ -11,7 +11,8 @@ from oracle import sana_oracle as O
 
 
 @pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention", "LiteLAReLURope",
-                                  "CachedCausalAttention"])
+                                  "CachedCausalAttention", "GLUMBConvTemp", "ChunkGLUMBConvTemp",
+                                  "CachedGLUMBConvTemp"])
 def test_constructor_and_forward_signatures_match(name):
     a, b = getattr(S, name), getattr(O, name)
     pa = list(inspect.signature(a.__init__).parameters)

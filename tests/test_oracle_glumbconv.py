@@ -107,3 +107,73 @@ def test_bf16_rounding_points():
     # identical up to fp32 accumulation order inside the library GEMM/conv: at most an ulp of bf16 here and there
     assert err <= 2 ** -7 * ref.abs().max().item(), err
     assert ((y.float() - ref).norm() / ref.norm()).item() < 2e-3
+
+
+# ---------------------------------------------------------------- temporal variants (basic_modules.py:200-399)
+
+def _temp(cls, C, Hd, seed):
+    torch.manual_seed(seed)
+    m = cls(C, Hd, use_bias=(True, True, False)).double()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(0, 0.3)
+    return m
+
+
+def test_temporal_conv_is_zero_initialised_and_then_the_module_is_the_plain_mix_ffn():
+    C, Hd, T, Hh, Ww = 8, 20, 3, 2, 5
+    torch.manual_seed(0)
+    m = O.GLUMBConvTemp(C, Hd, use_bias=(True, True, False)).double()
+    assert m.t_conv.weight.abs().max().item() == 0.0 and m.t_conv.bias is None
+    plain = O.GLUMBConv(C, Hd, use_bias=(True, True, False)).double()
+    plain.load_state_dict({k: v for k, v in m.state_dict().items() if not k.startswith("t_conv")})
+    x = torch.randn(2, T * Hh * Ww, C, dtype=torch.float64)
+    torch.testing.assert_close(m(x, HW=(T, Hh, Ww)), plain(x, HW=(T, Hh, Ww)), rtol=0, atol=0)
+
+
+def test_temporal_conv_against_explicit_loops():
+    """out[b, t, p, :] = y[b, t, p, :] + sum_dt W[:, :, dt] y[b, t + dt - 1, p, :] with zero frames outside."""
+    C, Hd, T, Hh, Ww = 4, 6, 4, 2, 3
+    m = _temp(O.GLUMBConvTemp, C, Hd, 1)
+    x = torch.randn(2, T * Hh * Ww, C, dtype=torch.float64)
+    plain = O.GLUMBConv(C, Hd, use_bias=(True, True, False)).double()
+    plain.load_state_dict({k: v for k, v in m.state_dict().items() if not k.startswith("t_conv")})
+    y = plain(x, HW=(T, Hh, Ww)).view(2, T, Hh * Ww, C)
+    Wt = m.t_conv.weight[:, :, :, 0]   # [co, ci, dt]
+    ref = y.clone()
+    for t in range(T):
+        for dt in range(3):
+            ts = t + dt - 1
+            if 0 <= ts < T:
+                ref[:, t] += y[:, ts] @ Wt[:, :, dt].T
+    torch.testing.assert_close(m(x, HW=(T, Hh, Ww)), ref.view(2, -1, C), rtol=1e-12, atol=1e-12)
+
+
+def test_cached_stream_equals_chunked_temporal_conv_and_frame_mask():
+    C, Hd, T, Hh, Ww = 6, 10, 7, 3, 2
+    P = Hh * Ww
+    chunked = _temp(O.ChunkGLUMBConvTemp, C, Hd, 2)
+    cached = O.CachedGLUMBConvTemp(C, Hd, use_bias=(True, True, False)).double()
+    cached.load_state_dict(chunked.state_dict())
+    x = torch.randn(2, T * P, C, dtype=torch.float64)
+    bounds = [0, 2, 3, 7]
+    full = chunked(x, HW=(T, Hh, Ww), chunk_index=bounds[:-1])
+    cache, outs = [None, None, None], []
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        o, cache = cached(x[:, a * P:b * P], HW=(b - a, Hh, Ww), save_kv_cache=True, kv_cache=cache)
+        assert cache[0] is None and cache[1] is None and cache[-1].shape == (2, C, 1, P)
+        outs.append(o)
+    torch.testing.assert_close(torch.cat(outs, 1), full, rtol=1e-12, atol=1e-12)
+    # one chunk = the unchunked module; a chunk boundary changes only the frame in front of it
+    whole = O.GLUMBConvTemp(C, Hd, use_bias=(True, True, False)).double()
+    whole.load_state_dict(chunked.state_dict())
+    w = whole(x, HW=(T, Hh, Ww))
+    torch.testing.assert_close(chunked(x, HW=(T, Hh, Ww), chunk_index=[0]), w, rtol=1e-12, atol=1e-12)
+    diff = (full - w).view(2, T, P, C).abs().amax(dim=(0, 2, 3))
+    assert (diff[[1, 2]] > 1e-6).all() and diff[[0, 3, 4, 5, 6]].max().item() < 1e-12
+    # masked frames are zero on the way in and on the way out
+    mask = torch.ones(2, T)
+    mask[:, 5:] = 0
+    wm = whole(x, HW=(T, Hh, Ww), frame_valid_mask=mask).view(2, T, P, C)
+    assert wm[:, 5:].abs().max().item() == 0.0
+    torch.testing.assert_close(wm[:, :4], w.view(2, T, P, C)[:, :4], rtol=1e-12, atol=1e-12)
