@@ -206,6 +206,57 @@ class LiteLA(_AttentionBase):
 # --------------------------------------------------------------------------
 
 
+class SelfAttnProcessorLiteLA:
+    """diffusion/model/nets/sana_blocks.py:677-717: LiteLA.forward restated on the module's parts
+    (``qkv``, ``q_norm``, ``k_norm``, ``dim``, ``kernel_func``, ``attn_matmul``, ``proj``)."""
+
+    def __init__(self, attn):
+        self.attn = attn
+
+    def _attend(self, x, rotary_emb):
+        a = self.attn
+        B, N, C = x.shape
+        qkv = a.qkv(x).reshape(B, N, 3, C)
+        q, k, v = qkv.unbind(2)
+        dtype = q.dtype
+        q = a.q_norm(q).transpose(-1, -2).reshape(B, C // a.dim, a.dim, N)
+        k = a.k_norm(k).transpose(-1, -2).reshape(B, C // a.dim, a.dim, N)
+        v = v.transpose(-1, -2).reshape(B, C // a.dim, a.dim, N)
+        if rotary_emb is not None:
+            q, k = rotary_real(q, rotary_emb), rotary_real(k, rotary_emb)
+        q, k = a.kernel_func(q), a.kernel_func(k)
+        out = a.attn_matmul(q, k.transpose(-1, -2), v).to(dtype)
+        return a.proj(out.view(B, C, N).permute(0, 2, 1))
+
+    def _identity(self, x_ptb):
+        """:615-622: the perturbed path replaces the attention by the identity: proj(v_linear(x))."""
+        a = self.attn
+        C = x_ptb.shape[-1]
+        y = torch.matmul(x_ptb, a.qkv.weight[C * 2:C * 3, :].t())
+        if a.qkv.bias is not None:
+            y = y + a.qkv.bias[C * 2:C * 3]
+        return a.proj(y.to(x_ptb.dtype))
+
+    def __call__(self, x, mask=None, HW=None, rotary_emb=None, block_id=None, block_mask=None, **kwargs):
+        return self._attend(x, rotary_emb)
+
+
+class PAGIdentitySelfAttnProcessorLiteLA(SelfAttnProcessorLiteLA):
+    """sana_blocks.py:627-674: batch = [cond | perturbed]."""
+
+    def __call__(self, x, mask=None, HW=None, rotary_emb=None, block_id=None, block_mask=None, **kwargs):
+        x_org, x_ptb = x.chunk(2)
+        return torch.cat([self._attend(x_org, rotary_emb), self._identity(x_ptb)])
+
+
+class PAGCFGIdentitySelfAttnProcessorLiteLA(SelfAttnProcessorLiteLA):
+    """sana_blocks.py:575-624: batch = [uncond | cond | perturbed]."""
+
+    def __call__(self, x, mask=None, HW=None, rotary_emb=None, block_id=None, block_mask=None, **kwargs):
+        x_uncond, x_org, x_ptb = x.chunk(3)
+        return torch.cat([self._attend(torch.cat([x_uncond, x_org]), rotary_emb), self._identity(x_ptb)])
+
+
 class LiteLAReLURope(_AttentionBase):
     """diffusion/model/nets/sana_blocks.py:304-388."""
 

@@ -634,7 +634,11 @@ class SanaMSBlock(nn.Module):
         if x.is_cuda and x.dtype == torch.bfloat16 and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
             # fused seams: LayerNorm + modulate in one kernel, gate * out + residual in the GEMM epilogue
             h = ops.layernorm_modulate(x, scale_msa, shift_msa, self.norm1.eps)
-            x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
+            if "forward" in self.attn.__dict__:
+                # a guidance processor was patched over attn.forward (dpm_solver.py:486-524): call it
+                x = x + gate_msa * self.attn(h, HW=HW, rotary_emb=image_rotary_emb)
+            else:
+                x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
             x = x + self.cross_attn(x, y, mask)
             h = ops.layernorm_modulate(x, scale_mlp, shift_mlp, self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)

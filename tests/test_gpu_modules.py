@@ -207,3 +207,32 @@ def test_temporal_mix_ffn_variants(cuda):
             o, cache = cm(x[:, a * P:b * P].to(cuda), HW=(b - a, H, W), save_kv_cache=True, kv_cache=cache)
             outs.append(o)
         assert (torch.cat(outs, 1).float() - full.float()).abs().max().item() <= 2 ** -6
+
+
+@pytest.mark.parametrize("mode", ["pag", "pag_cfg"])
+def test_guidance_processor_patched_over_attn_forward(cuda, mode):
+    """The sampler's way of enabling perturbed-attention guidance: patch a processor over
+    ``block.attn.forward`` (dpm_solver.py:486-524), run the tripled / doubled batch, restore."""
+    from sana_amd import pag
+    C, heads, HW = 96, 4, (6, 8)
+    N = HW[0] * HW[1]
+    ob, hb = _pair(C, heads, seed=5)
+    hb = hb.to(cuda)
+    nb = 2 if mode == "pag" else 3
+    x, y, t = (a.bfloat16() for a in O.block_inputs(nb, N, C, n_text=20, seed=5))
+    name = "PAGIdentitySelfAttnProcessorLiteLA" if mode == "pag" else "PAGCFGIdentitySelfAttnProcessorLiteLA"
+    with torch.no_grad():
+        import copy
+        o64 = copy.deepcopy(ob).double()
+        o64.attn.forward = getattr(O, name)(o64.attn)
+        ref = o64(x.double(), y.double(), t.double(), HW=HW)
+        plain = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
+        hb.attn.forward = getattr(pag, name)(hb.attn)
+        out = hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)
+        check(out, ref, name, block=True)
+        # the unperturbed part is what the block computes without the processor; the perturbed part is not
+        assert (out[:nb - 1].float() - plain[:nb - 1].float()).abs().max().item() <= 2 ** -5
+        assert (out[nb - 1:].float() - plain[nb - 1:].float()).abs().max().item() > 1e-2
+        hb.attn.forward = pag.SelfAttnProcessorLiteLA(hb.attn)     # what the sampler leaves behind
+        assert torch.equal(hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW), plain) or \
+            (hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW).float() - plain.float()).abs().max().item() <= 2 ** -5

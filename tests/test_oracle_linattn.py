@@ -152,3 +152,25 @@ def test_rotary_real_is_a_rotation_of_channel_pairs():
     # and the complex form used by the ReLU->RoPE family agrees with it
     y2 = O.rotary_complex(x, torch.polar(torch.ones_like(theta), theta)[None, None])
     torch.testing.assert_close(y2, ref, rtol=1e-12, atol=1e-12)
+
+
+def test_guidance_processors_restate_the_attention_forward():
+    """SelfAttnProcessorLiteLA is LiteLA.forward on the module's parts; the PAG processors run it on the
+    unperturbed part of the batch and proj(v_linear(x)) (identity attention) on the perturbed part
+    (sana_blocks.py:575-717)."""
+    torch.manual_seed(0)
+    C, N = 64, 24
+    attn = O.LiteLA(C, C, heads=2, eps=1e-8, qk_norm=True).double()
+    with torch.no_grad():
+        for p in attn.parameters():
+            p.normal_(0, 0.2)
+    x = torch.randn(3, N, C, dtype=torch.float64)
+    plain = attn(x)
+    torch.testing.assert_close(O.SelfAttnProcessorLiteLA(attn)(x), plain, rtol=1e-12, atol=1e-12)
+    v_only = attn.proj(x @ attn.qkv.weight[2 * C:].T)
+    out3 = O.PAGCFGIdentitySelfAttnProcessorLiteLA(attn)(x)
+    torch.testing.assert_close(out3[:2], plain[:2], rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(out3[2:], v_only[2:], rtol=1e-12, atol=1e-12)
+    out2 = O.PAGIdentitySelfAttnProcessorLiteLA(attn)(x[:2])
+    torch.testing.assert_close(out2[:1], plain[:1], rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(out2[1:], v_only[1:2], rtol=1e-12, atol=1e-12)
