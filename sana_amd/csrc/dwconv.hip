@@ -12,6 +12,8 @@
 // once; the next row's loads are in flight while the current row is computed.
 // The four waves of a workgroup take four adjacent strips so that the halo
 // columns hit in the CU's vector L1.
+#include <type_traits>
+
 #include "common.h"
 
 #ifndef SANA_DW_MINWAVES
@@ -223,6 +225,170 @@ __global__ __launch_bounds__(256) void dwconv_gate_kernel(const void* __restrict
   }
 }
 
+// ----------------------------------------------------------------------------
+// 16-bit io: the taps run on packed dot products.  The window keeps, per row, channel and column j,
+// the PAIR (x[j], x[j+1]) as two 16-bit values in one register (built with one byte-permute from the
+// loaded channel-pair words of pixels j and j+1), and a 3-tap row is
+//   dot2(pair[j], (w0, w1)) + dot2(pair[j+2], (w2, 0))
+// with fp32 accumulation: 6 instructions per output channel instead of 9 FMAs, and no unpacking of
+// the inputs at all (products of 16-bit values are exact in fp32).
+// ----------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float dot2_16(uint32_t a, uint32_t b, float c);
+template <>
+__device__ __forceinline__ float dot2_16<BF16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+template <>
+__device__ __forceinline__ float dot2_16<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+}
+
+template <typename T, int TW, bool ROUND>
+__global__ __launch_bounds__(256) void dwconv_gate16_kernel(const void* __restrict__ u, const void* __restrict__ w,
+                                                            const void* __restrict__ bias, void* __restrict__ y,
+                                                            int H, int W, int Ch, int R, int xgroups) {
+  typedef Pair<T> P;
+  constexpr int ESZ = 2;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  // Workgroups go round-robin to the 8 XCDs (own L2 each) in launch order, x fastest.  All slabs of a
+  // tile are launched together, so the eight XCDs read the same pixels at the same time -- whole
+  // contiguous 2*Ch-element pixel rows, which is what DRAM pages like -- and WHICH slab a workgroup
+  // takes is chosen from the XCD it landed on: slab m*q + j for the j-th workgroup of XCD m in this
+  // grid row (q = slabs / 8), the slabs left over going to whoever has a (q+1)-th workgroup.  A slab
+  // below 8*q is then always served by the same L2, which is where neighbouring tiles find their
+  // shared halo rows and columns.  (Giving each XCD its own slabs AND its own run of neighbouring
+  // tiles lowers the fetch size further but was measured slower: it breaks up the pixel rows.)
+  int slab;
+  {
+    const int nsl = gridDim.x, q = nsl >> 3;
+    const int xcd = (blockIdx.x + nsl * (blockIdx.y + gridDim.y * blockIdx.z)) & 7, j = blockIdx.x >> 3;
+    slab = j < q ? xcd * q + j : 8 * q + (blockIdx.x & 7);
+  }
+  const int bt = blockIdx.z;
+  const int xg = blockIdx.y % xgroups, band = blockIdx.y / xgroups;
+  const int c = slab * 128 + 2 * lane;
+  const int x0 = (xg * 4 + wave) * TW;
+  if (c >= Ch || x0 >= W) return;  // no barriers in this kernel
+  const int y0 = band * R, y1 = min(H, y0 + R);
+  const int64_t C2 = 2 * (int64_t)Ch;
+  const int64_t img = (int64_t)bt * H * W;
+  const uint32_t lane_b = (uint32_t)(2 * lane) * ESZ;
+  const char* ub = static_cast<const char*>(u) + (int64_t)slab * 128 * ESZ;
+  char* yb = static_cast<char*>(y) + (int64_t)slab * 128 * ESZ;
+  const int64_t g_off = (int64_t)Ch * ESZ;
+
+  // taps of the four channels of this lane [a0, a1, g0, g1], per filter row: (w0, w1) and (w2, 0) packed
+  uint32_t w01[4][3], w2z[4][3];
+  float bs[4];
+  const uint16_t* wp = static_cast<const uint16_t*>(w);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int64_t ch = c + (q & 1) + (q >> 1) * Ch;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      w01[q][r] = (uint32_t)wp[ch * 9 + 3 * r] | ((uint32_t)wp[ch * 9 + 3 * r + 1] << 16);
+      w2z[q][r] = (uint32_t)wp[ch * 9 + 3 * r + 2];
+    }
+    bs[q] = bias ? P::one(bias, ch) : 0.f;
+  }
+
+  uint32_t win[3][TW + 2][4];  // [row][column j][channel]: (x[j], x[j+1]); the last column pairs with 0
+  uint32_t ra[TW + 2], rg[TW + 2];
+  bool rowok = false;
+  const bool cols_inside = x0 >= 1 && x0 + TW <= W - 1;
+
+  // Buffer loads: the image (this slab's view of it) is one buffer resource in scalar registers, a pixel
+  // is a scalar byte offset and the lane's channel pair the vector offset, so no vector ALU work goes
+  // into addresses.  One image is below 2 GiB (the host checks).  Addresses are always valid
+  // (clamped); the resource's own range check is left wide open.
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(ub + img * C2 * ESZ), 0, -1, 0x00020000);
+  const int pix_b = (int)(C2 * ESZ), g_off32 = (int)g_off;
+  auto issue = [&](int yy) {
+    rowok = yy >= 0 && yy < H && yy <= y1;
+    const int yc = min(max(yy, 0), H - 1);
+#pragma unroll
+    for (int i = 0; i < TW + 2; ++i) {
+      const int xc = min(max(x0 - 1 + i, 0), W - 1);
+      const int soff = (yc * W + xc) * pix_b;
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, soff, 0);
+      rg[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, soff + g_off32, 0);
+    }
+  };
+  auto commit = [&](uint32_t (&row)[TW + 2][4]) {
+    if (!(rowok && cols_inside)) {  // out-of-image taps are zero
+#pragma unroll
+      for (int i = 0; i < TW + 2; ++i) {
+        const bool ok = rowok && (x0 - 1 + i >= 0) && (x0 - 1 + i < W);
+        ra[i] = ok ? ra[i] : 0u;
+        rg[i] = ok ? rg[i] : 0u;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TW + 2; ++i) {
+      const uint32_t na = i + 1 < TW + 2 ? ra[i + 1] : 0u, ng = i + 1 < TW + 2 ? rg[i + 1] : 0u;
+      row[i][0] = __builtin_amdgcn_perm(na, ra[i], 0x05040100u);  // low halves: channel c of pixels i, i+1
+      row[i][1] = __builtin_amdgcn_perm(na, ra[i], 0x07060302u);  // high halves: channel c+1
+      row[i][2] = __builtin_amdgcn_perm(ng, rg[i], 0x05040100u);
+      row[i][3] = __builtin_amdgcn_perm(ng, rg[i], 0x07060302u);
+    }
+  };
+  auto compute = [&](int yo, const uint32_t (&top)[TW + 2][4], const uint32_t (&mid)[TW + 2][4],
+                     const uint32_t (&bot)[TW + 2][4]) {
+    char* orow = yb + (img + (int64_t)yo * W + x0) * Ch * ESZ;
+#pragma unroll
+    for (int x = 0; x < TW; ++x) {
+      if (x0 + x >= W) break;
+      float acc[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float a = bs[q];
+        a = dot2_16<T>(top[x][q], w01[q][0], a);
+        a = dot2_16<T>(top[x + 2][q], w2z[q][0], a);
+        a = dot2_16<T>(mid[x][q], w01[q][1], a);
+        a = dot2_16<T>(mid[x + 2][q], w2z[q][1], a);
+        a = dot2_16<T>(bot[x][q], w01[q][2], a);
+        a = dot2_16<T>(bot[x + 2][q], w2z[q][2], a);
+        acc[q] = a;
+      }
+      float o0, o1;
+      if (ROUND) {
+        float a0, a1, g0, g1, s0, s1;
+        P::rnd2(acc[0], acc[1], a0, a1);
+        P::rnd2(acc[2], acc[3], g0, g1);
+        P::rnd2(silu_f32(g0), silu_f32(g1), s0, s1);
+        o0 = a0 * s0;
+        o1 = a1 * s1;
+      } else {
+        o0 = acc[0] * silu_f32(acc[2]);
+        o1 = acc[1] * silu_f32(acc[3]);
+      }
+      *reinterpret_cast<uint32_t*>(orow + (int64_t)x * Ch * ESZ + lane_b) = P::pack(o0, o1);
+    }
+  };
+
+  issue(y0 - 1);
+  commit(win[0]);
+  issue(y0);
+  commit(win[1]);
+  issue(y0 + 1);
+  for (int yo = y0; yo < y1; yo += 3) {
+    commit(win[2]);
+    issue(yo + 2);
+    compute(yo, win[0], win[1], win[2]);
+    if (yo + 1 >= y1) break;
+    commit(win[0]);
+    issue(yo + 3);
+    compute(yo + 1, win[1], win[2], win[0]);
+    if (yo + 2 >= y1) break;
+    commit(win[1]);
+    issue(yo + 4);
+    compute(yo + 2, win[2], win[0], win[1]);
+  }
+}
+
 template <typename T, int TW>
 int launch(const void* u, const void* w, const void* bias, void* y, int BT, int H, int W, int Ch, int round_ref,
            hipStream_t s) {
@@ -236,10 +402,24 @@ int launch(const void* u, const void* w, const void* bias, void* y, int BT, int 
   const int bands = (H + R - 1) / R;
   if ((int64_t)xgroups * bands > 65535 || BT > 65535) return SANA_ERR_SHAPE;
   dim3 grid(slabs, xgroups * bands, BT);
-  if (round_ref)
-    hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, true>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
-  else
-    hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, false>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+  // the 16-bit kernel addresses pixels of one image with 32-bit offsets
+  const bool small_image = (int64_t)H * W * 2 * Ch * 2 < ((int64_t)1 << 31);
+  bool launched = false;
+  if constexpr (!std::is_same<T, float>::value) {
+    if (small_image) {
+      if (round_ref)
+        hipLaunchKernelGGL((dwconv_gate16_kernel<T, TW, true>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+      else
+        hipLaunchKernelGGL((dwconv_gate16_kernel<T, TW, false>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+      launched = true;
+    }
+  }
+  if (!launched) {
+    if (round_ref)
+      hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, true>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+    else
+      hipLaunchKernelGGL((dwconv_gate_kernel<T, TW, false>), grid, dim3(256), 0, s, u, w, bias, y, H, W, Ch, R, xgroups);
+  }
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
