@@ -306,15 +306,16 @@ __global__ __launch_bounds__(256) void dwconv_gate16_kernel(const void* __restri
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(ub + img * C2 * ESZ), 0, -1, 0x00020000);
   const int pix_b = (int)(C2 * ESZ), g_off32 = (int)g_off;
+  int coff[TW + 2];  // byte offsets of the (clamped) footprint columns inside a row: scalar registers
+#pragma unroll
+  for (int i = 0; i < TW + 2; ++i) coff[i] = min(max(x0 - 1 + i, 0), W - 1) * pix_b;
   auto issue = [&](int yy) {
-    rowok = yy >= 0 && yy < H && yy <= y1;
-    const int yc = min(max(yy, 0), H - 1);
+    rowok = yy >= 0 && yy < H && yy <= y1;  // rows past the band's lower halo are never used
+    const int rowb = min(max(yy, 0), H - 1) * W * pix_b;
 #pragma unroll
     for (int i = 0; i < TW + 2; ++i) {
-      const int xc = min(max(x0 - 1 + i, 0), W - 1);
-      const int soff = (yc * W + xc) * pix_b;
-      ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, soff, 0);
-      rg[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, soff + g_off32, 0);
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, rowb + coff[i], 0);
+      rg[i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_b, rowb + coff[i] + g_off32, 0);
     }
   };
   auto commit = [&](uint32_t (&row)[TW + 2][4]) {
