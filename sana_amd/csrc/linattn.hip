@@ -360,15 +360,25 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     const uint16_t* __restrict__ Q, const float* __restrict__ state, void* __restrict__ out,
     const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int wg_tokens,
     int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, float eps,
-    const QkPre pre) {
+    const QkPre pre, int xranges, int ngroups) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pairs = (h + 1) >> 1;
   const int pgroups = (pairs + 3) >> 2;
-  const int b = blockIdx.z / pgroups, p = (blockIdx.z % pgroups) * 4 + wave;
+  // 3-D grid (token range, chunk, batch x head group), or -- with many (chunk, batch, head group)
+  // combinations -- a 1-D grid dealt so that all token ranges of one combination run on the same XCD
+  // (workgroup ids go round-robin to the 8 XCDs): their common state is then fetched into one L2 only.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if (ngroups > 0) {
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int grp = xcd + 8 * (idx / xranges);
+    if (grp >= ngroups) return;  // no barriers below
+    bx = idx % xranges, by = grp % n_chunks, bz = grp / n_chunks;
+  }
+  const int b = bz / pgroups, p = (bz % pgroups) * 4 + wave;
   if (p >= pairs) return;  // no barriers below
-  const int c = blockIdx.y;
+  const int c = by;
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
-  const int t0 = cr.begin + blockIdx.x * wg_tokens;
+  const int t0 = cr.begin + bx * wg_tokens;
   const int t1 = min(cr.end, t0 + wg_tokens);
   if (t0 >= t1) return;
   const int n = lane & 15, g = lane >> 4;
@@ -401,7 +411,7 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     for (int hh = 0; hh < 2; ++hh)
       if (hh < nheads) qw[hh] = *reinterpret_cast<const u32x4_t*>(pre.weight + p * 64 + hh * D + 8 * g);
   }
-  constexpr int U = SANA_LA_APPLY_U;  // 16-token steps in flight
+  constexpr int U = PRE ? SANA_LA_APPLY_U / 2 : SANA_LA_APPLY_U;  // 16-token steps in flight (registers: PRE carries the rope factors)
   for (int t = t0; t < t1; t += 16 * U) {
     u32x4_t qf[U][2];
     float rin[U];
@@ -751,10 +761,16 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
   if (io_dtype == SANA_DT_BF16) {
     const int pairs = (h + 1) / 2;
     dim3 grid(gx, n_chunks, B * ((pairs + 3) / 4));
+    // many distinct states (chunk-causal video shapes): keep the readers of one state on one XCD
+    int ngroups = n_chunks * B * ((pairs + 3) / 4);
+    if (ngroups >= 64 && (int64_t)((ngroups + 7) / 8) * 8 * gx < 0x7fffffff)
+      grid = dim3((unsigned)((ngroups + 7) / 8 * 8) * gx, 1, 1);
+    else
+      ngroups = 0;
 #define SANA_APPLY(F32, PRE)                                                                                   \
   hipLaunchKernelGGL((linattn_apply_bf16_kernel<F32, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(q), \
                      state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,     \
-                     o_stride_n, eps, pre)
+                     o_stride_n, eps, pre, (int)gx, ngroups)
     if (out_dtype == SANA_DT_F32) {
       if (use_pre) SANA_APPLY(true, true);
       else SANA_APPLY(true, false);
