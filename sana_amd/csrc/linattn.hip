@@ -411,20 +411,38 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     for (int hh = 0; hh < 2; ++hh)
       if (hh < nheads) qw[hh] = *reinterpret_cast<const u32x4_t*>(pre.weight + p * 64 + hh * D + 8 * g);
   }
-  constexpr int U = PRE ? SANA_LA_APPLY_U / 2 : SANA_LA_APPLY_U;  // 16-token steps in flight (registers: PRE carries the rope factors)
+  // Global accesses are whole 128-byte lines: lane l fetches 16-byte chunk l%8 of token l/8 (both heads
+  // of the pair), two instructions per 16-token step, and the step goes through wave-private LDS to
+  // reach the MFMA layout (lane = token n, channel group g); results return the same way, so a store
+  // instruction writes eight full lines.  (Fetching straight in MFMA layout touches every line twice
+  // with 64-byte pieces and is bound by the L1 tag rate: 4.2 TB/s read side against 5.8 here.)
+  // LDS slot of (token n of the step, chunk c): 16 * (8n + (c ^ (n/2) % 8)): conflict-free both ways.
+  constexpr int U = PRE ? SANA_LA_APPLY_U / 2 : SANA_LA_APPLY_U;  // 16-token steps in flight
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * (SANA_LA_APPLY_U + 1) * 2048];
+  unsigned char* stage = stage_all + wave * ((SANA_LA_APPLY_U + 1) * 2048);
+  const int ld_tok = lane >> 3, ld_chunk = lane & 7;
+  const uint16_t* qrow = Q + (int64_t)b * q_stride_b + p * 64 + 8 * ld_chunk;
+  const bool ld_ok = nheads == 2 || ld_chunk < 4;   // the second head of the last pair may not exist
+  int slot_w[2], slot_r[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int tl = 8 * j + ld_tok;
+    slot_w[j] = 16 * (8 * tl + (ld_chunk ^ ((tl >> 1) & 7)));
+  }
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) slot_r[hh] = 16 * (8 * n + ((4 * hh + g) ^ ((n >> 1) & 7)));
   for (int t = t0; t < t1; t += 16 * U) {
-    u32x4_t qf[U][2];
+    u32x4_t raw[U][2];
     float rin[U];
     f32x4_t cs[U][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int tok = t + 16 * u + n;
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        qf[u][hh] = (tok < t1 && hh < nheads)
-                        ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + hh * D)
-                        : zero4;
+      for (int j = 0; j < 2; ++j) {
+        const int tok = t + 16 * u + 8 * j + ld_tok;
+        raw[u][j] = (tok < t1 && ld_ok) ? *reinterpret_cast<const u32x4_t*>(qrow + (int64_t)tok * q_stride_n) : zero4;
       }
+      const int tok = t + 16 * u + n;
       if (has_norm) rin[u] = tok < t1 ? pre.rinv[(int64_t)b * N + tok] : 0.f;
       if (has_rope) {
         const float* rp = pre.rope + ((int64_t)min(tok, t1 - 1) * 16 + g * 4) * 2;
@@ -433,11 +451,17 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
       }
     }
 #pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) *reinterpret_cast<u32x4_t*>(stage + u * 2048 + slot_w[j]) = raw[u][j];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+    unsigned char* ostage = stage + SANA_LA_APPLY_U * 2048;
+#pragma unroll
     for (int u = 0; u < U; ++u) {
       const int tok = t + 16 * u + n;
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
-        u32x4_t qd = qf[u][hh];
+        u32x4_t qd = *reinterpret_cast<const u32x4_t*>(stage + u * 2048 + slot_r[hh]);
         if (has_norm) qd = rms_scale8(qd, rin[u], qw[hh]);
         qd = relu_pk16(qd);                                              // denominator operand
         const u32x4_t qb = has_rope ? rope8(qd, cs[u][0], cs[u][1]) : qd;  // numerator operand
@@ -451,10 +475,10 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
           a = mfma_16x16x32_bf16(st[hh].a[rb][0], bop, a);
           acc[rb] = a;
         }
-        if (tok < t1 && hh < nheads) {
-          const float den = acc[2][0] + eps;
-          const int64_t o_off = (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + p * 64 + hh * D + 8 * g;
-          if (OUT_F32) {
+        const float den = acc[2][0] + eps;
+        if (OUT_F32) {
+          if (tok < t1 && hh < nheads) {
+            const int64_t o_off = (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + p * 64 + hh * D + 8 * g;
             f32x4_t o0, o1;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
@@ -464,18 +488,31 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
             float* op = reinterpret_cast<float*>(out) + o_off;
             *reinterpret_cast<f32x4_t*>(op) = o0;
             *reinterpret_cast<f32x4_t*>(op + 4) = o1;
-          } else {
-            const float inv = __builtin_amdgcn_rcpf(den);
-            u32x4_t o;
-            o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
-            o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
-            o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
-            o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
-            *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + o_off) = o;
           }
+        } else {
+          const float inv = __builtin_amdgcn_rcpf(den);
+          u32x4_t o;
+          o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
+          o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
+          o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
+          o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
+          *reinterpret_cast<u32x4_t*>(ostage + slot_r[hh]) = o;
         }
       }
+      if (!OUT_F32) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int tok_s = t + 16 * u + 8 * j + ld_tok;
+          const u32x4_t o = *reinterpret_cast<const u32x4_t*>(ostage + slot_w[j]);
+          if (tok_s < t1 && ld_ok)
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + (int64_t)b * o_stride_b +
+                                        (int64_t)tok_s * o_stride_n + p * 64 + 8 * ld_chunk) = o;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the next step overwrites
+      }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
 }
 
