@@ -319,9 +319,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 //     before they are stored, the quad reloaded after its last piece);
 //   * the only barrier sits in k-step 3 after the last store; the slots behind it
 //     read k-step 0 of the next tile.
-// Rows past M / N and k chunks past K are clamped to valid addresses: clamped
-// rows only feed outputs that are never stored, and the last k-tile runs just the
-// k-steps that exist.  Needs K % 16 == 0 and K >= 64.
+// Rows past M / N read as zero (buffer range check) and only feed outputs that are
+// never stored; the last k-tile runs just the k-steps that exist.  Needs K % 16 == 0 and K >= 64.
 // ============================================================================
 template <bool W8, int EPI, int NI>
 __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
@@ -351,8 +350,6 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // int8 W: thread -> 16-value chunk tid%4, rows tid/4 + 64*q (q < NI); dequantised on the way to LDS.
   const int g_chunk = tid & 7, g_row = tid >> 3;
   const int a_last = min(BT, M - m0) - 1, w_last = min(BCN, N - n0) - 1;  // last valid row of each tile
-  const uint16_t* Abase = A + (int64_t)m0 * lda + 8 * g_chunk;
-  const uint16_t* Wbase = static_cast<const uint16_t*>(Wv) + (int64_t)n0 * ldw + 8 * g_chunk;
   const uint32_t ulda = (uint32_t)lda, uldw = (uint32_t)ldw;
   const int a_dst0 = swz(g_row, g_chunk);                            // rows +32*q keep the key: +4096 bytes each
   const int w_dst0 = TILE_BYTES + swz(wrow_to_lds(g_row), g_chunk);  // the row permutation stays inside 32-row blocks
@@ -360,7 +357,6 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   constexpr int NQ = 8 + NWQ;
   u32x4_t rs[NQ];  // the k-tile in flight: A quads 0..7, then the W quads
   const int q_chunk = tid & 3, q_row = tid >> 2;
-  const int8_t* Qbase = static_cast<const int8_t*>(Wv) + (int64_t)n0 * ldw + 16 * q_chunk;
   const int q_dst_lo = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk);  // rows +64*q: +8192 bytes, same key
   const int q_dst_hi = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk + 1);
   float wscale[NI], woff[NI];
@@ -387,17 +383,26 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   u32x4_t fw[2][NI], fa[2][4];
 
 #define SANA_G4_PIN() __builtin_amdgcn_sched_barrier(0)
+  // Operand tiles are read with buffer loads: the tile's rows are one resource each for A and W (scalar
+  // registers), the lane's (row, k chunk) is a constant vector offset, and the quad / k-tile part of the
+  // address is scalar, so a load costs one vector add.  The resource ends with the last valid row's
+  // K-th element: rows past M / N and anything past the end of the matrix read as zero instead of
+  // faulting (k chunks past K inside the matrix read the next row: they are never multiplied).
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(A + (int64_t)m0 * lda), 0, (int)(((int64_t)a_last * lda + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * (W8 ? 1 : 2)), 0,
+      (int)(((int64_t)w_last * ldw + K) * (W8 ? 1 : 2)), 0x00020000);
+  const int voff_a = (g_row * (int)ulda + 8 * g_chunk) * 2;
+  const int voff_w = W8 ? q_row * (int)uldw + 16 * q_chunk : (g_row * (int)uldw + 8 * g_chunk) * 2;
+  const int step_a = 32 * (int)ulda * 2, step_w = W8 ? 64 * (int)uldw : 32 * (int)uldw * 2;
   auto gload = [&](int q, int k0) {
-    // row offsets are recomputed (two VALU ops) rather than held in registers
     if (q < 8) {
-      const uint32_t kk = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
-      rs[q] = *reinterpret_cast<const u32x4_t*>(Abase + ((uint32_t)min(g_row + 32 * q, a_last) * ulda + kk));
-    } else if (!W8) {
-      const uint32_t kk = (uint32_t)min(k0, K - 8 - 8 * g_chunk);
-      rs[q] = *reinterpret_cast<const u32x4_t*>(Wbase + ((uint32_t)min(g_row + 32 * (q - 8), w_last) * uldw + kk));
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff_a + (q * step_a + k0 * 2), 0, 0);
+      rs[q] = __builtin_bit_cast(u32x4_t, v);
     } else {
-      const uint32_t kk = (uint32_t)min(k0, K - 16 - 16 * q_chunk);
-      rs[q] = *reinterpret_cast<const u32x4_t*>(Qbase + ((uint32_t)min(q_row + 64 * (q - 8), w_last) * uldw + kk));
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w + ((q - 8) * step_w + k0 * (W8 ? 1 : 2)), 0, 0);
+      rs[q] = __builtin_bit_cast(u32x4_t, v);
     }
   };
   auto lstore = [&](int q, int stage) {  // A quads, bf16 W quads
