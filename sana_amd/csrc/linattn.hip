@@ -402,7 +402,6 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     }
   }
 
-  const uint16_t* qp = Q + (int64_t)b * q_stride_b + p * 64 + 8 * g;
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
   const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
   u32x4_t qw[2] = {zero4, zero4};
