@@ -492,6 +492,22 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     }
   }
 #undef SANA_G4_PIN
+  // The lane's bias values (16 consecutive channels per MFMA tile, packed) are requested here, ahead of
+  // the last k-tile, so that their latency hides behind its MFMAs.
+  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
+  u32x4_t bpk[NI][2];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg + 8 * half;  // N % 8 == 0: a chunk is in or out
+        bpk[i][half] = (ep.bias && n < N) ? *reinterpret_cast<const u32x4_t*>(ep.bias + n) : u32x4_t{0u, 0u, 0u, 0u};
+      }
+  }
+  const int o_chunk = lane & 15, o_rsub = lane >> 4;
+  const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
+  const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
   {  // last k-tile: no successor, and K % 64 may leave fewer than four k-steps
     const unsigned char* st = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
     const int steps = (K - (KT - 1) * BK) / 16;
@@ -516,23 +532,11 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
   // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
   // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
-  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
   __syncthreads();  // every wave is done with the operand tiles
   unsigned char* stg = smem + wave * 32768;
-  float bv[NI][16];
-  if (HAS_BIAS) {
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) bv[i][r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
-    }
-  }
-  const int o_chunk = lane & 15, o_rsub = lane >> 4;
-  const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
-  const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
   // Gated residual: the residual rows this lane will add are requested now, a whole epilogue ahead
-  // of their use (128 registers that the main loop no longer needs).
+  // of their use (128 registers that the main loop no longer needs; asking for them before the last
+  // k-tile makes the compiler spill).
   u32x4_t res[4][8];
   if (EPI == SANA_EPI_GATE_RES) {
 #pragma unroll
@@ -542,6 +546,18 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
         const int m = m0 + wt * 128 + 32 * j + it * 4 + o_rsub;
         if (o_live && m < M) res[j][it] = *reinterpret_cast<const u32x4_t*>(ep.res + (int64_t)m * ep.ldr + o_n);
       }
+  }
+  float bv[NI][16];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          bv[i][8 * half + 2 * e] = bf16_lo(bpk[i][half][e]);
+          bv[i][8 * half + 2 * e + 1] = bf16_hi(bpk[i][half][e]);
+        }
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
