@@ -20,6 +20,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "linattn_common.h"
 
 // tuning knobs of the bf16 apply kernel: tokens per workgroup, 16-token steps in flight per wave
 #ifndef SANA_LA_APPLY_TOKENS
@@ -35,52 +36,6 @@ namespace {
 constexpr int D = 32;
 constexpr int STATE_ELEMS = (D + 1) * D;  // 1056
 constexpr int TILE = 32;                  // tokens per phase-1 tile
-
-struct ChunkRange {
-  int begin, end;
-};
-__device__ __forceinline__ ChunkRange chunk_range(const int32_t* chunk_starts, int c, int N) {
-  ChunkRange r;
-  if (chunk_starts) {
-    r.begin = chunk_starts[c];
-    r.end = chunk_starts[c + 1];
-  } else {
-    r.begin = 0;
-    r.end = N;
-  }
-  return r;
-}
-
-// Optional transforms of q / k on load (bf16 io): RMSNorm over all channels of the token
-// (per-token 1/rms from a statistics pass, per-channel weight), applied before the ReLU, and the
-// rotary embedding applied after it.  The rotation acts on adjacent channel pairs (2i, 2i+1) of a
-// head, i.e. on the two halves of one packed dword; only the numerator operands are rotated, the
-// ksum row / denominator use the unrotated values.
-struct QkPre {
-  const float* rinv;       // [B][N], or null
-  const uint16_t* weight;  // [h*32] bf16, with rinv
-  const float* rope;       // [N][16][2] (cos, sin) per token and pair of a head, or null
-};
-
-// bf16(w * (x * rinv)): the float chain of the reference RMSNorm, rounded once at the end
-__device__ __forceinline__ u32x4_t rms_scale8(u32x4_t x, float rinv, u32x4_t w) {
-  u32x4_t o;
-#pragma unroll
-  for (int e = 0; e < 4; ++e)
-    o[e] = pack_bf16(bf16_lo(w[e]) * (bf16_lo(x[e]) * rinv), bf16_hi(w[e]) * (bf16_hi(x[e]) * rinv));
-  return o;
-}
-// (x0 + i x1)(cos + i sin) on the four channel pairs of x; cs0 = (c, s) of pairs 0, 1; cs1 of pairs 2, 3
-__device__ __forceinline__ u32x4_t rope8(u32x4_t x, f32x4_t cs0, f32x4_t cs1) {
-  const float c[4] = {cs0[0], cs0[2], cs1[0], cs1[2]}, sn[4] = {cs0[1], cs0[3], cs1[1], cs1[3]};
-  u32x4_t o;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const float x0 = bf16_lo(x[e]), x1 = bf16_hi(x[e]);
-    o[e] = pack_bf16(fmaf(x0, c[e], -(x1 * sn[e])), fmaf(x0, sn[e], x1 * c[e]));
-  }
-  return o;
-}
 
 // ----------------------------------------------------------------------------
 // phase 1, 16-bit io
@@ -651,7 +606,8 @@ extern "C" __attribute__((visibility("default"))) size_t sana_hip_linattn_worksp
                                                                                           int n_chunks,
                                                                                           int max_chunk_tokens,
                                                                                           int io_dtype) {
-  if (B <= 0 || h <= 0 || d != D || n_chunks <= 0 || max_chunk_tokens <= 0) return 0;
+  if (B <= 0 || h <= 0 || (d != D && d != 112) || n_chunks <= 0 || max_chunk_tokens <= 0) return 0;
+  if (d == 112) return io_dtype == SANA_DT_F32 ? 0 : workspace_bytes112(B, h, n_chunks, max_chunk_tokens);
   const StatePlan pl = plan_state(B, h, n_chunks, max_chunk_tokens, io_dtype);
   return pl.nsplit > 1 ? (size_t)B * h * n_chunks * pl.nsplit * STATE_ELEMS * sizeof(float) : 0;
 }
@@ -673,16 +629,19 @@ static int state_impl(const void* k, const void* v, float* state, void* workspac
     const int rc = check_pre(pre, io_dtype);
     if (rc != SANA_OK) return rc;
   }
-  if (d != D) return SANA_ERR_SHAPE;
+  if (d != D && d != 112) return SANA_ERR_SHAPE;
   if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
   if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
   if (max_chunk_tokens <= 0 || max_chunk_tokens > N) return SANA_ERR_ARG;
   if (io_dtype != SANA_DT_F32 && io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
-  if (stride_n < (int64_t)h * D || stride_b < 0) return SANA_ERR_ARG;
+  if (stride_n < (int64_t)h * d || stride_b < 0) return SANA_ERR_ARG;
   if ((int64_t)B * h > (1 << 22) || n_chunks > 65535) return SANA_ERR_SHAPE;
   const int esz = io_dtype == SANA_DT_F32 ? 4 : 2;
   if (!aligned16(k) || !aligned16(v) || !aligned16(state) || (stride_n * esz) % 16 || (stride_b * esz) % 16)
     return SANA_ERR_ALIGN;
+  if (d == 112)
+    return launch_state112(k, v, state, workspace, workspace_bytes, B, N, h, stride_b, stride_n, chunk_starts, n_chunks,
+                           max_chunk_tokens, causal, io_dtype, pre, static_cast<hipStream_t>(stream));
   const StatePlan pl = plan_state(B, h, n_chunks, max_chunk_tokens, io_dtype);
   float* dst = state;
   if (pl.nsplit > 1) {
@@ -760,8 +719,9 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_qk_rms(const void
 
 extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_chunk_scan(float* state, int B, int h, int d, int n_chunks, void* stream) {
   if (!state || B <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
-  if (d != D) return SANA_ERR_SHAPE;
+  if (d != D && d != 112) return SANA_ERR_SHAPE;
   if (n_chunks == 1) return SANA_OK;
+  if (d == 112) return launch_scan112(state, B, h, n_chunks, static_cast<hipStream_t>(stream));
   const int64_t threads = (int64_t)B * h * STATE_ELEMS;
   hipLaunchKernelGGL(linattn_reduce_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), state, state, B * h, n_chunks, 1, 1);
@@ -778,13 +738,13 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
     const int rc = check_pre(pre, io_dtype);
     if (rc != SANA_OK) return rc;
   }
-  if (d != D) return SANA_ERR_SHAPE;
+  if (d != D && d != 112) return SANA_ERR_SHAPE;
   if (n_chunks > 1 && !chunk_starts) return SANA_ERR_ARG;
   if (n_chunks == 1 && !chunk_starts) max_chunk_tokens = N;
   if (max_chunk_tokens <= 0 || max_chunk_tokens > N) return SANA_ERR_ARG;
   if (io_dtype != SANA_DT_F32 && io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
   if (out_dtype != io_dtype && out_dtype != SANA_DT_F32) return SANA_ERR_DTYPE;
-  if (q_stride_n < (int64_t)h * D || o_stride_n < (int64_t)h * D || q_stride_b < 0 || o_stride_b < 0)
+  if (q_stride_n < (int64_t)h * d || o_stride_n < (int64_t)h * d || q_stride_b < 0 || o_stride_b < 0)
     return SANA_ERR_ARG;
   if ((int64_t)B * h > (1 << 22) || n_chunks > 65535) return SANA_ERR_SHAPE;
   const int qsz = io_dtype == SANA_DT_F32 ? 4 : 2, osz = out_dtype == SANA_DT_F32 ? 4 : 2;
@@ -792,6 +752,9 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
       (o_stride_n * osz) % 16 || (o_stride_b * osz) % 16)
     return SANA_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d == 112)
+    return launch_apply112(q, state, out, B, N, h, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
+                           n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, pre, s);
   const int wg_tokens = io_dtype == SANA_DT_BF16 ? SANA_LA_APPLY_TOKENS : 64;
   const unsigned gx = (unsigned)((max_chunk_tokens + wg_tokens - 1) / wg_tokens);
   if (io_dtype == SANA_DT_BF16) {

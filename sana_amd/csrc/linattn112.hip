@@ -1,0 +1,485 @@
+// ReLU linear attention for head_dim 112 (the `linear_head_dim: 112` video configurations) on gfx950,
+// bf16 / f16 io.  Same two phases and the same state layout as the head_dim-32 kernels --
+// fp32 [B][h][n_chunks][113][112], row 112 = sum_n relu(k_n) -- but one head is now a 112 x 112
+// problem of its own (3.5 x 3.5 MFMA tiles, padded to 4 x 4 with zero channels):
+//
+//   phase 1  workgroup = (batch, head, chunk, token split); each of its four waves takes interleaved
+//            32-token tiles and owns a whole 128 x 128 accumulator (256 registers).  Tiles go through
+//            wave-private LDS to become token-contiguous MFMA operands, as in the head_dim-32 kernel;
+//            the waves are summed in LDS in two rounds and a second kernel sums the splits in a
+//            fixed order.
+//   phase 2  workgroup = (batch, head, chunk, 64-token range); wave w produces output channels
+//            [32w, 32w+32) from its own slice of the state (two bf16 terms of the fp32 values as
+//            MFMA 16x16x32 A operands for bf16 output, three for fp32 output) plus a row block that
+//            carries ksum in every row, so each lane gets its token's denominator.
+#include "common.h"
+#include "linattn_common.h"
+
+namespace sana {
+namespace {
+
+constexpr int DH = 112;                 // head dim
+constexpr int SE = (DH + 1) * DH;       // 12656 state elements per (batch, head, chunk)
+constexpr int NCH = DH / 8;             // 14 16-byte chunks per token and head
+constexpr int TILE = 32;
+
+// ----------------------------------------------------------------------------
+// phase 1.  grid: x = token splits, y = n_chunks, z = B * h; block 256.
+// partial[(bh * n_chunks + c) * nsplit + split][SE]
+// ----------------------------------------------------------------------------
+constexpr int LR = 160;  // LDS tile row stride in elements: 320 B puts the two token groups of a read 16 banks apart
+constexpr int SMEM_BYTES = 2 * SE * 4;  // two fp32 states for the wave reduction (>= 4 waves x 2 tiles x 32 x LR x 2 B)
+static_assert(SMEM_BYTES >= 4 * 2 * TILE * LR * 2, "staging must fit");
+
+template <typename T, bool PRE>
+__global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
+                                                       float* __restrict__ partial,
+                                                       const int32_t* __restrict__ chunk_starts, int N, int h,
+                                                       int n_chunks, int nsplit, int split_tokens, int64_t stride_b,
+                                                       int64_t stride_n, const QkPre pre) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int b = blockIdx.z / h, head = blockIdx.z % h;
+  const int c = blockIdx.y, split = blockIdx.x;
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + split * split_tokens;
+  const int t1 = min(cr.end, t0 + split_tokens);
+  uint16_t* lds_k = reinterpret_cast<uint16_t*>(smem) + wave * (2 * TILE * LR);
+  uint16_t* lds_v = lds_k + TILE * LR;
+  // channels 112..127 of every tile row are written once, as zeros, and never again
+  for (int i = lane; i < 2 * TILE * 2; i += 64) {  // (2 tiles x 32 rows) x 2 chunks of 8; rows 32..63 are the V tile
+    const int row = i >> 1, chunk = NCH + (i & 1);
+    *reinterpret_cast<u32x4_t*>(lds_k + row * LR + chunk * 8) = u32x4_t{0u, 0u, 0u, 0u};
+  }
+
+  // load mapping: linear chunk id = lane + 64 i (i < 7): token id / 14, chunk id % 14 -- consecutive lanes
+  // read consecutive 16-byte pieces of a token's 224-byte head row
+  int ld_tok[7], ld_ch[7];
+#pragma unroll
+  for (int i = 0; i < 7; ++i) {
+    const int id = lane + 64 * i;
+    ld_tok[i] = id / NCH;
+    ld_ch[i] = id - ld_tok[i] * NCH;
+  }
+  const uint16_t* kbase = K + (int64_t)b * stride_b + head * DH;
+  const uint16_t* vbase = V + (int64_t)b * stride_b + head * DH;
+  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  float acck[4] = {0.f, 0.f, 0.f, 0.f};  // ksum of channel 32 jb + lane % 32 over this lane's token half
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  u32x4_t kreg[7], vreg[7];
+  auto issue_loads = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+      const int tok = tile + ld_tok[i];
+      if (tok < t1) {
+        kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n + ld_ch[i] * 8);
+        vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n + ld_ch[i] * 8);
+      } else {
+        kreg[i] = zero4;
+        vreg[i] = zero4;
+      }
+    }
+  };
+  // PRE: the MFMA operands in LDS are rotated, ksum needs the unrotated values: a second, unrotated
+  // copy of the K tile would double the LDS traffic, so ksum is accumulated per lane, load slot and
+  // channel here and folded over lanes once at the end
+  float ks8[PRE ? 7 : 1][8];
+  if (PRE) {
+#pragma unroll
+    for (int i = 0; i < 7; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ks8[i][e] = 0.f;
+  }
+
+  int tile = t0 + wave * TILE;
+  if (tile < t1) issue_loads(tile);
+  // operand read mapping: lane -> channel j = lane%32 of a 32-channel block, k-group g = lane/32;
+  // element r of k-step s is token 16*s + 2*r + g of the tile (both operands use the same bijection)
+  const int j = lane & 31, g = lane >> 5;
+  for (; tile < t1; tile += 4 * TILE) {
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+      u32x4_t kk = kreg[i];
+      if (PRE) {
+        const bool tok_ok = tile + ld_tok[i] < t1;
+        const int tok = min(tile + ld_tok[i], t1 - 1);
+        if (has_norm) {
+          const u32x4_t kw = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[i] * 8);
+          kk = rms_scale8(kk, tok_ok ? pre.rinv[(int64_t)b * N + tok] : 0.f, kw);
+        }
+        kk = relu_pk16(kk);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ks8[i][2 * e] += bf16_lo(kk[e]);
+          ks8[i][2 * e + 1] += bf16_hi(kk[e]);
+        }
+        if (has_rope) {
+          const float* rp = pre.rope + ((int64_t)tok * (DH / 2) + ld_ch[i] * 4) * 2;
+          kk = rope8(kk, *reinterpret_cast<const f32x4_t*>(rp), *reinterpret_cast<const f32x4_t*>(rp + 4));
+        }
+      } else {
+        kk = relu_pk16(kk);
+      }
+      *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
+      *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
+    }
+    if (tile + 4 * TILE < t1) issue_loads(tile + 4 * TILE);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      u32x4_t fk[4], fv[4];
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk) {
+#pragma unroll
+        for (int r2 = 0; r2 < 4; ++r2) {
+          const int ta = 16 * s + 2 * (2 * r2) + g, tb = 16 * s + 2 * (2 * r2 + 1) + g;
+          const uint32_t klo = lds_k[ta * LR + blk * 32 + j], khi = lds_k[tb * LR + blk * 32 + j];
+          const uint32_t vlo = lds_v[ta * LR + blk * 32 + j], vhi = lds_v[tb * LR + blk * 32 + j];
+          fk[blk][r2] = klo | (khi << 16);
+          fv[blk][r2] = vlo | (vhi << 16);
+        }
+      }
+#pragma unroll
+      for (int ib = 0; ib < 4; ++ib)
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb) acc[ib][jb] = mfma_32x32x16<T>(fv[ib], fk[jb], acc[ib][jb]);
+      if (!PRE) {
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+          for (int r2 = 0; r2 < 4; ++r2) acck[jb] = add_pk16<T>(fk[jb][r2], acck[jb]);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites
+  }
+
+  if (PRE) {
+    // load slot i of lane l held chunk (l + 64 i) % 14 of tile token (l + 64 i) / 14: through the wave's own
+    // LDS region ([448 ids][8] floats = 14 KB), then channel 32 jb + j sums its 32 tokens in a fixed order
+    float* fold = reinterpret_cast<float*>(lds_k);
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+      f32x4_t lo = {ks8[i][0], ks8[i][1], ks8[i][2], ks8[i][3]}, hi = {ks8[i][4], ks8[i][5], ks8[i][6], ks8[i][7]};
+      *reinterpret_cast<f32x4_t*>(fold + (lane + 64 * i) * 8) = lo;
+      *reinterpret_cast<f32x4_t*>(fold + (lane + 64 * i) * 8 + 4) = hi;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      const int ch = jb * 32 + j;
+      float sum = 0.f;
+      if (ch < DH)
+        for (int tk = 16 * g; tk < 16 * g + 16; ++tk) sum += fold[(tk * NCH + (ch >> 3)) * 8 + (ch & 7)];
+      acck[jb] = sum;
+    }
+  }
+#pragma unroll
+  for (int jb = 0; jb < 4; ++jb) acck[jb] += __shfl_xor(acck[jb], 32, 64);  // the two token halves
+
+  // cross-wave sum in LDS, two rounds (two states fit): waves 2, 3 -> waves 0, 1; wave 1 -> wave 0.
+  // D layout of 32x32 MFMA: lane -> column j = lane%32, register r -> row 8*(r/4) + 4*(lane/32) + r%4
+  float* red = reinterpret_cast<float*>(smem);
+  auto put = [&](float* dstp) {
+#pragma unroll
+    for (int ib = 0; ib < 4; ++ib)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        const int col = jb * 32 + j;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (row < DH && col < DH) dstp[row * DH + col] = acc[ib][jb][r];
+        }
+      }
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb)
+      if (g == 0 && jb * 32 + j < DH) dstp[DH * DH + jb * 32 + j] = acck[jb];
+  };
+  auto take = [&](const float* srcp) {
+#pragma unroll
+    for (int ib = 0; ib < 4; ++ib)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        const int col = jb * 32 + j;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (row < DH && col < DH) acc[ib][jb][r] += srcp[row * DH + col];
+        }
+      }
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb)
+      if (jb * 32 + j < DH) acck[jb] += srcp[DH * DH + jb * 32 + j];
+  };
+  __syncthreads();  // staging tiles are dead
+  if (wave >= 2) put(red + (wave - 2) * SE);
+  __syncthreads();
+  if (wave < 2) take(red + wave * SE);
+  __syncthreads();
+  if (wave == 1) put(red);
+  __syncthreads();
+  if (wave == 0) {
+    take(red);
+    const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nsplit + split;
+    put(partial + slot * SE);
+  }
+}
+
+// sum of the partials of one state in partial order (+ inclusive prefix over chunks when causal)
+__global__ __launch_bounds__(256) void reduce112_kernel(const float* partial, float* state,
+                                                        int BH, int n_chunks, int nparts, int causal) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (int64_t)BH * SE) return;
+  const int64_t bh = gid / SE;
+  const int e = (int)(gid - bh * SE);
+  float run = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float* p0 = partial + ((bh * n_chunks + c) * nparts) * SE + e;
+    float s = 0.f;
+    for (int sp0 = 0; sp0 < nparts; sp0 += 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = (sp0 + u < nparts) ? p0[(int64_t)(sp0 + u) * SE] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) s += v[u];
+    }
+    if (causal) {
+      run += s;
+      s = run;
+    }
+    state[(bh * n_chunks + c) * SE + e] = s;
+  }
+}
+
+// ----------------------------------------------------------------------------
+// phase 2.  1-D grid over (batch, chunk, token range, head), head fastest; block 256.
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ void split3_112(const float x[8], u32x4_t out[3]) {
+  uint32_t hi[8], mid[8], lo[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    hi[e] = f32_to_bf16_bits(x[e]);
+    const float r1 = x[e] - bf16_bits_to_f32(hi[e]);
+    mid[e] = f32_to_bf16_bits(r1);
+    lo[e] = f32_to_bf16_bits(r1 - bf16_bits_to_f32(mid[e]));
+  }
+#pragma unroll
+  for (int e2 = 0; e2 < 4; ++e2) {
+    out[0][e2] = hi[2 * e2] | (hi[2 * e2 + 1] << 16);
+    out[1][e2] = mid[2 * e2] | (mid[2 * e2 + 1] << 16);
+    out[2][e2] = lo[2 * e2] | (lo[2 * e2 + 1] << 16);
+  }
+}
+
+constexpr int APPLY_TOKENS = 256;  // tokens per workgroup
+
+template <bool OUT_F32, bool PRE>
+__global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
+                                                       void* __restrict__ out,
+                                                       const int32_t* __restrict__ chunk_starts, int N, int h,
+                                                       int n_chunks, int xranges, int64_t q_stride_b,
+                                                       int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
+                                                       float eps, const QkPre pre) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int head, bx, c, b;
+  {
+    int rest = blockIdx.x;
+    head = rest % h, rest /= h;
+    bx = rest % xranges, rest /= xranges;
+    c = rest % n_chunks, b = rest / n_chunks;
+  }
+  const ChunkRange cr = chunk_range(chunk_starts, c, N);
+  const int t0 = cr.begin + bx * APPLY_TOKENS;
+  const int t1 = min(cr.end, t0 + APPLY_TOKENS);
+  if (t0 >= t1) return;  // no barriers in this kernel
+  const int n = lane & 15, g = lane >> 4;
+
+  // A operands.  MFMA 16x16x32: A lane -> row lane%16, k = 8*(lane/16)+e.  Row r of row block rb of this
+  // wave is output channel 32*wave + 8*(r/4) + 4*rb + r%4, so that a lane (token n, group g') ends up
+  // with the 8 contiguous channels 32*wave + 8*g' .. +7 (registers s of blocks 0 and 1).  Block 2
+  // carries ksum in every row.  Channels and k indices past 112 are zero.
+  const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * SE;
+  constexpr int NT = OUT_F32 ? 3 : 2;  // bf16 terms of an fp32 state value: 24 / 16 mantissa bits
+  u32x4_t a[3][4][NT];                 // [row block][k block][term]
+#pragma unroll
+  for (int rb = 0; rb < 3; ++rb) {
+    const int ch = 32 * wave + 8 * (n >> 2) + 4 * rb + (n & 3);
+    const int row = rb < 2 ? ch : DH;
+    const bool row_ok = rb == 2 || ch < DH;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int k0 = kb * 32 + 8 * g;
+      float x[8];
+      if (row_ok && k0 < DH) {
+        const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(sp + row * DH + k0);
+        const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(sp + row * DH + k0 + 4);
+        x[0] = x0[0], x[1] = x0[1], x[2] = x0[2], x[3] = x0[3], x[4] = x1[0], x[5] = x1[1], x[6] = x1[2], x[7] = x1[3];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0.f;
+      }
+      u32x4_t t3[3];
+      split3_112(x, t3);
+#pragma unroll
+      for (int term = 0; term < NT; ++term) a[rb][kb][term] = t3[term];
+    }
+  }
+
+  const uint16_t* qp = Q + (int64_t)b * q_stride_b + head * DH + 8 * g;
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  u32x4_t qw[4] = {zero4, zero4, zero4, zero4};
+  if (has_norm) {
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+      if (kb * 32 + 8 * g < DH) qw[kb] = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + kb * 32 + 8 * g);
+  }
+  const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
+  for (int t = t0; t < t1; t += 16) {
+    const int tok = t + n;
+    const bool tok_ok = tok < t1;
+    u32x4_t qd[4], qb[4];
+    const float rin = has_norm && tok_ok ? pre.rinv[(int64_t)b * N + tok] : 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const bool ok = tok_ok && kb * 32 + 8 * g < DH;
+      u32x4_t x = ok ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + kb * 32) : zero4;
+      if (has_norm) x = rms_scale8(x, rin, qw[kb]);
+      x = relu_pk16(x);
+      qd[kb] = x;  // denominator operand (unrotated)
+      if (has_rope && ok) {
+        const float* rp = pre.rope + ((int64_t)tok * (DH / 2) + (kb * 4 + g) * 4) * 2;
+        x = rope8(x, *reinterpret_cast<const f32x4_t*>(rp), *reinterpret_cast<const f32x4_t*>(rp + 4));
+      }
+      qb[kb] = x;  // numerator operand
+    }
+    f32x4_t acc[3];
+#pragma unroll
+    for (int rb = 0; rb < 3; ++rb) {
+      f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int term = NT - 1; term >= 0; --term)  // smallest term first
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) s = mfma_16x16x32_bf16(a[rb][kb][term], rb < 2 ? qb[kb] : qd[kb], s);
+      acc[rb] = s;
+    }
+    if (tok_ok && och < DH) {
+      const float den = acc[2][0] + eps;
+      const int64_t o_off = (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + head * DH + och;
+      if (OUT_F32) {
+        f32x4_t o0, o1;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          o0[s] = acc[0][s] / den;
+          o1[s] = acc[1][s] / den;
+        }
+        float* op = reinterpret_cast<float*>(out) + o_off;
+        *reinterpret_cast<f32x4_t*>(op) = o0;
+        *reinterpret_cast<f32x4_t*>(op + 4) = o1;
+      } else {
+        const float inv = __builtin_amdgcn_rcpf(den);
+        u32x4_t o;
+        o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
+        o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
+        o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
+        o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
+        *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + o_off) = o;
+      }
+    }
+  }
+}
+
+struct Plan112 {
+  int nsplit, split_tokens;
+};
+Plan112 plan112(int B, int h, int n_chunks, int max_chunk_tokens) {
+  // one workgroup per CU (256 accumulator registers per wave: one wave per SIMD), splits of at least 512 tokens
+  const int items = B * h * n_chunks;
+  int ns = (256 + items - 1) / items;
+  const int cap = (max_chunk_tokens + 511) / 512;
+  if (ns > cap) ns = cap;
+  if (ns < 1) ns = 1;
+  if (ns > 64) ns = 64;
+  Plan112 pl;
+  pl.split_tokens = ((max_chunk_tokens + ns - 1) / ns + 127) / 128 * 128;
+  pl.nsplit = (max_chunk_tokens + pl.split_tokens - 1) / pl.split_tokens;
+  if (pl.nsplit < 1) pl.nsplit = 1;
+  return pl;
+}
+
+}  // namespace
+
+size_t workspace_bytes112(int B, int h, int n_chunks, int max_chunk_tokens) {
+  const Plan112 pl = plan112(B, h, n_chunks, max_chunk_tokens);
+  return (size_t)B * h * n_chunks * pl.nsplit * SE * sizeof(float);  // the partials are always written
+}
+
+int launch_state112(const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N,
+                    int h, int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts, int n_chunks,
+                    int max_chunk_tokens, int causal, int io_dtype, const QkPre& pre, hipStream_t s) {
+  if (io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
+  const bool use_pre = pre.rinv || pre.rope;
+  if (use_pre && io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  const Plan112 pl = plan112(B, h, n_chunks, max_chunk_tokens);
+  const size_t need = workspace_bytes112(B, h, n_chunks, max_chunk_tokens);
+  if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return SANA_ERR_ALIGN;
+  float* part = static_cast<float*>(workspace);
+  dim3 grid(pl.nsplit, n_chunks, B * h);
+  const uint16_t* kp = static_cast<const uint16_t*>(k);
+  const uint16_t* vp = static_cast<const uint16_t*>(v);
+#define SANA_ST112(T, PRE)                                                                                        \
+  hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(256), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
+                     pl.nsplit, pl.split_tokens, stride_b, stride_n, pre)
+  if (io_dtype == SANA_DT_F16) SANA_ST112(F16, false);
+  else if (use_pre) SANA_ST112(BF16, true);
+  else SANA_ST112(BF16, false);
+#undef SANA_ST112
+  if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+  const int64_t threads = (int64_t)B * h * SE;
+  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, part, state, B * h,
+                     n_chunks, pl.nsplit, (causal && n_chunks > 1) ? 1 : 0);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+int launch_scan112(float* state, int B, int h, int n_chunks, hipStream_t s) {
+  const int64_t threads = (int64_t)B * h * SE;
+  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, state, state, B * h,
+                     n_chunks, 1, 1);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+int launch_apply112(const void* q, const float* state, void* out, int B, int N, int h, int64_t q_stride_b,
+                    int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts,
+                    int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
+                    hipStream_t s) {
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  const bool use_pre = pre.rinv || pre.rope;
+  const int xranges = (max_chunk_tokens + APPLY_TOKENS - 1) / APPLY_TOKENS;
+  const int64_t total = (int64_t)xranges * n_chunks * B * h;
+  if (total > 0x7fffffff) return SANA_ERR_SHAPE;
+  dim3 grid((unsigned)total);
+  const uint16_t* qp = static_cast<const uint16_t*>(q);
+#define SANA_AP112(F32, PRE)                                                                                         \
+  hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
+                     xranges, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
+  if (out_dtype == SANA_DT_F32) {
+    if (use_pre) SANA_AP112(true, true);
+    else SANA_AP112(true, false);
+  } else {
+    if (use_pre) SANA_AP112(false, true);
+    else SANA_AP112(false, false);
+  }
+#undef SANA_AP112
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+}  // namespace sana

@@ -12,6 +12,7 @@ from ._lib import DT_BF16, DT_F16, DT_F32, SanaHipError
 
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 HEAD_DIM = 32
+HEAD_DIMS = (32, 112)   # head dims with kernels: 32 (all dtypes), 112 (bf16; the video configurations)
 
 _workspaces = {}     # (device index) -> uint8 tensor, grown on demand
 _chunk_tables = {}   # (device index, tuple) -> int32 tensor
@@ -71,7 +72,7 @@ def _token_major_view(t: torch.Tensor, what: str) -> Tuple[int, int]:
 class QkPre:
     """Transforms applied to q or k on load inside the attention kernels (bf16 io):
     RMSNorm over all channels (``rinv`` [B, N] fp32 from :func:`qk_rms` and the bf16
-    ``weight`` [C]) before the ReLU, rotary embedding (``rope`` [N, 16, 2] fp32 from
+    ``weight`` [C]) before the ReLU, rotary embedding (``rope`` [N, head_dim/2, 2] fp32 from
     :func:`rope_table`) after it, on the numerator operands only."""
 
     __slots__ = ("rinv", "weight", "rope")
@@ -81,7 +82,7 @@ class QkPre:
             raise SanaHipError("rinv and weight go together")
         self.rinv, self.weight, self.rope = rinv, weight, rope
 
-    def check(self, x: torch.Tensor) -> Tuple[Optional[int], Optional[int], Optional[int]]:
+    def check(self, x: torch.Tensor, head_dim: int = HEAD_DIM) -> Tuple[Optional[int], Optional[int], Optional[int]]:
         B, N, C = x.shape
         _need_cuda(self.rinv, self.weight, self.rope)
         if x.dtype != torch.bfloat16:
@@ -92,9 +93,9 @@ class QkPre:
             if self.weight.dtype != torch.bfloat16 or self.weight.numel() != C or not self.weight.is_contiguous():
                 raise SanaHipError(f"norm weight must be contiguous bf16 [{C}]")
         if self.rope is not None:
-            if self.rope.dtype != torch.float32 or tuple(self.rope.shape) != (N, HEAD_DIM // 2, 2) or \
+            if self.rope.dtype != torch.float32 or tuple(self.rope.shape) != (N, head_dim // 2, 2) or \
                     not self.rope.is_contiguous():
-                raise SanaHipError(f"rope must be contiguous fp32 {(N, HEAD_DIM // 2, 2)}")
+                raise SanaHipError(f"rope must be contiguous fp32 {(N, head_dim // 2, 2)}")
         ptr = lambda t: None if t is None else t.data_ptr()
         return ptr(self.rinv), ptr(self.weight), ptr(self.rope)
 
@@ -115,54 +116,63 @@ def qk_rms(q: torch.Tensor, k: torch.Tensor, eps: float) -> Tuple[torch.Tensor, 
     return rq, rk
 
 
-def rope_table(freqs: torch.Tensor, N: int, device) -> torch.Tensor:
-    """Complex rotary factors [..., N, 16] (any leading singleton dims, as the reference passes
-    ``rotary_emb`` [1, 1, N, d/2]) -> fp32 (cos, sin) table [N, 16, 2] on ``device``."""
+def rope_table(freqs: torch.Tensor, N: int, device, head_dim: int = HEAD_DIM) -> torch.Tensor:
+    """Complex rotary factors [..., N, d/2] (any leading singleton dims, as the reference passes
+    ``rotary_emb`` [1, 1, N, d/2]) -> fp32 (cos, sin) table [N, d/2, 2] on ``device``."""
     if not torch.is_complex(freqs):
         raise SanaHipError("rotary_emb must be a complex tensor of unit factors")
     f = freqs.reshape(-1, freqs.shape[-1])
-    if tuple(f.shape) != (N, HEAD_DIM // 2):
-        raise SanaHipError(f"rotary_emb must broadcast over batch and heads: expected [.., {N}, {HEAD_DIM // 2}], "
+    if tuple(f.shape) != (N, head_dim // 2):
+        raise SanaHipError(f"rotary_emb must broadcast over batch and heads: expected [.., {N}, {head_dim // 2}], "
                            f"got {tuple(freqs.shape)}")
     return torch.view_as_real(f.to(torch.complex64)).to(device=device, dtype=torch.float32).contiguous()
 
 
+def _head_dim(d: int) -> int:
+    if d not in HEAD_DIMS:
+        raise SanaHipError(f"head_dim {d} has no kernel (supported: {HEAD_DIMS})")
+    return d
+
+
 def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False,
-                  pre: Optional[QkPre] = None) -> torch.Tensor:
-    """Phase 1.  k, v: [B, N, C] token-major views (C = h*32).  Returns the fp32
-    state [B, h, n_chunks, 33, 32] (inclusive prefix over chunks when causal)."""
+                  pre: Optional[QkPre] = None, head_dim: int = HEAD_DIM) -> torch.Tensor:
+    """Phase 1.  k, v: [B, N, C] token-major views (C = h*d).  Returns the fp32
+    state [B, h, n_chunks, d+1, d] (inclusive prefix over chunks when causal)."""
+    d = _head_dim(head_dim)
     _need_cuda(k, v)
     same = all(a == b or n == 1 for a, b, n in zip(k.stride(), v.stride(), k.shape))
     if k.shape != v.shape or k.dtype != v.dtype or not same:
         raise SanaHipError("k and v must share shape, dtype and strides")
     B, N, C = k.shape
-    if C % HEAD_DIM:
-        raise SanaHipError(f"C={C} is not a multiple of head_dim {HEAD_DIM}")
-    h = C // HEAD_DIM
+    if C % d:
+        raise SanaHipError(f"C={C} is not a multiple of head_dim {d}")
+    h = C // d
     sb, sn = _token_major_view(k, "k")
     tab, n_chunks, longest = chunk_table(chunk_tokens, N, k.device)
     lib = _lib.load()
-    state = torch.empty(B, h, n_chunks, HEAD_DIM + 1, HEAD_DIM, dtype=torch.float32, device=k.device)
-    nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, HEAD_DIM, n_chunks, longest, _dt(k))
+    state = torch.empty(B, h, n_chunks, d + 1, d, dtype=torch.float32, device=k.device)
+    nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, d, n_chunks, longest, _dt(k))
     ws = _workspace(k.device, nbytes)
     args = (k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
-            B, N, h, HEAD_DIM, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
+            B, N, h, d, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
             1 if causal else 0, _dt(k))
     if pre is None:
         code = lib.sana_hip_linattn_state(*args, _stream())
     else:
-        code = lib.sana_hip_linattn_state_pre(*args, *pre.check(k), _stream())
+        code = lib.sana_hip_linattn_state_pre(*args, *pre.check(k, d), _stream())
     _lib.check(code, "sana_hip_linattn_state")
     return state
 
 
 def linattn_chunk_scan_(state: torch.Tensor) -> torch.Tensor:
-    """In-place inclusive prefix sum over the chunk axis of [B, h, n_chunks, 33, 32] fp32."""
+    """In-place inclusive prefix sum over the chunk axis of [B, h, n_chunks, d+1, d] fp32."""
     _need_cuda(state)
-    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 5:
-        raise SanaHipError("state must be contiguous fp32 [B, h, n_chunks, 33, 32]")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 5 or \
+            state.shape[3] != state.shape[4] + 1:
+        raise SanaHipError("state must be contiguous fp32 [B, h, n_chunks, d+1, d]")
     B, h, n_chunks = state.shape[:3]
-    code = _lib.load().sana_hip_linattn_chunk_scan(state.data_ptr(), B, h, HEAD_DIM, n_chunks, _stream())
+    d = _head_dim(state.shape[4])
+    code = _lib.load().sana_hip_linattn_chunk_scan(state.data_ptr(), B, h, d, n_chunks, _stream())
     _lib.check(code, "sana_hip_linattn_chunk_scan")
     return state
 
@@ -174,32 +184,35 @@ def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens
     Returns [B, N, C] in ``out_dtype`` (q's dtype or fp32)."""
     _need_cuda(q, state)
     B, N, C = q.shape
-    h = C // HEAD_DIM
+    d = _head_dim(state.shape[-1])
+    h = C // d
     qsb, qsn = _token_major_view(q, "q")
     tab, n_chunks, longest = chunk_table(chunk_tokens, N, q.device)
     if state.dtype != torch.float32 or not state.is_contiguous() or \
-            tuple(state.shape) != (B, h, n_chunks, HEAD_DIM + 1, HEAD_DIM):
-        raise SanaHipError(f"state must be contiguous fp32 {(B, h, n_chunks, 33, 32)}, got {tuple(state.shape)}")
+            tuple(state.shape) != (B, h, n_chunks, d + 1, d):
+        raise SanaHipError(f"state must be contiguous fp32 {(B, h, n_chunks, d + 1, d)}, "
+                           f"got {tuple(state.shape)}")
     out_dtype = out_dtype or q.dtype
     if out is None:
         out = torch.empty(B, N, C, dtype=out_dtype, device=q.device)
     elif out.shape != q.shape or out.dtype != out_dtype:
         raise SanaHipError("out has the wrong shape or dtype")
     osb, osn = _token_major_view(out, "out")
-    args = (q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, HEAD_DIM, qsb, qsn, osb, osn,
+    args = (q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, d, qsb, qsn, osb, osn,
             tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype])
     if pre is None:
         code = _lib.load().sana_hip_linattn_apply(*args, _stream())
     else:
-        code = _lib.load().sana_hip_linattn_apply_pre(*args, *pre.check(q), _stream())
+        code = _lib.load().sana_hip_linattn_apply_pre(*args, *pre.check(q, d), _stream())
     _lib.check(code, "sana_hip_linattn_apply")
     return out
 
 
-def relu_linear_attention(q, k, v, eps: float, chunk_tokens=None, out_dtype=None) -> torch.Tensor:
+def relu_linear_attention(q, k, v, eps: float, chunk_tokens=None, out_dtype=None,
+                          head_dim: int = HEAD_DIM) -> torch.Tensor:
     """Both phases on token-major [B, N, C] views; chunk-causal when ``chunk_tokens`` has > 1 entry."""
     causal = chunk_tokens is not None and len(chunk_tokens) > 1
-    state = linattn_state(k, v, chunk_tokens, causal=causal)
+    state = linattn_state(k, v, chunk_tokens, causal=causal, head_dim=head_dim)
     return linattn_apply(q, state, eps, chunk_tokens, out_dtype)
 
 
