@@ -163,7 +163,32 @@ def kernel_rooflines(dev, iters=50, warmup=10):
     add("linattn_apply_chunk_causal_cfg5", "hbm", la5,
         event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st5, 1e-8, starts, out=out5), iters, warmup),
         "cfg5: Q read + out write + 21 states")
-    del qkv5, out5
+    # the same video shape with 112-wide heads (linear_head_dim = 112: 20 heads at C = 2240), q/k RMSNorm and rotary
+    # embedding on load as the video blocks use them; whole sequence as one chunk, and 21 causal chunks
+    D2 = 112
+    h2 = C // D2
+    rq5, rk5 = ops.qk_rms(qkv5[:, :, 0], qkv5[:, :, 1], 1e-5)
+    theta = torch.rand(Nv, D2 // 2, generator=g, dtype=torch.float64) * 6.283
+    rope5 = ops.rope_table(torch.polar(torch.ones_like(theta), theta), Nv, dev, head_dim=D2)
+    pk5, pq5 = ops.QkPre(rk5, wn, rope5), ops.QkPre(rq5, wn, rope5)
+    se2 = h2 * (D2 + 1) * D2 * 4
+    st112 = ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], head_dim=D2)
+    add("linattn_state_d112", "hbm", 2 * Nv * C * 2 + se2,
+        event_time_us(lambda: ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], head_dim=D2), iters, warmup),
+        "N=32760, 20 heads of 112; K,V read + state")
+    add("linattn_apply_d112", "hbm", 2 * Nv * C * 2 + se2,
+        event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st112, 1e-8, out=out5), iters, warmup),
+        "N=32760, 20 heads of 112; Q read + out write + state")
+    rope_bytes5 = Nv * (D2 // 2) * 2 * 4 + Nv * 4
+    add("linattn_state_d112_norm_rope_chunk_causal", "hbm", la5 - 21 * (C // 32) * 33 * 32 * 4 + 21 * se2 + rope_bytes5,
+        event_time_us(lambda: ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts, causal=True, pre=pk5,
+                                                head_dim=D2), iters, warmup),
+        "cfg5 with 112-wide heads: K,V read + 21 states + rope table (448 B/token) + 1/rms")
+    st112c = ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts, causal=True, pre=pk5, head_dim=D2)
+    add("linattn_apply_d112_norm_rope_chunk_causal", "hbm", la5 - 21 * (C // 32) * 33 * 32 * 4 + 21 * se2 + rope_bytes5,
+        event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st112c, 1e-8, starts, out=out5, pre=pq5), iters, warmup),
+        "cfg5 with 112-wide heads: Q read + out write + 21 states + rope table + 1/rms")
+    del qkv5, out5, st112, st112c, rope5
     u = torch.randn(B, 128, 128, 2 * HID, generator=g).bfloat16().to(dev)
     dw = (torch.randn(2 * HID, 1, 3, 3, generator=g) * 0.3).bfloat16().to(dev)
     db = torch.zeros(2 * HID, dtype=torch.bfloat16, device=dev)

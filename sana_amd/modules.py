@@ -168,8 +168,9 @@ class LiteLA(nn.Module):
             raise NotImplementedError("LiteLA: in_dim != out_dim is not used by any Sana block")
         self.in_dim, self.out_dim, self.heads = in_dim, out_dim, heads
         self.dim = out_dim // heads
-        if self.dim != HEAD_DIM:
-            raise NotImplementedError(f"the gfx950 attention kernels are built for head_dim {HEAD_DIM}, got {self.dim}")
+        if self.dim not in ops.HEAD_DIMS:
+            raise NotImplementedError(f"the gfx950 attention kernels are built for head_dim {ops.HEAD_DIMS}, "
+                                      f"got {self.dim}")
         self.eps = eps
         self.num_heads = heads
         self.scale = self.dim ** -0.5
@@ -195,7 +196,7 @@ class LiteLA(nn.Module):
         vt = _as_token_major(v, 3)
         if any(a != b and n > 1 for a, b, n in zip(kt.stride(), vt.stride(), kt.shape)):
             kt, vt = kt.contiguous(), vt.contiguous()
-        out = ops.relu_linear_attention(qt, kt, vt, self.eps, out_dtype=torch.float32)  # ReLU is applied in-kernel
+        out = ops.relu_linear_attention(qt, kt, vt, self.eps, out_dtype=torch.float32, head_dim=d)  # ReLU in-kernel
         return out.view(B, N, h, d).permute(0, 2, 3, 1)
 
     def _qkv_tokens(self, x: torch.Tensor, rotary_emb=None) -> torch.Tensor:
@@ -222,7 +223,7 @@ class LiteLA(nn.Module):
             out = self._attend(self.qkv(x).view(B, N, 3, C), None)
         else:
             qkv = self._qkv_tokens(x, rotary_emb)
-            out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps)
+            out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps, head_dim=self.dim)
         return self.proj(out, gate=gate, residual=residual)
 
     def _pre(self, qkv: torch.Tensor, rotary_emb):
@@ -238,7 +239,7 @@ class LiteLA(nn.Module):
             cache = self.__dict__.get("_rope_cache")
             key = (id(rotary_emb), rotary_emb._version, N, qkv.device)
             if cache is None or cache[0] != key:
-                cache = (key, ops.rope_table(rotary_emb, N, qkv.device))
+                cache = (key, ops.rope_table(rotary_emb, N, qkv.device, head_dim=self.dim))
                 self.__dict__["_rope_cache"] = cache
             rope = cache[1]
         if norm:
@@ -253,7 +254,8 @@ class LiteLA(nn.Module):
     def _attend(self, qkv, rotary_emb, chunk_tokens=None):
         pre_q, pre_k = self._pre(qkv, rotary_emb)
         causal = chunk_tokens is not None and len(chunk_tokens) > 1
-        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], chunk_tokens, causal=causal, pre=pre_k)
+        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], chunk_tokens, causal=causal, pre=pre_k,
+                                  head_dim=self.dim)
         return ops.linattn_apply(qkv[:, :, 0], state, self.eps, chunk_tokens, pre=pre_q)
 
 
@@ -319,15 +321,16 @@ class CachedCausalAttention(LiteLAReLURope):
         B, N, C = x.shape
         qkv = self.qkv(x).view(B, N, 3, C)
         pre_q, pre_k = self._pre(qkv, rotary_emb)
-        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], pre=pre_k)   # [B, h, 1, 33, 32]: this chunk only
+        d = self.dim
+        state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], pre=pre_k, head_dim=d)  # [B, h, 1, d+1, d]: this chunk only
         if kv_cache is not None:
             past_vk, past_ks = kv_cache[0], kv_cache[1]
             if save_kv_cache:
-                kv_cache[0] = state[:, :, 0, :HEAD_DIM].clone()
-                kv_cache[1] = state[:, :, 0, HEAD_DIM:].clone()
+                kv_cache[0] = state[:, :, 0, :d].clone()
+                kv_cache[1] = state[:, :, 0, d:].clone()
             if past_vk is not None and past_ks is not None:
-                state[:, :, 0, :HEAD_DIM] += past_vk.to(state)
-                state[:, :, 0, HEAD_DIM:] += past_ks.to(state)
+                state[:, :, 0, :d] += past_vk.to(state)
+                state[:, :, 0, d:] += past_ks.to(state)
         out = self.proj(ops.linattn_apply(qkv[:, :, 0], state, self.eps, pre=pre_q))
         if kv_cache is not None:
             return out, kv_cache

@@ -24,14 +24,14 @@ def check(out, ref, what=""):
     assert mx <= 2e-2 and rl <= 1e-2, f"{what}: max-abs {mx:.3e} rel-L2 {rl:.3e}"
 
 
-def freqs(N, seed=0):
-    """Unit complex rotary factors [1, 1, N, 16], as the reference passes rotary_emb."""
-    theta = torch.rand(N, 16, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * 6.283
+def freqs(N, seed=0, head_dim=32):
+    """Unit complex rotary factors [1, 1, N, head_dim/2], as the reference passes rotary_emb."""
+    theta = torch.rand(N, head_dim // 2, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * 6.283
     return torch.polar(torch.ones_like(theta), theta)[None, None]
 
 
-def make(cls_name, C, qk_norm, seed):
-    heads = C // 32
+def make(cls_name, C, qk_norm, seed, head_dim=32):
+    heads = C // head_dim
     om = getattr(O, cls_name)(C, C, heads=heads, eps=1e-8, qk_norm=qk_norm)
     g = torch.Generator().manual_seed(seed)
     with torch.no_grad():
@@ -77,6 +77,46 @@ def test_litela_relu_rope(cuda, B, N, C, qk_norm, rot):
         out = hm(x.to(cuda), rotary_emb=None if f is None else f.to(cuda))
     assert out.dtype == torch.bfloat16 and out.shape == (B, N, C)
     check(out, ref, f"LiteLAReLURope norm={qk_norm} rope={rot}")
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
+@pytest.mark.parametrize("B,N,C", [(2, 640, 224), (1, 4096, 2240)])
+def test_litela_relu_rope_head_dim_112(cuda, B, N, C, qk_norm):
+    """The video configurations' linear_head_dim = 112 (2240 = 20 heads of 112)."""
+    om, hm = make("LiteLAReLURope", C, qk_norm, seed=N, head_dim=112)
+    hm = hm.to(cuda)
+    assert hm.dim == 112
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(1)).bfloat16()
+    f = freqs(N, head_dim=112)
+    with torch.no_grad():
+        ref = ref64(om, x, rotary_emb=f)
+        out = hm(x.to(cuda), rotary_emb=f.to(cuda))
+    check(out, ref, f"LiteLAReLURope d=112 norm={qk_norm}")
+
+
+def test_cached_stream_head_dim_112(cuda):
+    """Streaming chunks with 112-wide heads: each step against the oracle's cached module, and the saved state
+    has the reference's kv_cache shapes."""
+    B, hw, C = 1, 48, 224
+    om, hm = make("CachedCausalAttention", C, True, seed=6, head_dim=112)
+    hm = hm.to(cuda)
+    o64 = copy.deepcopy(om).double()
+    starts = [0, 2, 3, 5]
+    N = starts[-1] * hw
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(7)).bfloat16()
+    fr = freqs(N, 8, head_dim=112)
+    acc, acc_ref = None, None
+    with torch.no_grad():
+        for a, b in zip(starts[:-1], starts[1:]):
+            xs, fs = x[:, a * hw:b * hw], fr[:, :, a * hw:b * hw]
+            cache = [None, None] if acc is None else [acc[0], acc[1]]
+            out, cache = hm(xs.to(cuda), rotary_emb=fs.to(cuda), save_kv_cache=True, kv_cache=cache)
+            assert cache[0].shape == (B, 2, 112, 112) and cache[1].shape == (B, 2, 1, 112)
+            acc = S.accumulate_kv_cache(acc, cache)
+            cache_ref = [None, None] if acc_ref is None else [acc_ref[0], acc_ref[1]]
+            ref, cache_ref = o64(xs.double(), rotary_emb=fs, save_kv_cache=True, kv_cache=cache_ref)
+            acc_ref = cache_ref if acc_ref is None else [acc_ref[0] + cache_ref[0], acc_ref[1] + cache_ref[1]]
+            check(out, ref, f"cached chunk {a}:{b} d=112")
 
 
 def test_rotation_is_numerator_only_and_unit_rotation_is_identity(cuda):

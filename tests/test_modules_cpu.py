@@ -43,7 +43,8 @@ def test_qk_norm_keys():
 
 def test_unsupported_options_fail_loudly():
     with pytest.raises(NotImplementedError):
-        S.LiteLA(224, 224, dim=112)
+        S.LiteLA(128, 128, dim=64)          # head dims with kernels: 32 and 112
+    assert S.LiteLA(224, 224, dim=112).heads == 2
     with pytest.raises(NotImplementedError):
         S.GLUMBConv(64, 160, dilation=2)
     with pytest.raises(NotImplementedError):
