@@ -261,6 +261,12 @@ __global__ __launch_bounds__(256) void reduce112_kernel(const float* partial, fl
 
 // ----------------------------------------------------------------------------
 // phase 2.  1-D grid over (batch, chunk, token range, head), head fastest; block 256.
+//
+// The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
+// only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
+// (transforms applied once, here) into an LDS tile, every wave takes its MFMA B operands from that
+// tile, results go to an LDS output tile and leave as whole rows again.  Tiles are double buffered,
+// the next tile's loads are in flight during the MFMAs: one barrier per step.
 // ----------------------------------------------------------------------------
 __device__ __forceinline__ void split3_112(const float x[8], u32x4_t out[3]) {
   uint32_t hi[8], mid[8], lo[8];
@@ -280,6 +286,10 @@ __device__ __forceinline__ void split3_112(const float x[8], u32x4_t out[3]) {
 }
 
 constexpr int APPLY_TOKENS = 256;  // tokens per workgroup
+constexpr int TT = 32;             // tokens per step
+constexpr int QROW = 120;          // LDS row stride of the 16-bit tiles, elements: 240 B = 60 banks, so the 16 tokens
+                                   // of a b128 operand read land on 16 disjoint groups of 4 banks
+constexpr int OROW32 = 116;        // row stride of the fp32 output tile, floats (same argument: 116 % 64 = 52)
 
 template <bool OUT_F32, bool PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
@@ -288,7 +298,11 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
                                                        int n_chunks, int xranges, int64_t q_stride_b,
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  constexpr int NQ = PRE ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
+  constexpr int OT = OUT_F32 ? TT * OROW32 * 2 : TT * QROW;  // output tile, in 16-bit units
+  __shared__ __attribute__((aligned(16))) uint16_t lds_q[2 * NQ * TT * QROW];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_o[2 * OT];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   int head, bx, c, b;
   {
     int rest = blockIdx.x;
@@ -299,8 +313,9 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
   const int t0 = cr.begin + bx * APPLY_TOKENS;
   const int t1 = min(cr.end, t0 + APPLY_TOKENS);
-  if (t0 >= t1) return;  // no barriers in this kernel
+  if (t0 >= t1) return;  // uniform over the workgroup
   const int n = lane & 15, g = lane >> 4;
+  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
 
   // A operands.  MFMA 16x16x32: A lane -> row lane%16, k = 8*(lane/16)+e.  Row r of row block rb of this
   // wave is output channel 32*wave + 8*(r/4) + 4*rb + r%4, so that a lane (token n, group g') ends up
@@ -333,65 +348,132 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
     }
   }
 
-  const uint16_t* qp = Q + (int64_t)b * q_stride_b + head * DH + 8 * g;
+  // tile load mapping: piece id = tid + 256 i (i < 2, id < 448): token id / 14, 16-byte piece id % 14
+  int ld_tok[2], ld_ch[2];
+  bool ld_ok[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int id = tid + 256 * i;
+    ld_ok[i] = id < TT * NCH;
+    ld_tok[i] = id / NCH;
+    ld_ch[i] = id - ld_tok[i] * NCH;
+  }
+  const uint16_t* qp = Q + (int64_t)b * q_stride_b + head * DH;
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
-  u32x4_t qw[4] = {zero4, zero4, zero4, zero4};
+  const f32x4_t zerof = {0.f, 0.f, 0.f, 0.f};
+  u32x4_t qreg[2], qw[2] = {zero4, zero4};
+  float rin[2] = {0.f, 0.f};
+  f32x4_t cs[2][2] = {{zerof, zerof}, {zerof, zerof}};
   if (has_norm) {
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-      if (kb * 32 + 8 * g < DH) qw[kb] = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + kb * 32 + 8 * g);
+    for (int i = 0; i < 2; ++i)
+      if (ld_ok[i]) qw[i] = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[i] * 8);
   }
-  const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
-  for (int t = t0; t < t1; t += 16) {
-    const int tok = t + n;
-    const bool tok_ok = tok < t1;
-    u32x4_t qd[4], qb[4];
-    const float rin = has_norm && tok_ok ? pre.rinv[(int64_t)b * N + tok] : 0.f;
+  auto issue = [&](int t) {
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      const bool ok = tok_ok && kb * 32 + 8 * g < DH;
-      u32x4_t x = ok ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + kb * 32) : zero4;
-      if (has_norm) x = rms_scale8(x, rin, qw[kb]);
-      x = relu_pk16(x);
-      qd[kb] = x;  // denominator operand (unrotated)
-      if (has_rope && ok) {
-        const float* rp = pre.rope + ((int64_t)tok * (DH / 2) + (kb * 4 + g) * 4) * 2;
-        x = rope8(x, *reinterpret_cast<const f32x4_t*>(rp), *reinterpret_cast<const f32x4_t*>(rp + 4));
+    for (int i = 0; i < 2; ++i) {
+      const int tok = t + ld_tok[i];
+      const bool ok = ld_ok[i] && tok < t1;
+      qreg[i] = ok ? *reinterpret_cast<const u32x4_t*>(qp + (int64_t)tok * q_stride_n + ld_ch[i] * 8) : zero4;
+      if (has_norm) rin[i] = ok ? pre.rinv[(int64_t)b * N + tok] : 0.f;
+      if (has_rope) {
+        const float* rp = pre.rope + ((int64_t)min(tok, t1 - 1) * (DH / 2) + ld_ch[i] * 4) * 2;
+        cs[i][0] = ok ? *reinterpret_cast<const f32x4_t*>(rp) : zerof;
+        cs[i][1] = ok ? *reinterpret_cast<const f32x4_t*>(rp + 4) : zerof;
       }
-      qb[kb] = x;  // numerator operand
     }
-    f32x4_t acc[3];
+  };
+  auto stage = [&](int buf) {  // registers -> LDS tile(s); tokens past the range are zeros
+    uint16_t* td = lds_q + buf * NQ * TT * QROW;  // unrotated: the denominator operand (and the numerator without rope)
 #pragma unroll
-    for (int rb = 0; rb < 3; ++rb) {
-      f32x4_t s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int term = NT - 1; term >= 0; --term)  // smallest term first
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb) s = mfma_16x16x32_bf16(a[rb][kb][term], rb < 2 ? qb[kb] : qd[kb], s);
-      acc[rb] = s;
+    for (int i = 0; i < 2; ++i) {
+      if (!ld_ok[i]) continue;
+      u32x4_t x = qreg[i];
+      if (has_norm) x = rms_scale8(x, rin[i], qw[i]);
+      x = relu_pk16(x);
+      *reinterpret_cast<u32x4_t*>(td + ld_tok[i] * QROW + ld_ch[i] * 8) = x;
+      if (has_rope)
+        *reinterpret_cast<u32x4_t*>(td + TT * QROW + ld_tok[i] * QROW + ld_ch[i] * 8) = rope8(x, cs[i][0], cs[i][1]);
     }
-    if (tok_ok && och < DH) {
-      const float den = acc[2][0] + eps;
-      const int64_t o_off = (int64_t)b * o_stride_b + (int64_t)tok * o_stride_n + head * DH + och;
-      if (OUT_F32) {
-        f32x4_t o0, o1;
+  };
+
+  const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
+  issue(t0);
+  stage(0);
+  if (t0 + TT < t1) issue(t0 + TT);
+  __syncthreads();
+  int buf = 0;
+  for (int t = t0; t < t1; t += TT, buf ^= 1) {
+    const uint16_t* td = lds_q + buf * NQ * TT * QROW;
+    const uint16_t* tb = has_rope ? td + TT * QROW : td;
+    uint16_t* to = lds_o + buf * OT;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          o0[s] = acc[0][s] / den;
-          o1[s] = acc[1][s] / den;
+    for (int ss = 0; ss < TT / 16; ++ss) {
+      u32x4_t qd[4], qb[4];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const bool ok = kb * 4 + g < NCH;  // pieces 14, 15 of the padded k range: zero, whatever the tile holds there
+        const int off = (16 * ss + n) * QROW + (kb * 4 + g) * 8;
+        qb[kb] = ok ? *reinterpret_cast<const u32x4_t*>(tb + off) : zero4;
+        if (PRE) qd[kb] = ok ? *reinterpret_cast<const u32x4_t*>(td + off) : zero4;
+      }
+      f32x4_t acc[3];
+#pragma unroll
+      for (int rb = 0; rb < 3; ++rb) {
+        f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int term = NT - 1; term >= 0; --term)  // smallest term first
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb) s = mfma_16x16x32_bf16(a[rb][kb][term], (PRE && rb == 2) ? qd[kb] : qb[kb], s);
+        acc[rb] = s;
+      }
+      if (och < DH) {
+        const float den = acc[2][0] + eps;
+        if (OUT_F32) {
+          f32x4_t o0, o1;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            o0[s] = acc[0][s] / den;
+            o1[s] = acc[1][s] / den;
+          }
+          float* op = reinterpret_cast<float*>(to) + (16 * ss + n) * OROW32 + och;
+          *reinterpret_cast<f32x4_t*>(op) = o0;
+          *reinterpret_cast<f32x4_t*>(op + 4) = o1;
+        } else {
+          const float inv = __builtin_amdgcn_rcpf(den);
+          u32x4_t o;
+          o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
+          o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
+          o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
+          o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
+          *reinterpret_cast<u32x4_t*>(to + (16 * ss + n) * QROW + och) = o;
         }
-        float* op = reinterpret_cast<float*>(out) + o_off;
-        *reinterpret_cast<f32x4_t*>(op) = o0;
-        *reinterpret_cast<f32x4_t*>(op + 4) = o1;
-      } else {
-        const float inv = __builtin_amdgcn_rcpf(den);
-        u32x4_t o;
-        o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
-        o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
-        o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
-        o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
-        *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + o_off) = o;
+      }
+    }
+    // next tile: registers -> the other q tile (its last readers passed the previous barrier); loads of the one after
+    if (t + TT < t1) {
+      stage(buf ^ 1);
+      if (t + 2 * TT < t1) issue(t + 2 * TT);
+    }
+    __syncthreads();
+    // this step's output tile leaves as whole rows (it is next written two steps from now, behind the next barrier)
+    if (OUT_F32) {
+      float* ob = reinterpret_cast<float*>(out) + (int64_t)b * o_stride_b + head * DH;
+      const float* tf = reinterpret_cast<const float*>(to);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int id = tid + 256 * i, tok = id / (2 * NCH), piece = id - tok * (2 * NCH);
+        if (id < TT * 2 * NCH && t + tok < t1)
+          *reinterpret_cast<f32x4_t*>(ob + (int64_t)(t + tok) * o_stride_n + piece * 4) =
+              *reinterpret_cast<const f32x4_t*>(tf + tok * OROW32 + piece * 4);
+      }
+    } else {
+      uint16_t* ob = reinterpret_cast<uint16_t*>(out) + (int64_t)b * o_stride_b + head * DH;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (ld_ok[i] && t + ld_tok[i] < t1)
+          *reinterpret_cast<u32x4_t*>(ob + (int64_t)(t + ld_tok[i]) * o_stride_n + ld_ch[i] * 8) =
+              *reinterpret_cast<const u32x4_t*>(to + ld_tok[i] * QROW + ld_ch[i] * 8);
       }
     }
   }
