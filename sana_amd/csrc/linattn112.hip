@@ -23,8 +23,25 @@ constexpr int SE = (DH + 1) * DH;       // 12656 state elements per (batch, head
 constexpr int NCH = DH / 8;             // 14 16-byte chunks per token and head
 constexpr int TILE = 32;
 
+// Workgroup index -> (unit of four adjacent heads, head within it).  Four 224-byte head rows are seven whole
+// 128-byte lines; a single head's row shares its first / last line with a neighbour.  Workgroup i runs on XCD
+// i % 8, so the four heads of a unit take consecutive slots of ONE XCD: the shared lines are then fetched into
+// one L2, once, instead of into two.  Returns false for the padding of the grid.
+struct HeadUnit {
+  int unit, head;
+};
+__device__ __forceinline__ bool head_unit(int idx, int units, int h, HeadUnit& u) {
+  const int xcd = idx & 7, slot = idx >> 3;
+  const int hgroups = (h + 3) >> 2;
+  const int un = (slot >> 2) * 8 + xcd;
+  u.unit = un / hgroups;
+  u.head = (un - u.unit * hgroups) * 4 + (slot & 3);
+  return un < units * hgroups && u.head < h;
+}
+inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) / 4) + 7) / 8 * 8 * 4; }
+
 // ----------------------------------------------------------------------------
-// phase 1.  grid: x = token splits, y = n_chunks, z = B * h; block 256.
+// phase 1.  1-D grid over units (batch, chunk, token split) x heads, see head_unit; block 256.
 // partial[(bh * n_chunks + c) * nsplit + split][SE]
 // ----------------------------------------------------------------------------
 constexpr int LR = 160;  // LDS tile row stride in elements: 320 B puts the two token groups of a read 16 banks apart
@@ -35,12 +52,14 @@ template <typename T, bool PRE>
 __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
                                                        float* __restrict__ partial,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int nsplit, int split_tokens, int64_t stride_b,
-                                                       int64_t stride_n, const QkPre pre) {
+                                                       int n_chunks, int nsplit, int split_tokens, int units,
+                                                       int64_t stride_b, int64_t stride_n, const QkPre pre) {
   __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int b = blockIdx.z / h, head = blockIdx.z % h;
-  const int c = blockIdx.y, split = blockIdx.x;
+  HeadUnit hu;
+  if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
+  const int head = hu.head;
+  const int split = hu.unit % nsplit, c = (hu.unit / nsplit) % n_chunks, b = hu.unit / (nsplit * n_chunks);
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
   const int t0 = cr.begin + split * split_tokens;
   const int t1 = min(cr.end, t0 + split_tokens);
@@ -260,7 +279,7 @@ __global__ __launch_bounds__(256) void reduce112_kernel(const float* partial, fl
 }
 
 // ----------------------------------------------------------------------------
-// phase 2.  1-D grid over (batch, chunk, token range, head), head fastest; block 256.
+// phase 2.  1-D grid over units (batch, chunk, token range) x heads, see head_unit; block 256.
 //
 // The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
 // only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
@@ -295,7 +314,7 @@ template <bool OUT_F32, bool PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
                                                        void* __restrict__ out,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int xranges, int64_t q_stride_b,
+                                                       int n_chunks, int xranges, int units, int64_t q_stride_b,
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
   constexpr int NQ = PRE ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
@@ -303,13 +322,10 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   __shared__ __attribute__((aligned(16))) uint16_t lds_q[2 * NQ * TT * QROW];
   __shared__ __attribute__((aligned(16))) uint16_t lds_o[2 * OT];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  int head, bx, c, b;
-  {
-    int rest = blockIdx.x;
-    head = rest % h, rest /= h;
-    bx = rest % xranges, rest /= xranges;
-    c = rest % n_chunks, b = rest / n_chunks;
-  }
+  HeadUnit hu;
+  if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
+  const int head = hu.head;
+  const int bx = hu.unit % xranges, c = (hu.unit / xranges) % n_chunks, b = hu.unit / (xranges * n_chunks);
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
   const int t0 = cr.begin + bx * APPLY_TOKENS;
   const int t1 = min(cr.end, t0 + APPLY_TOKENS);
@@ -485,7 +501,7 @@ struct Plan112 {
 Plan112 plan112(int B, int h, int n_chunks, int max_chunk_tokens) {
   // one workgroup per CU (256 accumulator registers per wave: one wave per SIMD), splits of at least 512 tokens
   const int items = B * h * n_chunks;
-  int ns = (256 + items - 1) / items;
+  int ns = 256 / items;  // rounding down: 260 workgroups on 256 CUs would take two rounds
   const int cap = (max_chunk_tokens + 511) / 512;
   if (ns > cap) ns = cap;
   if (ns < 1) ns = 1;
@@ -515,12 +531,14 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
   if (!aligned16(workspace)) return SANA_ERR_ALIGN;
   float* part = static_cast<float*>(workspace);
-  dim3 grid(pl.nsplit, n_chunks, B * h);
+  const int64_t units = (int64_t)B * n_chunks * pl.nsplit, nwg = head_unit_grid(units, h);
+  if (nwg > 0x7fffffff) return SANA_ERR_SHAPE;
+  dim3 grid((unsigned)nwg);
   const uint16_t* kp = static_cast<const uint16_t*>(k);
   const uint16_t* vp = static_cast<const uint16_t*>(v);
 #define SANA_ST112(T, PRE)                                                                                        \
   hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(256), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
-                     pl.nsplit, pl.split_tokens, stride_b, stride_n, pre)
+                     pl.nsplit, pl.split_tokens, (int)units, stride_b, stride_n, pre)
   if (io_dtype == SANA_DT_F16) SANA_ST112(F16, false);
   else if (use_pre) SANA_ST112(BF16, true);
   else SANA_ST112(BF16, false);
@@ -546,13 +564,13 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
   const bool use_pre = pre.rinv || pre.rope;
   const int xranges = (max_chunk_tokens + APPLY_TOKENS - 1) / APPLY_TOKENS;
-  const int64_t total = (int64_t)xranges * n_chunks * B * h;
+  const int64_t units = (int64_t)xranges * n_chunks * B, total = head_unit_grid(units, h);
   if (total > 0x7fffffff) return SANA_ERR_SHAPE;
   dim3 grid((unsigned)total);
   const uint16_t* qp = static_cast<const uint16_t*>(q);
 #define SANA_AP112(F32, PRE)                                                                                         \
   hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
-                     xranges, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
+                     xranges, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
   if (out_dtype == SANA_DT_F32) {
     if (use_pre) SANA_AP112(true, true);
     else SANA_AP112(true, false);
