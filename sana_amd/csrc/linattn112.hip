@@ -71,12 +71,16 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
     *reinterpret_cast<u32x4_t*>(lds_k + row * LR + chunk * 8) = u32x4_t{0u, 0u, 0u, 0u};
   }
 
-  // load mapping: linear chunk id = lane + 64 i (i < 7): token id / 14, chunk id % 14 -- consecutive lanes
-  // read consecutive 16-byte pieces of a token's 224-byte head row
-  int ld_tok[7], ld_ch[7];
+  // load mapping, consecutive lanes on consecutive 16-byte pieces of a token's 224-byte head row:
+  //   plain      piece id = lane + 64 i (i < 7): token id / 14, piece id % 14
+  //   transforms lanes 0..55: token 4 i + lane / 14 (i < 8), piece lane % 14 -- a lane keeps ONE piece, so its norm
+  //              weights are loop invariant and its ksum is 8 registers; the other 8 lanes idle during loads
+  constexpr int NSLOT = PRE ? 8 : 7;
+  const bool lane_ok = !PRE || lane < 4 * NCH;
+  int ld_tok[NSLOT], ld_ch[NSLOT];
 #pragma unroll
-  for (int i = 0; i < 7; ++i) {
-    const int id = lane + 64 * i;
+  for (int i = 0; i < NSLOT; ++i) {
+    const int id = PRE ? 4 * NCH * i + lane : lane + 64 * i;
     ld_tok[i] = id / NCH;
     ld_ch[i] = id - ld_tok[i] * NCH;
   }
@@ -93,62 +97,76 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   float acck[4] = {0.f, 0.f, 0.f, 0.f};  // ksum of channel 32 jb + lane % 32 over this lane's token half
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  u32x4_t kreg[7], vreg[7];
+  // The next tile's loads (and what its transforms need: 1/rms, rotary factors) are in flight during the MFMAs
+  // of the current one.  (A second register set, two tiles ahead, measured no faster.)
+  u32x4_t kreg[NSLOT], vreg[NSLOT];
+  float rin[PRE ? NSLOT : 1];
+  f32x4_t cs[PRE ? NSLOT : 1][2];
+  u32x4_t kw = zero4;
+  if (has_norm && lane_ok) kw = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[0] * 8);
+  // Buffer loads: a resource ends with the last token of the range, so pieces of tokens past it (and everything
+  // of the idle lanes, whose offsets start at 2^31) read as zeros -- no branches or selects around the loads.
+  // The range check covers the vector offset only, so the tile's part of the address goes there.
+  const int row_b = (int)stride_n * 2;
+  const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(kbase), 0, (int)(((int64_t)(t1 - 1) * stride_n + DH) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(vbase), 0, (int)(((int64_t)(t1 - 1) * stride_n + DH) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(has_norm ? pre.rinv + (int64_t)b * N : nullptr), 0, has_norm ? t1 * 4 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(pre.rope), 0, has_rope ? t1 * (DH * 4) : 0, 0x00020000);
+  const int idle = (int)0x80000000u;
+  int voff[NSLOT];
+#pragma unroll
+  for (int i = 0; i < NSLOT; ++i) voff[i] = lane_ok ? ld_tok[i] * row_b + ld_ch[i] * 16 : idle;
   auto issue_loads = [&](int tile) {
 #pragma unroll
-    for (int i = 0; i < 7; ++i) {
-      const int tok = tile + ld_tok[i];
-      if (tok < t1) {
-        kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n + ld_ch[i] * 8);
-        vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n + ld_ch[i] * 8);
-      } else {
-        kreg[i] = zero4;
-        vreg[i] = zero4;
+    for (int i = 0; i < NSLOT; ++i) {
+      const int off = tile * row_b + voff[i];
+      kreg[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, off, 0, 0));
+      vreg[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, off, 0, 0));
+      if (PRE) {
+        const int tok = lane_ok ? tile + ld_tok[i] : idle / (DH * 4);
+        if (has_norm) rin[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_r, tok * 4, 0, 0));
+        if (has_rope) {
+          const int ro = tok * (DH * 4) + ld_ch[i] * 32;
+          cs[i][0] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_c, ro, 0, 0));
+          cs[i][1] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_c, ro + 16, 0, 0));
+        }
       }
     }
   };
   // PRE: the MFMA operands in LDS are rotated, ksum needs the unrotated values: a second, unrotated
-  // copy of the K tile would double the LDS traffic, so ksum is accumulated per lane, load slot and
-  // channel here and folded over lanes once at the end
-  float ks8[PRE ? 7 : 1][8];
-  if (PRE) {
-#pragma unroll
-    for (int i = 0; i < 7; ++i)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) ks8[i][e] = 0.f;
-  }
+  // copy of the K tile would double the LDS traffic, so ksum is accumulated per lane and channel
+  // here and folded over the lanes that share a piece once at the end
+  float ks8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  int tile = t0 + wave * TILE;
-  if (tile < t1) issue_loads(tile);
+  const int tile0 = t0 + wave * TILE;
+  if (tile0 < t1) issue_loads(tile0);
   // operand read mapping: lane -> channel j = lane%32 of a 32-channel block, k-group g = lane/32;
   // element r of k-step s is token 16*s + 2*r + g of the tile (both operands use the same bijection)
   const int j = lane & 31, g = lane >> 5;
-  for (; tile < t1; tile += 4 * TILE) {
+  for (int tile = tile0; tile < t1; tile += 4 * TILE) {
 #pragma unroll
-    for (int i = 0; i < 7; ++i) {
+    for (int i = 0; i < NSLOT; ++i) {
       u32x4_t kk = kreg[i];
       if (PRE) {
-        const bool tok_ok = tile + ld_tok[i] < t1;
-        const int tok = min(tile + ld_tok[i], t1 - 1);
-        if (has_norm) {
-          const u32x4_t kw = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[i] * 8);
-          kk = rms_scale8(kk, tok_ok ? pre.rinv[(int64_t)b * N + tok] : 0.f, kw);
-        }
+        if (has_norm) kk = rms_scale8(kk, rin[i], kw);
         kk = relu_pk16(kk);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          ks8[i][2 * e] += bf16_lo(kk[e]);
-          ks8[i][2 * e + 1] += bf16_hi(kk[e]);
+          ks8[2 * e] += bf16_lo(kk[e]);
+          ks8[2 * e + 1] += bf16_hi(kk[e]);
         }
-        if (has_rope) {
-          const float* rp = pre.rope + ((int64_t)tok * (DH / 2) + ld_ch[i] * 4) * 2;
-          kk = rope8(kk, *reinterpret_cast<const f32x4_t*>(rp), *reinterpret_cast<const f32x4_t*>(rp + 4));
-        }
+        if (has_rope) kk = rope8(kk, cs[i][0], cs[i][1]);
       } else {
         kk = relu_pk16(kk);
       }
-      *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
-      *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
+      if (lane_ok) {
+        *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
+        *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
+      }
     }
     if (tile + 4 * TILE < t1) issue_loads(tile + 4 * TILE);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
@@ -181,22 +199,22 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
   }
 
   if (PRE) {
-    // load slot i of lane l held chunk (l + 64 i) % 14 of tile token (l + 64 i) / 14: through the wave's own
-    // LDS region ([448 ids][8] floats = 14 KB), then channel 32 jb + j sums its 32 tokens in a fixed order
+    // lanes l, l + 14, l + 28, l + 42 hold the same piece of different tokens: through the wave's own LDS
+    // region ([56 lanes][8] floats), then channel 32 jb + j adds its four entries, two per token half g
     float* fold = reinterpret_cast<float*>(lds_k);
-#pragma unroll
-    for (int i = 0; i < 7; ++i) {
-      f32x4_t lo = {ks8[i][0], ks8[i][1], ks8[i][2], ks8[i][3]}, hi = {ks8[i][4], ks8[i][5], ks8[i][6], ks8[i][7]};
-      *reinterpret_cast<f32x4_t*>(fold + (lane + 64 * i) * 8) = lo;
-      *reinterpret_cast<f32x4_t*>(fold + (lane + 64 * i) * 8 + 4) = hi;
+    if (lane_ok) {
+      *reinterpret_cast<f32x4_t*>(fold + lane * 8) = f32x4_t{ks8[0], ks8[1], ks8[2], ks8[3]};
+      *reinterpret_cast<f32x4_t*>(fold + lane * 8 + 4) = f32x4_t{ks8[4], ks8[5], ks8[6], ks8[7]};
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
       const int ch = jb * 32 + j;
       float sum = 0.f;
-      if (ch < DH)
-        for (int tk = 16 * g; tk < 16 * g + 16; ++tk) sum += fold[(tk * NCH + (ch >> 3)) * 8 + (ch & 7)];
+      if (ch < DH) {
+        const float* f0 = fold + ((2 * g) * NCH + (ch >> 3)) * 8 + (ch & 7);
+        sum = f0[0] + f0[NCH * 8];
+      }
       acck[jb] = sum;
     }
   }
@@ -526,6 +544,8 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   if (io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
   const bool use_pre = pre.rinv || pre.rope;
   if (use_pre && io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  // the kernel addresses one batch entry's tokens with 32-bit byte offsets (buffer loads)
+  if ((int64_t)N * stride_n * 2 >= (int64_t)1 << 31 || (int64_t)N * DH * 4 >= (int64_t)1 << 31) return SANA_ERR_SHAPE;
   const Plan112 pl = plan112(B, h, n_chunks, max_chunk_tokens);
   const size_t need = workspace_bytes112(B, h, n_chunks, max_chunk_tokens);
   if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
