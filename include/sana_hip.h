@@ -10,7 +10,9 @@
  *   - Return value: SANA_OK (0) or a negative SANA_ERR_* code.  Nothing is
  *     launched when an error is returned.  sana_hip_strerror() names a code.
  *   - Strides are in ELEMENTS of the io dtype.  The channel stride is always 1.
- *   - Channel c belongs to head c / d, lane c % d (d = head_dim = 32).
+ *   - Channel c belongs to head c / d, lane c % d.  d = head_dim is 32 (every io dtype;
+ *     the image models) or 112 (bf16 io, f16 for phase 1 only; the `linear_head_dim: 112`
+ *     video models); any other d returns SANA_ERR_SHAPE.
  *
  * The reference (NVlabs/Sana) has no native seam for this path: its seam is the
  * Python module API (attn_type / ffn_type selection,
@@ -74,6 +76,8 @@ const char* sana_hip_strerror(int code);
  *   workspace     at least sana_hip_linattn_workspace_bytes(...) bytes, 16-byte aligned
  *                 (may be NULL when that function returns 0)
  * Accumulation is fp32 and deterministic (fixed summation order, no atomics).
+ * d = 112 addresses the tokens of one batch entry with 32-bit byte offsets:
+ * N * stride_n * 2 must stay below 2^31 (SANA_ERR_SHAPE otherwise).
  */
 size_t sana_hip_linattn_workspace_bytes(int B, int h, int d, int n_chunks, int max_chunk_tokens,
                                         int io_dtype);
