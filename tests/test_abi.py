@@ -45,6 +45,14 @@ def test_argument_validation_needs_no_gpu():
     assert lib.sana_hip_linattn_state(16, 16, 16, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 7, None) == -6  # dtype
     assert lib.sana_hip_linattn_state(16, 18, 16, None, 0, 1, 16, 1, 32, 0, 32, None, 1, 16, 0, 1, None) == -3  # align
     assert lib.sana_hip_linattn_apply(16, 16, 16, 1, 16, 1, 32, 0, 32, 0, 32, None, 1, 16, 1e-8, 1, 2, None) == -6
+    # head_dim 112: bf16 only (f16 for phase 1), needs its workspace, 32-bit byte offsets inside a batch entry
+    F32, BF16, F16 = 0, 1, 2
+    assert lib.sana_hip_linattn_state(16, 16, 16, 16, 1 << 30, 1, 16, 1, 112, 0, 112, None, 1, 16, 0, F32, None) == -6
+    assert lib.sana_hip_linattn_state(16, 16, 16, None, 0, 1, 16, 1, 112, 0, 112, None, 1, 16, 0, BF16, None) == -4
+    assert lib.sana_hip_linattn_state(16, 16, 16, 16, 1 << 30, 1, 1 << 20, 1, 112, 0, 1 << 12, None, 1, 1 << 20, 0,
+                                      BF16, None) == -2
+    assert lib.sana_hip_linattn_state(16, 16, 16, 16, 1 << 30, 1, 16, 1, 112, 0, 96, None, 1, 16, 0, BF16, None) == -1
+    assert lib.sana_hip_linattn_apply(16, 16, 16, 1, 16, 1, 112, 0, 112, 0, 112, None, 1, 16, 1e-8, F16, F16, None) == -6
     assert lib.sana_hip_dwconv3x3_silu_gate(16, 16, None, 16, 1, 4, 4, 3, 1, 1, None) == -2  # odd Ch
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 20, 24, 24, 8, 0, None) == -2      # K % 8
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None) == -1      # bias epilogue, no bias
@@ -59,6 +67,9 @@ def test_workspace_query():
     # short sequences are never split (a split is at least 256 tokens): no workspace
     assert lib.sana_hip_linattn_workspace_bytes(16, 70, 32, 1, 256, 1) == 0
     assert lib.sana_hip_linattn_workspace_bytes(64, 70, 32, 4, 300, 1) == 0
+    # head_dim 112 always goes through per-split partial states: 20 heads at the video shape -> 12 splits
+    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 1, 32760, 1) == 20 * 12 * 113 * 112 * 4
+    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 64, 1, 32760, 1) == 0   # no kernel for this head dim
 
 
 def test_ops_refuse_cpu_tensors():
