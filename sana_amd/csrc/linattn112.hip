@@ -46,9 +46,11 @@ inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) /
 // ----------------------------------------------------------------------------
 constexpr int LR = 160;  // LDS tile row stride in elements: 320 B puts the two token groups of a read 16 banks apart
 constexpr int SMEM_BYTES = 2 * SE * 4;  // two fp32 states for the wave reduction (>= 4 waves x 2 tiles x 32 x LR x 2 B)
-static_assert(SMEM_BYTES >= 4 * 2 * TILE * LR * 2, "staging must fit");
+static_assert(SMEM_BYTES >= 4 * 2 * (TILE + 1) * LR * 2, "staging must fit");
 
-template <typename T, bool PRE>
+// PRE: on-load transforms, compile-time so that the tile code stays one branch-free block: bit 0 = q/k RMSNorm,
+// bit 1 = rotary embedding
+template <typename T, int PRE>
 __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
                                                        float* __restrict__ partial,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
@@ -63,30 +65,35 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
   const int t0 = cr.begin + split * split_tokens;
   const int t1 = min(cr.end, t0 + split_tokens);
-  uint16_t* lds_k = reinterpret_cast<uint16_t*>(smem) + wave * (2 * TILE * LR);
-  uint16_t* lds_v = lds_k + TILE * LR;
+  // tokens per tile: 32, or 16 with transforms (their operands -- rotary factors above all -- travel with the
+  // tile, and a 32-token tile of them does not fit the registers next to the accumulator)
+  constexpr int TT_ = PRE ? 16 : TILE;
+  constexpr int TROWS = TT_ + 1;  // one spare row per tile: where the idle lanes of the transform mapping write
+  uint16_t* lds_k = reinterpret_cast<uint16_t*>(smem) + wave * (2 * TROWS * LR);
+  uint16_t* lds_v = lds_k + TROWS * LR;
   // channels 112..127 of every tile row are written once, as zeros, and never again
-  for (int i = lane; i < 2 * TILE * 2; i += 64) {  // (2 tiles x 32 rows) x 2 chunks of 8; rows 32..63 are the V tile
+  for (int i = lane; i < 2 * TROWS * 2; i += 64) {  // (K rows, V rows) x 2 chunks of 8
     const int row = i >> 1, chunk = NCH + (i & 1);
     *reinterpret_cast<u32x4_t*>(lds_k + row * LR + chunk * 8) = u32x4_t{0u, 0u, 0u, 0u};
   }
 
   // load mapping, consecutive lanes on consecutive 16-byte pieces of a token's 224-byte head row:
   //   plain      piece id = lane + 64 i (i < 7): token id / 14, piece id % 14
-  //   transforms lanes 0..55: token 4 i + lane / 14 (i < 8), piece lane % 14 -- a lane keeps ONE piece, so its norm
-  //              weights are loop invariant and its ksum is 8 registers; the other 8 lanes idle during loads
-  constexpr int NSLOT = PRE ? 8 : 7;
+  //   transforms lanes 0..55: token 4 i + lane / 14 (i < 4), piece lane % 14 -- a lane keeps ONE piece, so its norm
+  //              weights are loop invariant and its ksum is 8 registers; the other 8 lanes load nothing (zeros)
+  //              and write them to the spare row
+  constexpr int NSLOT = PRE ? 4 : 7;
   const bool lane_ok = !PRE || lane < 4 * NCH;
   int ld_tok[NSLOT], ld_ch[NSLOT];
 #pragma unroll
   for (int i = 0; i < NSLOT; ++i) {
     const int id = PRE ? 4 * NCH * i + lane : lane + 64 * i;
-    ld_tok[i] = id / NCH;
-    ld_ch[i] = id - ld_tok[i] * NCH;
+    ld_tok[i] = lane_ok ? id / NCH : TT_;
+    ld_ch[i] = lane_ok ? id - (id / NCH) * NCH : lane - 4 * NCH;
   }
   const uint16_t* kbase = K + (int64_t)b * stride_b + head * DH;
   const uint16_t* vbase = V + (int64_t)b * stride_b + head * DH;
-  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
 
   f32x16_t acc[4][4];
 #pragma unroll
@@ -100,8 +107,8 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
   // The next tile's loads (and what its transforms need: 1/rms, rotary factors) are in flight during the MFMAs
   // of the current one.  (A second register set, two tiles ahead, measured no faster.)
   u32x4_t kreg[NSLOT], vreg[NSLOT];
-  float rin[PRE ? NSLOT : 1];
-  f32x4_t cs[PRE ? NSLOT : 1][2];
+  float rin[has_norm ? NSLOT : 1];
+  f32x4_t cs[has_rope ? NSLOT : 1][2];
   u32x4_t kw = zero4;
   if (has_norm && lane_ok) kw = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[0] * 8);
   // Buffer loads: a resource ends with the last token of the range, so pieces of tokens past it (and everything
@@ -142,12 +149,12 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
   // here and folded over the lanes that share a piece once at the end
   float ks8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  const int tile0 = t0 + wave * TILE;
+  const int tile0 = t0 + wave * TT_;
   if (tile0 < t1) issue_loads(tile0);
   // operand read mapping: lane -> channel j = lane%32 of a 32-channel block, k-group g = lane/32;
   // element r of k-step s is token 16*s + 2*r + g of the tile (both operands use the same bijection)
   const int j = lane & 31, g = lane >> 5;
-  for (int tile = tile0; tile < t1; tile += 4 * TILE) {
+  for (int tile = tile0; tile < t1; tile += 4 * TT_) {
 #pragma unroll
     for (int i = 0; i < NSLOT; ++i) {
       u32x4_t kk = kreg[i];
@@ -163,15 +170,13 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
       } else {
         kk = relu_pk16(kk);
       }
-      if (lane_ok) {
-        *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
-        *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
-      }
+      *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
+      *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
     }
-    if (tile + 4 * TILE < t1) issue_loads(tile + 4 * TILE);
+    if (tile + 4 * TT_ < t1) issue_loads(tile + 4 * TT_);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < TT_ / 16; ++s) {
       u32x4_t fk[4], fv[4];
 #pragma unroll
       for (int blk = 0; blk < 4; ++blk) {
@@ -328,14 +333,14 @@ constexpr int QROW = 120;          // LDS row stride of the 16-bit tiles, elemen
                                    // of a b128 operand read land on 16 disjoint groups of 4 banks
 constexpr int OROW32 = 116;        // row stride of the fp32 output tile, floats (same argument: 116 % 64 = 52)
 
-template <bool OUT_F32, bool PRE>
+template <bool OUT_F32, int PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
                                                        void* __restrict__ out,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
                                                        int n_chunks, int xranges, int units, int64_t q_stride_b,
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
-  constexpr int NQ = PRE ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
+  constexpr int NQ = (PRE & 2) ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
   constexpr int OT = OUT_F32 ? TT * OROW32 * 2 : TT * QROW;  // output tile, in 16-bit units
   __shared__ __attribute__((aligned(16))) uint16_t lds_q[2 * NQ * TT * QROW];
   __shared__ __attribute__((aligned(16))) uint16_t lds_o[2 * OT];
@@ -349,7 +354,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   const int t1 = min(cr.end, t0 + APPLY_TOKENS);
   if (t0 >= t1) return;  // uniform over the workgroup
   const int n = lane & 15, g = lane >> 4;
-  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
 
   // A operands.  MFMA 16x16x32: A lane -> row lane%16, k = 8*(lane/16)+e.  Row r of row block rb of this
   // wave is output channel 32*wave + 8*(r/4) + 4*rb + r%4, so that a lane (token n, group g') ends up
@@ -449,7 +454,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
         const bool ok = kb * 4 + g < NCH;  // pieces 14, 15 of the padded k range: zero, whatever the tile holds there
         const int off = (16 * ss + n) * QROW + (kb * 4 + g) * 8;
         qb[kb] = ok ? *reinterpret_cast<const u32x4_t*>(tb + off) : zero4;
-        if (PRE) qd[kb] = ok ? *reinterpret_cast<const u32x4_t*>(td + off) : zero4;
+        if (has_rope) qd[kb] = ok ? *reinterpret_cast<const u32x4_t*>(td + off) : zero4;
       }
       f32x4_t acc[3];
 #pragma unroll
@@ -458,7 +463,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
 #pragma unroll
         for (int term = NT - 1; term >= 0; --term)  // smallest term first
 #pragma unroll
-          for (int kb = 0; kb < 4; ++kb) s = mfma_16x16x32_bf16(a[rb][kb][term], (PRE && rb == 2) ? qd[kb] : qb[kb], s);
+          for (int kb = 0; kb < 4; ++kb) s = mfma_16x16x32_bf16(a[rb][kb][term], (has_rope && rb == 2) ? qd[kb] : qb[kb], s);
         acc[rb] = s;
       }
       if (och < DH) {
@@ -559,9 +564,12 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
 #define SANA_ST112(T, PRE)                                                                                        \
   hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(256), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
                      pl.nsplit, pl.split_tokens, (int)units, stride_b, stride_n, pre)
-  if (io_dtype == SANA_DT_F16) SANA_ST112(F16, false);
-  else if (use_pre) SANA_ST112(BF16, true);
-  else SANA_ST112(BF16, false);
+  const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+  if (io_dtype == SANA_DT_F16) SANA_ST112(F16, 0);
+  else if (mode == 3) SANA_ST112(BF16, 3);
+  else if (mode == 2) SANA_ST112(BF16, 2);
+  else if (mode == 1) SANA_ST112(BF16, 1);
+  else SANA_ST112(BF16, 0);
 #undef SANA_ST112
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
   const int64_t threads = (int64_t)B * h * SE;
@@ -582,7 +590,6 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
                     int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
                     hipStream_t s) {
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
-  const bool use_pre = pre.rinv || pre.rope;
   const int xranges = (max_chunk_tokens + APPLY_TOKENS - 1) / APPLY_TOKENS;
   const int64_t units = (int64_t)xranges * n_chunks * B, total = head_unit_grid(units, h);
   if (total > 0x7fffffff) return SANA_ERR_SHAPE;
@@ -591,12 +598,17 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
 #define SANA_AP112(F32, PRE)                                                                                         \
   hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
                      xranges, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
+  const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
   if (out_dtype == SANA_DT_F32) {
-    if (use_pre) SANA_AP112(true, true);
-    else SANA_AP112(true, false);
+    if (mode == 3) SANA_AP112(true, 3);
+    else if (mode == 2) SANA_AP112(true, 2);
+    else if (mode == 1) SANA_AP112(true, 1);
+    else SANA_AP112(true, 0);
   } else {
-    if (use_pre) SANA_AP112(false, true);
-    else SANA_AP112(false, false);
+    if (mode == 3) SANA_AP112(false, 3);
+    else if (mode == 2) SANA_AP112(false, 2);
+    else if (mode == 1) SANA_AP112(false, 1);
+    else SANA_AP112(false, 0);
   }
 #undef SANA_AP112
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
