@@ -42,7 +42,8 @@ constexpr int TILE = 32;                  // tokens per phase-1 tile
 // grid: x = nsplit, y = n_chunks, z = B * pairs;  block 256
 // dst: when nsplit == 1 the final state, else partial[(bh*n_chunks + c)*nsplit + split][1056]
 // ----------------------------------------------------------------------------
-template <typename T, bool PRE>
+// PRE: on-load transforms as compile-time bits (1 = q/k RMSNorm, 2 = rotary embedding)
+template <typename T, int PRE>
 __global__ __launch_bounds__(256) void linattn_state16_kernel(
     const uint16_t* __restrict__ K, const uint16_t* __restrict__ V, float* __restrict__ dst,
     const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int nsplit, int split_tokens,
@@ -81,15 +82,15 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
   }
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
   u32x4_t kreg[4], vreg[4];
   // PRE: per-token 1/rms and this lane's four (cos, sin) pairs travel with the tile; the norm weight
   // of the lane's 8 channels is loop-invariant; ksum is accumulated here, per lane and channel,
   // from the unrotated values (the MFMA operands in LDS are rotated).
-  float rin[4];
-  f32x4_t cs[4][2];
+  float rin[has_norm ? 4 : 1];
+  f32x4_t cs[has_rope ? 4 : 1][2];
   u32x4_t kw = zero4;
   float ks8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
   if (has_norm && ch_ok) kw = *reinterpret_cast<const u32x4_t*>(pre.weight + ld_ch);
   auto issue_loads = [&](int tile) {
 #pragma unroll
@@ -310,7 +311,7 @@ __device__ __forceinline__ void split3(const float x[8], u32x4_t out[3]) {
   }
 }
 
-template <bool OUT_F32, bool PRE>
+template <bool OUT_F32, int PRE>
 __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
     const uint16_t* __restrict__ Q, const float* __restrict__ state, void* __restrict__ out,
     const int32_t* __restrict__ chunk_starts, int N, int h, int n_chunks, int wg_tokens,
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
   }
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  const bool has_norm = PRE && pre.rinv != nullptr, has_rope = PRE && pre.rope != nullptr;
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
   u32x4_t qw[2] = {zero4, zero4};
   if (has_norm) {
 #pragma unroll
@@ -387,8 +388,8 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
   for (int hh = 0; hh < 2; ++hh) slot_r[hh] = 16 * (8 * n + ((4 * hh + g) ^ ((n >> 1) & 7)));
   for (int t = t0; t < t1; t += 16 * U) {
     u32x4_t raw[U][2];
-    float rin[U];
-    f32x4_t cs[U][2];
+    float rin[has_norm ? U : 1];
+    f32x4_t cs[has_rope ? U : 1][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -624,7 +625,6 @@ static int state_impl(const void* k, const void* v, float* state, void* workspac
                       int N, int h, int d, int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts,
                       int n_chunks, int max_chunk_tokens, int causal, int io_dtype, const QkPre pre, void* stream) {
   if (!k || !v || !state || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
-  const bool use_pre = pre.rinv || pre.rope;
   {
     const int rc = check_pre(pre, io_dtype);
     if (rc != SANA_OK) return rc;
@@ -658,18 +658,17 @@ static int state_impl(const void* k, const void* v, float* state, void* workspac
                        pl.split_tokens, stride_b, stride_n);
   } else {
     dim3 grid(pl.nsplit, n_chunks, B * ((h + 1) / 2));
-    if (io_dtype == SANA_DT_BF16 && use_pre)
-      hipLaunchKernelGGL((linattn_state16_kernel<BF16, true>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(k),
-                         static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,
-                         pl.split_tokens, stride_b, stride_n, pre);
-    else if (io_dtype == SANA_DT_BF16)
-      hipLaunchKernelGGL((linattn_state16_kernel<BF16, false>), grid, dim3(256), 0, s,
-                         static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v), dst, chunk_starts, N, h,
-                         n_chunks, pl.nsplit, pl.split_tokens, stride_b, stride_n, pre);
-    else
-      hipLaunchKernelGGL((linattn_state16_kernel<F16, false>), grid, dim3(256), 0, s,
-                         static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(v), dst, chunk_starts, N, h,
-                         n_chunks, pl.nsplit, pl.split_tokens, stride_b, stride_n, pre);
+    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+#define SANA_STATE16(T, PRE)                                                                                  \
+  hipLaunchKernelGGL((linattn_state16_kernel<T, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(k), \
+                     static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,           \
+                     pl.split_tokens, stride_b, stride_n, pre)
+    if (io_dtype == SANA_DT_F16) SANA_STATE16(F16, 0);
+    else if (mode == 3) SANA_STATE16(BF16, 3);
+    else if (mode == 2) SANA_STATE16(BF16, 2);
+    else if (mode == 1) SANA_STATE16(BF16, 1);
+    else SANA_STATE16(BF16, 0);
+#undef SANA_STATE16
   }
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
   const bool scan = causal && n_chunks > 1;
@@ -733,7 +732,6 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
                       int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre pre,
                       void* stream) {
   if (!q || !state || !out || B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
-  const bool use_pre = pre.rinv || pre.rope;
   {
     const int rc = check_pre(pre, io_dtype);
     if (rc != SANA_OK) return rc;
@@ -770,12 +768,17 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
   hipLaunchKernelGGL((linattn_apply_bf16_kernel<F32, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(q), \
                      state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,     \
                      o_stride_n, eps, pre, (int)gx, ngroups)
+    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
     if (out_dtype == SANA_DT_F32) {
-      if (use_pre) SANA_APPLY(true, true);
-      else SANA_APPLY(true, false);
+      if (mode == 3) SANA_APPLY(true, 3);
+      else if (mode == 2) SANA_APPLY(true, 2);
+      else if (mode == 1) SANA_APPLY(true, 1);
+      else SANA_APPLY(true, 0);
     } else {
-      if (use_pre) SANA_APPLY(false, true);
-      else SANA_APPLY(false, false);
+      if (mode == 3) SANA_APPLY(false, 3);
+      else if (mode == 2) SANA_APPLY(false, 2);
+      else if (mode == 1) SANA_APPLY(false, 1);
+      else SANA_APPLY(false, 0);
     }
 #undef SANA_APPLY
   } else {
