@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 2
+#define SANA_HIP_ABI_VERSION 3
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -234,6 +234,29 @@ int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_sc
 int sana_hip_layernorm_modulate(const void* x, const void* scale, const void* shift, void* out,
                                 int64_t M, int C, int64_t ldx, int64_t ldo,
                                 int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Temporal (t, 1) convolution over frames with full channel mixing, plus its residual, as ONE GEMM over a
+ * virtual im2col of the token-major buffer (no copy of the activations):
+ *
+ *   out[m][:] = X[m + (taps/2)*tap_rows][:] + sum_{t < taps} W[:, t*C:(t+1)*C] . X[m + t*tap_rows][:]
+ *
+ * for m < M, where rows of X at or past x_rows read as zero.  With tap_rows = tokens per frame this is
+ * `x + t_conv(x)` of GLUMBConvTemp.forward (diffusion/model/nets/basic_modules.py:250-264,
+ * t_conv = Conv2d(C, C, (3, 1), padding (1, 0), bias=False)) on the frames of one batch entry: X points
+ * at the frame in FRONT of the first output frame (zeros at the start of a sequence, the previous
+ * chunk's last frame for ChunkGLUMBConvTemp / CachedGLUMBConvTemp, :302-349 / :374-392), and x_rows =
+ * M + tap_rows ends the buffer behind the last output frame, which gives the zero padding on the right.
+ * Roundings as the reference's: the convolution result to bf16, then the sum to bf16.
+ *
+ *   X     bf16 rows of C channels, row stride ldx; x_rows >= M + (taps/2)*tap_rows rows exist
+ *   W     bf16 [C][taps*C], row stride ldw: W[o][t*C + i] = t_conv.weight[o][i][t][0]
+ *   out   bf16 [M][C], row stride ldo (must not overlap X)
+ *   taps  odd; C % 64 == 0; x_rows * ldx * 2 < 2^31
+ */
+int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,
+                            int64_t tap_rows, int64_t x_rows, int64_t ldx, int64_t ldw, int64_t ldo,
+                            void* stream);
 
 #ifdef __cplusplus
 }

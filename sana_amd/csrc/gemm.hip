@@ -58,6 +58,16 @@ struct EpiArgs {
 };
 #define SANA_EPI_GATE_RES 3
 
+// Virtual concatenation of the A operand along k: columns [t*kc, (t+1)*kc) of the GEMM's A are columns
+// [0, kc) of the matrix whose row m is row m + t*stride of the buffer (a convolution over rows as one GEMM,
+// without materialising its im2col matrix).  rows = rows of the buffer that exist, counted from A: reads
+// past them return zero (the convolution's zero padding on that side).
+struct Taps {
+  int kc;          // columns per tap, a multiple of the k-tile
+  int64_t stride;  // rows between taps
+  int64_t rows;
+};
+
 // 8 outputs of one row: accumulator (+bias) -> io dtype, per the epilogue kind (everything except
 // the gated residual, which needs the row's residual and gate and is applied at store time).
 template <int EPI>
@@ -322,11 +332,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 // Rows past M / N read as zero (buffer range check) and only feed outputs that are
 // never stored; the last k-tile runs just the k-steps that exist.  Needs K % 16 == 0 and K >= 64.
 // ============================================================================
-template <bool W8, int EPI, int NI>
+template <bool W8, int EPI, int NI, bool TAPS = false>
 __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
                                                     const float* __restrict__ scale, const EpiArgs ep,
                                                     uint16_t* __restrict__ C, int M, int N, int K, int64_t lda,
-                                                    int64_t ldw, int64_t ldc, int tiles_t, int tiles_c) {
+                                                    int64_t ldw, int64_t ldc, int tiles_t, int tiles_c,
+                                                    const Taps tp) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int total = tiles_t * tiles_c;
@@ -388,8 +399,15 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // address is scalar, so a load costs one vector add.  The resource ends with the last valid row's
   // K-th element: rows past M / N and anything past the end of the matrix read as zero instead of
   // faulting (k chunks past K inside the matrix read the next row: they are never multiplied).
+  // (TAPS: the resource ends with the buffer's last existing row instead, so a tap that reaches past it is zero)
+  const int64_t a_bytes = TAPS ? (tp.rows > m0 ? ((tp.rows - m0 - 1) * lda + tp.kc) * 2 : 0)
+                               : ((int64_t)a_last * lda + K) * 2;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(A + (int64_t)m0 * lda), 0, (int)(((int64_t)a_last * lda + K) * 2), 0x00020000);
+      const_cast<uint16_t*>(A + (int64_t)m0 * lda), 0, (int)a_bytes, 0x00020000);
+  // byte offset of k-tile k0 inside a row of A (TAPS: tap k0 / kc starts tp.stride rows further down)
+  const int tap_b = TAPS ? (int)(tp.stride * lda * 2) : 0;
+  auto a_koff = [&](int k0) { return TAPS ? (k0 / tp.kc) * tap_b + (k0 % tp.kc) * 2 : k0 * 2; };
+  int a_kb = 0, a_kin = 0;  // offset of the k-tile being requested, and its column inside the tap
   const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * (W8 ? 1 : 2)), 0,
       (int)(((int64_t)w_last * ldw + K) * (W8 ? 1 : 2)), 0x00020000);
@@ -398,7 +416,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int step_a = 32 * (int)ulda * 2, step_w = W8 ? 64 * (int)uldw : 32 * (int)uldw * 2;
   auto gload = [&](int q, int k0) {
     if (q < 8) {
-      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff_a + (q * step_a + k0 * 2), 0, 0);
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff_a + (q * step_a + (TAPS ? a_kb : k0 * 2)), 0, 0);
       rs[q] = __builtin_bit_cast(u32x4_t, v);
     } else {
       const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w + ((q - 8) * step_w + k0 * (W8 ? 1 : 2)), 0, 0);
@@ -435,6 +453,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // prologue: k-tile 0 -> stage 0, k-tile 1 in flight
 #pragma unroll
   for (int q = 0; q < NQ; ++q) gload(q, 0);
+  if (TAPS) a_kb = a_koff(BK);
 #pragma unroll
   for (int q = 0; q < (W8 ? 8 : NQ); ++q) lstore(q, 0);
   if (W8) {
@@ -443,6 +462,10 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   }
 #pragma unroll
   for (int q = 0; q < NQ; ++q) gload(q, BK);
+  if (TAPS) {
+    a_kb = a_koff(2 * BK);
+    a_kin = (2 * BK) % tp.kc;
+  }
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < NFR; ++q) fread(smem, 0, 0, q);
@@ -488,6 +511,14 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
           if (slot >= 10 && slot <= 2 + 8 * NI && (slot - 10) % 8 == 0) gload(8 + (slot - 10) / 8, (kt + 2) * BK);
         }
         SANA_G4_PIN();
+      }
+    }
+    if (TAPS) {  // the next iteration requests k-tile kt + 3
+      a_kin += BK;
+      a_kb += BK * 2;
+      if (a_kin >= tp.kc) {
+        a_kin -= tp.kc;
+        a_kb += tap_b - tp.kc * 2;
       }
     }
   }
@@ -565,8 +596,8 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     // one gate row serves the whole group unless a batch boundary runs through its 32 tokens
     const int m_first = m0 + wt * 128 + 32 * j;
     const int g_first = m_first / ep.rows_per_gate, g_last = min(m_first + 31, M - 1) / ep.rows_per_gate;
-    u32x4_t gate = {0u, 0u, 0u, 0u};
-    if (EPI == SANA_EPI_GATE_RES && o_live && m_first < M)
+    u32x4_t gate = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // no gate: 1.0, a plain residual add
+    if (EPI == SANA_EPI_GATE_RES && ep.gate && o_live && m_first < M)
       gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -589,7 +620,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       if (o_live && m < M) {
         if (EPI == SANA_EPI_GATE_RES) {
           u32x4_t g = gate;
-          if (g_first != g_last && m / ep.rows_per_gate != g_first)
+          if (ep.gate && g_first != g_last && m / ep.rows_per_gate != g_first)
             g = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
           o = gate_res8v(o, g, res[j][it]);
         }
@@ -613,12 +644,19 @@ int compute_units() {
 
 template <bool W8, int NI>
 int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N, int K,
-            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
+            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr) {
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + 64 * NI - 1) / (64 * NI);
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
+  const Taps none = {0, 0, 0};
+  if (taps) {  // only the bf16 gated-residual instance exists with taps
+    if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
+    hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, true>), grid, block, 0, s, a, W, scale, ep, c, M, N,
+                       K, lda, ldw, ldc, tiles_t, tiles_c, *taps);
+    return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+  }
 #define SANA_LAUNCH4(EPI)                                                                                         \
   hipLaunchKernelGGL((gemm4_kernel<W8, EPI, NI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
-                     tiles_t, tiles_c)
+                     tiles_t, tiles_c, none)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
     case SANA_EPI_BIAS: SANA_LAUNCH4(SANA_EPI_BIAS); break;
@@ -632,7 +670,7 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
 
 template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
-           int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
+           int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr) {
   const int64_t tiles_t = (M + BT - 1) / BT;
   if (tiles_t * ((N + 127) / 128) > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
@@ -644,9 +682,10 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
     const int64_t cu = compute_units();
     const int64_t t256 = tiles_t * ((N + 255) / 256), t192 = tiles_t * ((N + 191) / 192);
     const double cost256 = (double)((t256 + cu - 1) / cu) * 4.0, cost192 = (double)((t192 + cu - 1) / cu) * 3.0 * 1.04;
-    return cost192 < cost256 ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s)
-                             : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
+    return cost192 < cost256 ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps)
+                             : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps);
   }
+  if (taps) return SANA_ERR_SHAPE;
   const int tiles_c = (N + BC - 1) / BC;
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
 #define SANA_LAUNCH(EPI)                                                                                        \
@@ -727,4 +766,20 @@ SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const flo
   hipStream_t s = static_cast<hipStream_t>(stream);
   return w8 ? launch<true>(A, W, w8_scale, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s)
             : launch<false>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s);
+}
+
+SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,
+                                     int64_t tap_rows, int64_t x_rows, int64_t ldx, int64_t ldw, int64_t ldo,
+                                     void* stream) {
+  if (!X || !W || !out || M <= 0 || C <= 0 || taps <= 0 || !(taps & 1) || tap_rows <= 0) return SANA_ERR_ARG;
+  if (C % 64) return SANA_ERR_SHAPE;  // a tap is a whole number of k-tiles
+  if (x_rows < (taps / 2) * tap_rows + M) return SANA_ERR_ARG;  // the centre tap (= the residual) must exist for every row
+  if (ldx < C || ldw < (int64_t)taps * C || ldo < C) return SANA_ERR_ARG;
+  if (ldx % 8 || ldw % 8 || ldo % 8 || !aligned16(X) || !aligned16(W) || !aligned16(out)) return SANA_ERR_ALIGN;
+  if (x_rows * ldx * 2 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;  // 32-bit byte offsets inside the buffer
+  const uint16_t* x = static_cast<const uint16_t*>(X);
+  const EpiArgs e = {nullptr, nullptr, x + (taps / 2) * tap_rows * ldx, ldx, 0, M};
+  const Taps tp = {C, tap_rows, x_rows};
+  return launch<false>(X, W, nullptr, e, out, M, C, taps * C, ldx, ldw, ldo, SANA_EPI_GATE_RES,
+                       static_cast<hipStream_t>(stream), &tp);
 }

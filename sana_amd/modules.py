@@ -60,9 +60,10 @@ class HipLinear(nn.Linear):
                           getattr(self, "weight_q", None), getattr(self, "weight_scale", None), gate, residual)
 
 
-def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None, gate=None, residual=None):
+def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None, gate=None, residual=None, out=None):
     """y = epilogue(x @ W^T + b) over the last dim of x.  epilogue: None | "silu".
-    With ``gate`` [B, 1, C] and ``residual`` [B, N, C]: residual + gate * y (one fused kernel in bf16)."""
+    With ``gate`` [B, 1, C] and ``residual`` [B, N, C]: residual + gate * y (one fused kernel in bf16).
+    ``out``: a [rows, C_out] bf16 view to write into (bf16 GEMM without gate only)."""
     _no_grad_only(x, weight, bias)
     lead = x.shape[:-1]
     K = x.shape[-1]
@@ -80,9 +81,9 @@ def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None,
             bias = torch.zeros(weight_q.shape[0] if weight_q is not None else weight.shape[0],
                                dtype=torch.bfloat16, device=x.device)
         if weight_q is not None:
-            y = ops.gemm_w8a16(x2, weight_q, weight_scale, bias, epi)
+            y = ops.gemm_w8a16(x2, weight_q, weight_scale, bias, epi, out=out)
         else:
-            y = ops.gemm_bf16(x2, weight.reshape(weight.shape[0], -1), bias, epi)
+            y = ops.gemm_bf16(x2, weight.reshape(weight.shape[0], -1), bias, epi, out=out)
         return y.view(*lead, y.shape[-1])
     if not x.is_cuda:
         raise SanaHipError("the HIP path needs device tensors (no CPU path exists)")
@@ -404,8 +405,9 @@ class GLUMBConv(nn.Module):
     def forward(self, x: torch.Tensor, HW=None) -> torch.Tensor:
         return self.forward_gated(x, HW, None, None)
 
-    def forward_gated(self, x, HW, gate, residual) -> torch.Tensor:
-        """forward(x, HW), or residual + gate * forward(x, HW) fused into the point-conv GEMM."""
+    def forward_gated(self, x, HW, gate, residual, out=None) -> torch.Tensor:
+        """forward(x, HW), or residual + gate * forward(x, HW) fused into the point-conv GEMM.
+        ``out``: [B*N, C_out] bf16 view that receives the result (bf16 device path without gate only)."""
         _no_grad_only(x)
         B, N, C = x.shape
         if HW is None:
@@ -421,9 +423,8 @@ class GLUMBConv(nn.Module):
         u = hip_linear(x, ic.weight, ic.bias, "silu", getattr(ic, "weight_q", None), getattr(ic, "weight_scale", None))
         y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
                                     round_like_reference=self.round_like_reference)
-        out = hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
-                         getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual)
-        return out
+        return hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
+                          getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual, out)
 
     def quantize_w8_(self) -> "GLUMBConv":
         for conv in (self.inverted_conv.conv, self.point_conv.conv):
@@ -463,8 +464,64 @@ class GLUMBConvTemp(GLUMBConv):
         B, C, T, P = x_bcthw.shape
         return x_bcthw.permute(0, 2, 3, 1).reshape(B, T * P, C)
 
+    # -- the temporal conv as one GEMM over a virtual im2col of the token-major frames (bf16, 3 taps,
+    #    C % 64 == 0, no frame mask); anything else takes the stock convolution below
+    def _tconv_gemm_ok(self, x: torch.Tensor, kwargs) -> bool:
+        C = self.t_conv.out_channels
+        return (x.is_cuda and x.dtype == torch.bfloat16 and self.t_conv.weight.dtype == torch.bfloat16
+                and self.t_conv.kernel_size == (3, 1) and self.t_conv.in_channels == C and C % 64 == 0
+                and kwargs.get("frame_valid_mask") is None and not torch.is_grad_enabled())
+
+    def _tconv_weight(self) -> torch.Tensor:
+        """t_conv.weight [C, C, t, 1] -> [C, t*C] with k = tap * C + input channel (derived data, rebuilt when
+        the parameter changes; not part of the state_dict)."""
+        w = self.t_conv.weight
+        key = (w.data_ptr(), w._version, w.device)
+        cache = self.__dict__.get("_tconv_cache")
+        if cache is None or cache[0] != key:
+            with torch.no_grad():
+                w2 = w[:, :, :, 0].permute(0, 2, 1).reshape(w.shape[0], -1).contiguous()
+            cache = (key, w2)
+            self.__dict__["_tconv_cache"] = cache
+        return cache[1]
+
+    def _spatial_into_frames(self, x: torch.Tensor, HW) -> torch.Tensor:
+        """The per-frame Mix-FFN of x [B, T*P, C] written behind one spare frame: returns buf [B, (T+1)*P, C_out]
+        with buf[:, P:] = Mix-FFN(x) (the point-conv GEMM stores there directly when B == 1) and buf[:, :P]
+        left for the caller (the frame in front of frame 0)."""
+        if HW is None or len(HW) != 3:
+            raise ValueError("HW must be a tuple of (T, H, W)")
+        B, N, _ = x.shape
+        P = HW[1] * HW[2]
+        buf = x.new_empty(B, N + P, self.t_conv.out_channels)
+        if B == 1:
+            GLUMBConv.forward_gated(self, x, HW, None, None, out=buf[0, P:])
+        else:
+            buf[:, P:].copy_(GLUMBConv.forward_gated(self, x, HW, None, None))
+        return buf
+
+    def _tconv_residual(self, buf: torch.Tensor, HW, bounds, left: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """buf: [B, (T+1)*P, C] from :meth:`_spatial_into_frames`; bounds: first frame of every chunk and T; left:
+        the frame in front of frame 0 as tokens [B, P, C], or None for zeros.  A chunk sees the frame in front of
+        it and zeros behind it.  Returns y + t_conv(y) [B, T*P, C] for y = buf[:, P:]."""
+        B, _, C = buf.shape
+        T, P = HW[0], HW[1] * HW[2]
+        if left is None:
+            buf[:, :P].zero_()
+        else:
+            buf[:, :P].copy_(left)
+        out = buf.new_empty(B, T * P, C)
+        w2 = self._tconv_weight()
+        for b in range(B):
+            for f0, f1 in zip(bounds[:-1], bounds[1:]):
+                ops.tconv_residual(buf[b, f0 * P:(f1 + 1) * P], w2, (f1 - f0) * P, P, out=out[b, f0 * P:f1 * P])
+        return out
+
     def forward(self, x: torch.Tensor, HW=None, **kwargs) -> torch.Tensor:
         B = x.shape[0]
+        if self._tconv_gemm_ok(x, kwargs):
+            buf = self._spatial_into_frames(x, HW)
+            return self._tconv_residual(buf, HW, [0, HW[0]])
         xr = self._spatial_bcthw(x, HW)
         frame_mask = kwargs.get("frame_valid_mask", None)
         if frame_mask is not None:
@@ -484,6 +541,10 @@ class ChunkGLUMBConvTemp(GLUMBConvTemp):
         if chunk_index is None:
             chunk_index = [0]
         B = x.shape[0]
+        if self._tconv_gemm_ok(x, kwargs):
+            buf = self._spatial_into_frames(x, HW)
+            T = HW[0]
+            return self._tconv_residual(buf, HW, sorted({0, *(int(i) for i in chunk_index if 0 < int(i) < T), T}))
         xr = self._spatial_bcthw(x, HW)
         T = HW[0]
         frame_mask = kwargs.get("frame_valid_mask")
@@ -510,6 +571,17 @@ class CachedGLUMBConvTemp(GLUMBConvTemp):
     ``save_kv_cache``); returns ``(out, kv_cache)`` when a cache list is passed."""
 
     def forward(self, x: torch.Tensor, HW=None, save_kv_cache=False, kv_cache=None, **kwargs):
+        if self._tconv_gemm_ok(x, kwargs):
+            buf = self._spatial_into_frames(x, HW)
+            T, P = HW[0], HW[1] * HW[2]
+            left = None
+            if kv_cache is not None:
+                if kv_cache[-1] is not None:     # (B, C, frames, P): the last saved frame, as tokens
+                    left = kv_cache[-1][:, :, -1].to(buf).transpose(1, 2)
+                if save_kv_cache:                # saved un-convolved, in the reference's (B, C, 1, P) layout
+                    kv_cache[-1] = buf[:, T * P:].transpose(1, 2).unsqueeze(2).detach().clone()
+            out = self._tconv_residual(buf, HW, [0, T], left)
+            return (out, kv_cache) if kv_cache is not None else out
         xr = self._spatial_bcthw(x, HW)
         pad = self.t_conv.kernel_size[0] // 2
         x_in, padded = xr, 0

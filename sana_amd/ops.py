@@ -333,6 +333,34 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     return out.view(B, Ntok, C)
 
 
+def tconv_residual(xp: torch.Tensor, weight: torch.Tensor, n_rows: int, tap_rows: int,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Temporal conv over frames plus its residual, as one GEMM over a virtual im2col.
+
+    xp: [rows, C] bf16 (unit channel stride), the frame in front of the first output frame followed by the
+    frames themselves (``rows >= n_rows + tap_rows``; rows past the end read as zero: the right padding);
+    weight: [C, taps*C] bf16 with ``weight[o, t*C + i] = t_conv.weight[o, i, t, 0]``.  Returns
+    ``out[m] = xp[m + (taps//2)*tap_rows] + sum_t weight[:, t*C:(t+1)*C] @ xp[m + t*tap_rows]``, m < n_rows."""
+    _need_cuda(xp, weight, out)
+    if xp.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise SanaHipError("tconv_residual is bf16 only")
+    x2, ldx = _rows(xp, "xp")
+    w2, ldw = _rows(weight, "weight")
+    rows, C = x2.shape
+    if w2.shape[0] != C or w2.shape[1] % C:
+        raise SanaHipError(f"weight must be [C, taps*C] with C={C}, got {tuple(w2.shape)}")
+    taps = w2.shape[1] // C
+    if out is None:
+        out = torch.empty(n_rows, C, dtype=torch.bfloat16, device=xp.device)
+    o2, ldo = _rows(out, "out")
+    if tuple(o2.shape) != (n_rows, C) or o2.dtype != torch.bfloat16:
+        raise SanaHipError("out has the wrong shape or dtype")
+    code = _lib.load().sana_hip_tconv_residual(x2.data_ptr(), w2.data_ptr(), o2.data_ptr(), n_rows, C, taps,
+                                               tap_rows, rows, ldx, ldw, ldo, _stream())
+    _lib.check(code, "sana_hip_tconv_residual")
+    return out
+
+
 def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
     """LN(x) * (1 + scale) + shift over the last dim; x: [B, N, C] bf16, scale/shift: [B, 1, C]."""
     _need_cuda(x, scale, shift)

@@ -32,7 +32,7 @@ def test_exports_every_declared_symbol():
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.sana_hip_abi_version() == 2
+    assert lib.sana_hip_abi_version() == 3
     assert b"aligned" in lib.sana_hip_strerror(-3)
     assert b"unknown" in lib.sana_hip_strerror(-99)
 
@@ -57,6 +57,11 @@ def test_argument_validation_needs_no_gpu():
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 20, 24, 24, 8, 0, None) == -2      # K % 8
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None) == -1      # bias epilogue, no bias
     assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None) == -1  # no scale
+    # temporal conv: C % 64, odd taps, the centre tap must exist for every output row
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 96, 3, 16, 80, 96, 288, 96, None) == -2
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 2, 16, 80, 64, 128, 64, None) == -1
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 64, 64, 192, 64, None) == -1
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 80, 64, 128, 64, None) == -1   # ldw < taps * C
 
 
 def test_workspace_query():

@@ -206,3 +206,38 @@ def test_layernorm_modulate_matches_stock_op_chain(cuda, B, Ntok, C):
     mag = chain.float().abs() + shift.float().abs()
     assert (diff > 2 ** -6 * mag + 1e-6).sum().item() == 0
     assert (diff == 0).float().mean().item() > 0.98
+
+
+@pytest.mark.parametrize("C,T,P,B", [(64, 4, 30, 1), (128, 6, 35, 2), (2240, 3, 300, 1)])
+def test_temporal_conv_residual_matches_conv2d(cuda, C, T, P, B):
+    """x + t_conv(x) over frames (zero frame in front, zeros behind) against F.conv2d in fp64, with the
+    reference's two roundings (conv output to bf16, then the sum)."""
+    g = torch.Generator().manual_seed(C + T)
+    y = torch.randn(B, T * P, C, generator=g).bfloat16()
+    w = (torch.randn(C, C, 3, 1, generator=g) * (1.0 / (3 * C)) ** 0.5).bfloat16()
+    xr = y.double().view(B, T, P, C).permute(0, 3, 1, 2)                          # (B, C, T, P) as the reference
+    conv = F.conv2d(xr, w.double(), padding=(1, 0))
+    ref = (xr + conv.bfloat16().double()).permute(0, 2, 3, 1).reshape(B, T * P, C)
+    w2 = w[:, :, :, 0].permute(0, 2, 1).reshape(C, 3 * C).contiguous().to(cuda)
+    buf = torch.zeros(B, (T + 1) * P, C, dtype=torch.bfloat16, device=cuda)
+    buf[:, P:] = y.to(cuda)
+    out = torch.stack([ops.tconv_residual(buf[b], w2, T * P, P) for b in range(B)])
+    err = (out.cpu().double() - ref).abs()
+    assert err.max().item() <= 2e-2 and rel_l2(out.cpu(), ref) <= 3e-3
+    # all but a few results are the reference's bits (the fp32 sums of 3C products differ in order)
+    assert (out.cpu().double() != ref.bfloat16().double()).double().mean().item() < 0.02
+    # a chunk of frames [1, 3): the frame in front is real data, the frame behind reads as zero
+    if T >= 4:
+        seg = F.conv2d(torch.cat([xr[:, :, 0:3], torch.zeros_like(xr[:, :, :1])], 2), w.double(), padding=(1, 0))
+        ref_c = (xr[:, :, 1:3] + seg[:, :, 1:3].bfloat16().double()).permute(0, 2, 3, 1).reshape(B, 2 * P, C)
+        out_c = torch.stack([ops.tconv_residual(buf[b, P:4 * P], w2, 2 * P, P) for b in range(B)])
+        assert (out_c.cpu().double() - ref_c).abs().max().item() <= 2e-2 and rel_l2(out_c.cpu(), ref_c) <= 3e-3
+
+
+def test_temporal_conv_zero_weight_is_identity(cuda):
+    """t_conv is zero-initialised in the reference: x + 0 must come back bit for bit."""
+    C, T, P = 128, 3, 50
+    y = torch.randn(T * P, C, generator=torch.Generator().manual_seed(3)).bfloat16().to(cuda)
+    buf = torch.cat([torch.zeros(P, C, dtype=torch.bfloat16, device=cuda), y])
+    out = ops.tconv_residual(buf, torch.zeros(C, 3 * C, dtype=torch.bfloat16, device=cuda), T * P, P)
+    assert torch.equal(out, y)

@@ -182,9 +182,12 @@ def _temp_pair(name, C, Hd, seed):
     return om, hm
 
 
-def test_temporal_mix_ffn_variants(cuda):
-    """GLUMBConvTemp / ChunkGLUMBConvTemp against the fp64 oracle, and the cached stream against the chunked call."""
-    C, Hd, (T, H, W), B = 96, 240, (6, 5, 7), 2
+@pytest.mark.parametrize("C,Hd", [(96, 240), (128, 320)])
+def test_temporal_mix_ffn_variants(cuda, C, Hd):
+    """GLUMBConvTemp / ChunkGLUMBConvTemp against the fp64 oracle, and the cached stream against the chunked call.
+    C = 128 takes the temporal conv as a GEMM over the token-major frames, C = 96 (not a multiple of the k-tile)
+    and the masked call the stock convolution."""
+    (T, H, W), B = (6, 5, 7), 2
     P = H * W
     x = torch.randn(B, T * P, C, generator=torch.Generator().manual_seed(11)).bfloat16()
     with torch.no_grad():
