@@ -222,6 +222,21 @@ def kernel_rooflines(dev, iters=50, warmup=10):
         t_lib = event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 20, 5)
         rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt, plain GEMM(+bias) of the same shape, for scale only
         del a, w, o
+    # temporal (3, 1) conv of the video Mix-FFN (GLUMBConvTemp) + its residual at the cfg5 frame grid, as one GEMM over
+    # the token-major frames; the stock convolution on the reference's (B, C, T, HW) view beside it
+    Tf, Pf = 21, 30 * 52
+    buf = torch.randn((Tf + 1) * Pf, C, generator=g).bfloat16().to(dev)
+    buf[:Pf].zero_()
+    wt = (torch.randn(C, 3 * C, generator=g) * 0.01).bfloat16().to(dev)
+    ot = torch.empty(Tf * Pf, C, dtype=torch.bfloat16, device=dev)
+    add("tconv_residual_cfg5", "mfma", 2 * Tf * Pf * 3 * C * C,
+        event_time_us(lambda: ops.tconv_residual(buf, wt, Tf * Pf, Pf, out=ot), 10, 3),
+        f"2*M*3C*C, M={Tf * Pf} (21 frames of 1560 tokens), C={C}")
+    xr = buf[Pf:].view(1, Tf, Pf, C).permute(0, 3, 1, 2)
+    w4 = wt.view(C, 3, C).permute(0, 2, 1).unsqueeze(-1).contiguous()
+    rows[-1]["library_conv_us"] = round(event_time_us(
+        lambda: xr + torch.nn.functional.conv2d(xr, w4, padding=(1, 0)), 3, 1), 2)
+    del buf, ot, xr
     # plain device copy as a bandwidth yardstick of this box
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
