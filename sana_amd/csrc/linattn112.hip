@@ -327,7 +327,6 @@ __device__ __forceinline__ void split3_112(const float x[8], u32x4_t out[3]) {
   }
 }
 
-constexpr int APPLY_TOKENS = 256;  // tokens per workgroup
 constexpr int TT = 32;             // tokens per step
 constexpr int QROW = 120;          // LDS row stride of the 16-bit tiles, elements: 240 B = 60 banks, so the 16 tokens
                                    // of a b128 operand read land on 16 disjoint groups of 4 banks
@@ -337,7 +336,8 @@ template <bool OUT_F32, int PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
                                                        void* __restrict__ out,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int xranges, int units, int64_t q_stride_b,
+                                                       int n_chunks, int xranges, int wg_tokens, int units,
+                                                       int64_t q_stride_b,
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
   constexpr int NQ = (PRE & 2) ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
@@ -350,8 +350,8 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   const int head = hu.head;
   const int bx = hu.unit % xranges, c = (hu.unit / xranges) % n_chunks, b = hu.unit / (xranges * n_chunks);
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
-  const int t0 = cr.begin + bx * APPLY_TOKENS;
-  const int t1 = min(cr.end, t0 + APPLY_TOKENS);
+  const int t0 = cr.begin + bx * wg_tokens;
+  const int t1 = min(cr.end, t0 + wg_tokens);
   if (t0 >= t1) return;  // uniform over the workgroup
   const int n = lane & 15, g = lane >> 4;
   constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
@@ -518,6 +518,18 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   }
 }
 
+int compute_units112() {
+  static int n = 0;  // same value from every thread that races here
+  if (n == 0) {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
+      cu = 256;
+    n = cu;
+  }
+  return n;
+}
+
 struct Plan112 {
   int nsplit, split_tokens;
 };
@@ -590,15 +602,32 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
                     int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
                     hipStream_t s) {
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
-  const int xranges = (max_chunk_tokens + APPLY_TOKENS - 1) / APPLY_TOKENS;
+  // Tokens per workgroup (a multiple of the 32-token step): long enough to pay for building the state
+  // operands once (~256), and such that the grid fills whole rounds of the chip -- 3 workgroups per CU
+  // fit (2 with transforms or fp32 output: registers), so 4 rounds of 256 tokens with the last one a third
+  // full lose to 3 rounds of 288.
+  const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+  int wg_tokens = 256;
+  {
+    const int64_t slots = (int64_t)compute_units112() * ((mode || out_dtype == SANA_DT_F32) ? 2 : 3);
+    double best = 1e30;
+    for (int t = 192; t <= 512; t += 32) {
+      const int64_t wgs = (int64_t)((max_chunk_tokens + t - 1) / t) * n_chunks * B * h;
+      const double cost = (double)((wgs + slots - 1) / slots) * (t + 48);  // + the operand build, in token-equivalents
+      if (cost < best) {
+        best = cost;
+        wg_tokens = t;
+      }
+    }
+  }
+  const int xranges = (max_chunk_tokens + wg_tokens - 1) / wg_tokens;
   const int64_t units = (int64_t)xranges * n_chunks * B, total = head_unit_grid(units, h);
   if (total > 0x7fffffff) return SANA_ERR_SHAPE;
   dim3 grid((unsigned)total);
   const uint16_t* qp = static_cast<const uint16_t*>(q);
 #define SANA_AP112(F32, PRE)                                                                                         \
   hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
-                     xranges, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
-  const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+                     xranges, wg_tokens, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
   if (out_dtype == SANA_DT_F32) {
     if (mode == 3) SANA_AP112(true, 3);
     else if (mode == 2) SANA_AP112(true, 2);
