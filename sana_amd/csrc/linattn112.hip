@@ -310,26 +310,28 @@ __global__ __launch_bounds__(256) void reduce112_kernel(const float* partial, fl
 // tile, results go to an LDS output tile and leave as whole rows again.  Tiles are double buffered,
 // the next tile's loads are in flight during the MFMAs: one barrier per step.
 // ----------------------------------------------------------------------------
-__device__ __forceinline__ void split3_112(const float x[8], u32x4_t out[3]) {
-  uint32_t hi[8], mid[8], lo[8];
+// fp32 -> bf16 terms hi + mid (+ lo), pairwise: one packed convert rounds two values
+template <int NT>
+__device__ __forceinline__ void split_terms(const float x[8], u32x4_t out[NT]) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    hi[e] = f32_to_bf16_bits(x[e]);
-    const float r1 = x[e] - bf16_bits_to_f32(hi[e]);
-    mid[e] = f32_to_bf16_bits(r1);
-    lo[e] = f32_to_bf16_bits(r1 - bf16_bits_to_f32(mid[e]));
-  }
+  for (int e = 0; e < 4; ++e) {
+    float r0 = x[2 * e], r1 = x[2 * e + 1];
 #pragma unroll
-  for (int e2 = 0; e2 < 4; ++e2) {
-    out[0][e2] = hi[2 * e2] | (hi[2 * e2 + 1] << 16);
-    out[1][e2] = mid[2 * e2] | (mid[2 * e2 + 1] << 16);
-    out[2][e2] = lo[2 * e2] | (lo[2 * e2 + 1] << 16);
+    for (int term = 0; term < NT; ++term) {
+      const uint32_t pk = pack_bf16(r0, r1);
+      out[term][e] = pk;
+      if (term + 1 < NT) {
+        r0 -= bf16_lo(pk);
+        r1 -= bf16_hi(pk);
+      }
+    }
   }
 }
 
 constexpr int TT = 32;             // tokens per step
-constexpr int QROW = 120;          // LDS row stride of the 16-bit tiles, elements: 240 B = 60 banks, so the 16 tokens
-                                   // of a b128 operand read land on 16 disjoint groups of 4 banks
+constexpr int QROW = 136;          // LDS row stride of the 16-bit tiles, elements: 272 B = 68 banks, so the 16 tokens
+                                   // of a b128 operand read land on 16 disjoint groups of 4 banks; pieces 14
+                                   // and 15 of a row (the padded k range 112..127) stay zero
 constexpr int OROW32 = 116;        // row stride of the fp32 output tile, floats (same argument: 116 % 64 = 52)
 
 template <bool OUT_F32, int PRE>
@@ -363,27 +365,23 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * SE;
   constexpr int NT = OUT_F32 ? 3 : 2;  // bf16 terms of an fp32 state value: 24 / 16 mantissa bits
   u32x4_t a[3][4][NT];                 // [row block][k block][term]
+  {
+    // buffer loads: rows / k groups outside the head's state get an out-of-range offset and read as zero
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sp), 0, SE * 4, 0x00020000);
 #pragma unroll
-  for (int rb = 0; rb < 3; ++rb) {
-    const int ch = 32 * wave + 8 * (n >> 2) + 4 * rb + (n & 3);
-    const int row = rb < 2 ? ch : DH;
-    const bool row_ok = rb == 2 || ch < DH;
+    for (int rb = 0; rb < 3; ++rb) {
+      const int ch = 32 * wave + 8 * (n >> 2) + 4 * rb + (n & 3);
+      const int row = rb < 2 ? ch : DH;
+      const bool row_ok = rb == 2 || ch < DH;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      const int k0 = kb * 32 + 8 * g;
-      float x[8];
-      if (row_ok && k0 < DH) {
-        const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(sp + row * DH + k0);
-        const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(sp + row * DH + k0 + 4);
-        x[0] = x0[0], x[1] = x0[1], x[2] = x0[2], x[3] = x0[3], x[4] = x1[0], x[5] = x1[1], x[6] = x1[2], x[7] = x1[3];
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = 0.f;
+      for (int kb = 0; kb < 4; ++kb) {
+        const int k0 = kb * 32 + 8 * g;
+        const int off = (row_ok && k0 < DH) ? (row * DH + k0) * 4 : (int)0x80000000u;
+        const f32x4_t x0 = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, off, 0, 0));
+        const f32x4_t x1 = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, off + 16, 0, 0));
+        const float x[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        split_terms<NT>(x, a[rb][kb]);
       }
-      u32x4_t t3[3];
-      split3_112(x, t3);
-#pragma unroll
-      for (int term = 0; term < NT; ++term) a[rb][kb][term] = t3[term];
     }
   }
 
@@ -437,6 +435,8 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   };
 
   const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
+  for (int i = tid; i < 2 * NQ * TT * 3; i += 256)  // pieces 14..16 of every q tile row: written once, as zeros
+    *reinterpret_cast<u32x4_t*>(lds_q + (i / 3) * QROW + (NCH + i % 3) * 8) = zero4;
   issue(t0);
   stage(0);
   if (t0 + TT < t1) issue(t0 + TT);
@@ -451,10 +451,9 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
       u32x4_t qd[4], qb[4];
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const bool ok = kb * 4 + g < NCH;  // pieces 14, 15 of the padded k range: zero, whatever the tile holds there
-        const int off = (16 * ss + n) * QROW + (kb * 4 + g) * 8;
-        qb[kb] = ok ? *reinterpret_cast<const u32x4_t*>(tb + off) : zero4;
-        if (has_rope) qd[kb] = ok ? *reinterpret_cast<const u32x4_t*>(td + off) : zero4;
+        const int off = (16 * ss + n) * QROW + (kb * 4 + g) * 8;  // pieces 14, 15 (kb = 3, g >= 2) hold zeros
+        qb[kb] = *reinterpret_cast<const u32x4_t*>(tb + off);
+        if (has_rope) qd[kb] = *reinterpret_cast<const u32x4_t*>(td + off);
       }
       f32x4_t acc[3];
 #pragma unroll
