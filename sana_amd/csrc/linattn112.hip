@@ -45,7 +45,8 @@ inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) /
 // partial[(bh * n_chunks + c) * nsplit + split][SE]
 // ----------------------------------------------------------------------------
 constexpr int LR = 160;  // LDS tile row stride in elements: 320 B puts the two token groups of a read 16 banks apart
-constexpr int SMEM_BYTES = 2 * SE * 4;  // two fp32 states for the wave reduction (>= 4 waves x 2 tiles x 32 x LR x 2 B)
+constexpr int SMEM_BYTES = 2 * 128 * 128 * 4;  // two padded fp32 accumulator images for the wave reduction
+                                             // (>= 4 waves x 2 tiles x 33 x LR x 2 B of staging)
 static_assert(SMEM_BYTES >= 4 * 2 * (TILE + 1) * LR * 2, "staging must fit");
 
 // PRE: on-load transforms, compile-time so that the tile code stays one branch-free block: bit 0 = q/k RMSNorm,
@@ -226,52 +227,54 @@ __global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restric
 #pragma unroll
   for (int jb = 0; jb < 4; ++jb) acck[jb] += __shfl_xor(acck[jb], 32, 64);  // the two token halves
 
-  // cross-wave sum in LDS, two rounds (two states fit): waves 2, 3 -> waves 0, 1; wave 1 -> wave 0.
-  // D layout of 32x32 MFMA: lane -> column j = lane%32, register r -> row 8*(r/4) + 4*(lane/32) + r%4
+  // Cross-wave sum in LDS, two images of the padded 128 x 128 accumulator (no predicates): waves 2, 3 -> images
+  // 0, 1; waves 0, 1 add them and write their sums back; then all four waves add the two images and store the
+  // 113 x 112 state as whole 16-byte pieces.  ksum travels as row 112 of the image (that accumulator row belongs
+  // to a zero channel).  D layout of 32x32 MFMA: lane -> column j = lane%32, register r -> row 8*(r/4) +
+  // 4*(lane/32) + r%4.
   float* red = reinterpret_cast<float*>(smem);
-  auto put = [&](float* dstp) {
+  auto put = [&](float* img) {
 #pragma unroll
     for (int ib = 0; ib < 4; ++ib)
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
-        const int col = jb * 32 + j;
+      for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (row < DH && col < DH) dstp[row * DH + col] = acc[ib][jb][r];
-        }
-      }
+        for (int r = 0; r < 16; ++r)
+          img[(ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + jb * 32 + j] = acc[ib][jb][r];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the zero row 112 is written before ksum replaces it
+    if (g == 0) {
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb)
-      if (g == 0 && jb * 32 + j < DH) dstp[DH * DH + jb * 32 + j] = acck[jb];
+      for (int jb = 0; jb < 4; ++jb) img[DH * 128 + jb * 32 + j] = acck[jb];
+    }
   };
-  auto take = [&](const float* srcp) {
+  auto take = [&](const float* img) {
 #pragma unroll
     for (int ib = 0; ib < 4; ++ib)
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
-        const int col = jb * 32 + j;
+      for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (row < DH && col < DH) acc[ib][jb][r] += srcp[row * DH + col];
-        }
-      }
+        for (int r = 0; r < 16; ++r)
+          acc[ib][jb][r] += img[(ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + jb * 32 + j];
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb)
-      if (jb * 32 + j < DH) acck[jb] += srcp[DH * DH + jb * 32 + j];
+    for (int jb = 0; jb < 4; ++jb) acck[jb] += img[DH * 128 + jb * 32 + j];
   };
   __syncthreads();  // staging tiles are dead
-  if (wave >= 2) put(red + (wave - 2) * SE);
+  if (wave >= 2) put(red + (wave - 2) * 128 * 128);
   __syncthreads();
-  if (wave < 2) take(red + wave * SE);
+  if (wave < 2) {  // a wave rewrites the image it has just read itself: no barrier in between
+    take(red + wave * 128 * 128);
+    put(red + wave * 128 * 128);
+  }
   __syncthreads();
-  if (wave == 1) put(red);
-  __syncthreads();
-  if (wave == 0) {
-    take(red);
+  {
     const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nsplit + split;
-    put(partial + slot * SE);
+    float* dst = partial + slot * SE;
+    for (int p = threadIdx.x; p < (DH + 1) * (DH / 4); p += 256) {  // 16-byte pieces of the 113 x 112 state
+      const int row = p / (DH / 4), c4 = p - row * (DH / 4);
+      const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(red + row * 128 + c4 * 4);
+      const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(red + 128 * 128 + row * 128 + c4 * 4);
+      *reinterpret_cast<f32x4_t*>(dst + row * DH + c4 * 4) = x0 + x1;
+    }
   }
 }
 
