@@ -127,6 +127,16 @@ __device__ __forceinline__ u32x4_t gate_res8v(u32x4_t y, u32x4_t g, u32x4_t r) {
   o.w = gate_res2(y.w, g.w, r.w);
   return o;
 }
+// the same with the gate values already unpacked (they are the same for every row a lane handles)
+__device__ __forceinline__ u32x4_t gate_res8f(u32x4_t y, const float* g, u32x4_t r) {
+  u32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t t = pack_bf16(g[2 * e] * bf16_lo(y[e]), g[2 * e + 1] * bf16_hi(y[e]));  // one convert rounds both
+    o[e] = pack_bf16(bf16_lo(r[e]) + bf16_lo(t), bf16_hi(r[e]) + bf16_hi(t));
+  }
+  return o;
+}
 // y: 8 linear outputs (already rounded to bf16) of row m, columns n..n+7
 __device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m, int n) {
   const u32x4_t g = *reinterpret_cast<const u32x4_t*>(e.gate + (int64_t)(m / e.rows_per_gate) * e.gate_stride + n);
@@ -565,18 +575,32 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
   __syncthreads();  // every wave is done with the operand tiles
   unsigned char* stg = smem + wave * 32768;
+  // Global accesses of the epilogue are buffer loads / stores on the wave's 128 rows of C (and of the
+  // residual): a row costs one vector add for its offset, rows past M and channel pieces past N fall
+  // outside the resource (loads return zero, stores are dropped) -- no 64-bit address arithmetic, no
+  // per-row predication.
+  const int wrow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;  // first row of this wave (a scalar: it goes into resources)
+  const int wrows = max(0, min(128, M - wrow0));          // its rows that exist
+  const int idle_off = (int)0x80000000u;
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+      C + (int64_t)wrow0 * ldc, 0, wrows ? (int)((((int64_t)wrows - 1) * ldc + N) * 2) : 0, 0x00020000);
+  const int c_off0 = o_live ? (o_rsub * (int)ldc + o_n) * 2 : idle_off, c_step = 4 * (int)ldc * 2;
   // Gated residual: the residual rows this lane will add are requested now, a whole epilogue ahead
   // of their use (128 registers that the main loop no longer needs; asking for them before the last
   // k-tile makes the compiler spill).
   u32x4_t res[4][8];
+  const bool gated = EPI == SANA_EPI_GATE_RES;
+  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(gated ? ep.res + (int64_t)wrow0 * ep.ldr : nullptr), 0,
+      gated && wrows ? (int)((((int64_t)wrows - 1) * ep.ldr + N) * 2) : 0, 0x00020000);
+  const int r_off0 = o_live ? (o_rsub * (int)ep.ldr + o_n) * 2 : idle_off, r_step = 4 * (int)ep.ldr * 2;
   if (EPI == SANA_EPI_GATE_RES) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int m = m0 + wt * 128 + 32 * j + it * 4 + o_rsub;
-        if (o_live && m < M) res[j][it] = *reinterpret_cast<const u32x4_t*>(ep.res + (int64_t)m * ep.ldr + o_n);
-      }
+      for (int it = 0; it < 8; ++it)
+        res[j][it] = __builtin_bit_cast(
+            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, 0));
   }
   float bv[NI][16];
   if (HAS_BIAS) {
@@ -593,12 +617,22 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int tok = 32 * j + fr;
-    // one gate row serves the whole group unless a batch boundary runs through its 32 tokens
-    const int m_first = m0 + wt * 128 + 32 * j;
-    const int g_first = m_first / ep.rows_per_gate, g_last = min(m_first + 31, M - 1) / ep.rows_per_gate;
-    u32x4_t gate = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // no gate: 1.0, a plain residual add
-    if (EPI == SANA_EPI_GATE_RES && ep.gate && o_live && m_first < M)
-      gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
+    // The lane's eight gate values, as floats.  One gate row serves the whole group of 32 tokens unless a
+    // batch boundary runs through it: then the rows from m_switch on take the next gate row (gates are per
+    // batch entry; entries shorter than 32 tokens take the slow way, a division per row).
+    const int m_first = wrow0 + 32 * j;
+    const int g_first = m_first / ep.rows_per_gate;
+    const int m_switch = (g_first + 1) * ep.rows_per_gate;
+    const bool two_gates = EPI == SANA_EPI_GATE_RES && ep.gate && m_switch < min(m_first + 32, M);
+    float gf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // no gate: 1.0, a plain residual add
+    if (EPI == SANA_EPI_GATE_RES && ep.gate && o_live && m_first < M) {
+      const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        gf[2 * e] = bf16_lo(gate[e]);
+        gf[2 * e + 1] = bf16_hi(gate[e]);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
 #pragma unroll
@@ -615,16 +649,22 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
       const int row = 32 * j + it * 4 + o_rsub;
-      const int m = m0 + wt * 128 + row;
       u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-      if (o_live && m < M) {
-        if (EPI == SANA_EPI_GATE_RES) {
-          u32x4_t g = gate;
-          if (ep.gate && g_first != g_last && m / ep.rows_per_gate != g_first)
-            g = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
-          o = gate_res8v(o, g, res[j][it]);
+      if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[j][it]);
+      __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * j + it) * c_step, 0, 0);
+    }
+    if (two_gates) {  // uniform, rare: rows behind the boundary are redone with their own gate row and stored again
+#pragma unroll 1
+      for (int it = 0; it < 8; ++it) {
+        const int row = 32 * j + it * 4 + o_rsub, m = wrow0 + row;
+        if (o_live && m >= m_switch && m < M) {
+          const u32x4_t y = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
+          const u32x4_t r = __builtin_bit_cast(
+              u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, 0));
+          const u32x4_t g2 = *reinterpret_cast<const u32x4_t*>(
+              ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
+          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * j + it) * c_step, 0, 0);
         }
-        *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + o_n) = o;
       }
     }
   }
