@@ -167,7 +167,8 @@ def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilog
 
 
 @pytest.mark.parametrize("B,Ntok,C,K,w8", [(1, 16384, 2240, 2240, False), (2, 1024, 2240, 5600, False),
-                                          (3, 100, 96, 240, False), (2, 1024, 2240, 5600, True)])
+                                          (3, 100, 96, 240, False), (2, 1024, 2240, 5600, True),
+                                          (7, 20, 96, 128, False)])   # several gate rows inside one 32-token group
 def test_gemm_gate_residual_matches_stock_op_chain(cuda, B, Ntok, C, K, w8):
     g = torch.Generator().manual_seed(B + K)
     a = torch.randn(B, Ntok, K, generator=g).bfloat16().to(cuda)
