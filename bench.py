@@ -203,7 +203,8 @@ def kernel_rooflines(dev, iters=50, warmup=10):
         "M*C*2 B read + M*C*2 B write")
     for name, Nn, Kk, epi in (("gemm_qkv", 3 * C, C, None), ("gemm_proj_gate_residual", C, C, "gate_res"),
                               ("gemm_inverted", 2 * HID, C, "bias_silu"), ("gemm_point_gate_residual", C, HID, "gate_res"),
-                              ("gemm_inverted_w8a16", 2 * HID, C, "w8_bias_silu")):
+                              ("gemm_inverted_w8a16", 2 * HID, C, "w8_bias_silu"),
+                              ("gemm_inverted_w8a16_in_loop", 2 * HID, C, "w8_bias_silu_fused")):
         a = torch.randn(M, Kk, generator=g).bfloat16().to(dev)
         w = (torch.randn(Nn, Kk, generator=g) * 0.02).bfloat16().to(dev)
         bias = torch.zeros(Nn, dtype=torch.bfloat16, device=dev) if epi else None
@@ -211,10 +212,13 @@ def kernel_rooflines(dev, iters=50, warmup=10):
         lib_extra = ""
         if epi == "gate_res":     # x + gate * (a @ w.T + bias): the two gated residual seams of the block
             fn = lambda: ops.gemm_gate_residual(a.view(B, N, Kk), w, bias, mod[:, 2:3], x_ln)
-        elif epi == "w8_bias_silu":
+        elif epi in ("w8_bias_silu", "w8_bias_silu_fused"):
+            # int8 weights: expanded to bf16 by a kernel of its own in front of the bf16 GEMM (what the library
+            # picks at this M), or converted inside the GEMM's main loop (the path for small M)
             from sana_amd.modules import quantize_w8
             wq, sc = quantize_w8(w)
-            fn = lambda: ops.gemm_w8a16(a, wq, sc, bias, "bias_silu", out=o)
+            fused = epi.endswith("_fused")
+            fn = lambda: ops.gemm_w8a16(a, wq, sc, bias, "bias_silu", out=o, expand=not fused)
         else:
             fn = lambda: ops.gemm_bf16(a, w, bias, epi, out=o)
         t_us = event_time_us(fn, 20, 5)

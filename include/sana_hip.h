@@ -236,6 +236,17 @@ int sana_hip_layernorm_modulate(const void* x, const void* scale, const void* sh
                                 int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * int8 weight -> bf16: W[n][k] = bf16((float)Wq[n][k] * scale[n]), one rounding -- bit for bit the value
+ * the int8 path of the GEMM feeds its MFMAs (and torch's `(Wq.float() * scale[:, None]).bfloat16()`).
+ * No counterpart in the reference (W8A16 is defined by the benchmark configuration).  For GEMMs with many
+ * rows (M of a few thousand and more) expanding the weight once per call and running the bf16 GEMM is
+ * faster than converting inside the GEMM's main loop; the results are identical.
+ *   Wq int8 [N][K] (row stride ldw, K % 16 == 0), scale fp32 [N], W bf16 [N][K] (row stride ldo)
+ */
+int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, int N, int K,
+                        int64_t ldw, int64_t ldo, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Temporal (t, 1) convolution over frames with full channel mixing, plus its residual, as ONE GEMM over a
  * virtual im2col of the token-major buffer (no copy of the activations):
  *

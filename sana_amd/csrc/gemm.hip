@@ -46,6 +46,28 @@ __device__ __forceinline__ uint32_t dequant2(uint32_t q4, int which, float s, fl
   return pack_bf16(fmaf(f0, s, off), fmaf(f1, s, off));
 }
 
+// int8 weight [N][K] + per-row scale -> bf16 [N][K], with the rounding of dequant2: the expansion the GEMM's
+// int8 path performs on its way to LDS, as a streaming kernel of its own (16 values per thread).
+__global__ __launch_bounds__(256) void dequant_w8_kernel(const int8_t* __restrict__ wq, const float* __restrict__ scale,
+                                                         uint16_t* __restrict__ out, int N, int K, int64_t ldw,
+                                                         int64_t ldo) {
+  const int pieces = K >> 4;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)N * pieces) return;
+  const int n = (int)(id / pieces), p = (int)(id - (int64_t)n * pieces);
+  u32x4_t q = *reinterpret_cast<const u32x4_t*>(wq + n * ldw + 16 * p);
+  const float s = scale[n], off = -128.f * s;
+  u32x4_t lo, hi;
+  q.x ^= 0x80808080u, q.y ^= 0x80808080u, q.z ^= 0x80808080u, q.w ^= 0x80808080u;
+  lo.x = dequant2(q.x, 0, s, off), lo.y = dequant2(q.x, 1, s, off);
+  lo.z = dequant2(q.y, 0, s, off), lo.w = dequant2(q.y, 1, s, off);
+  hi.x = dequant2(q.z, 0, s, off), hi.y = dequant2(q.z, 1, s, off);
+  hi.z = dequant2(q.w, 0, s, off), hi.w = dequant2(q.w, 1, s, off);
+  uint16_t* o = out + n * ldo + 16 * p;
+  *reinterpret_cast<u32x4_t*>(o) = lo;
+  *reinterpret_cast<u32x4_t*>(o + 8) = hi;
+}
+
 // Epilogue operands.  SANA_EPI_GATE_RES: C = res + gate[row / rows_per_gate] * (acc + bias), i.e. the
 // gated residual update of the block (x + gate * module(x)), with the reference's three roundings
 // (linear output, gate product, residual sum) reproduced in registers.
@@ -822,4 +844,17 @@ SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, in
   const Taps tp = {C, tap_rows, x_rows};
   return launch<false>(X, W, nullptr, e, out, M, C, taps * C, ldx, ldw, ldo, SANA_EPI_GATE_RES,
                        static_cast<hipStream_t>(stream), &tp);
+}
+
+SANA_API int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, int N, int K, int64_t ldw,
+                                 int64_t ldo, void* stream) {
+  if (!Wq || !scale || !W || N <= 0 || K <= 0) return SANA_ERR_ARG;
+  if (K % 16) return SANA_ERR_SHAPE;
+  if (ldw < K || ldo < K) return SANA_ERR_ARG;
+  if (ldw % 16 || ldo % 8 || !aligned16(Wq) || !aligned16(W)) return SANA_ERR_ALIGN;
+  const int64_t threads = (int64_t)N * (K / 16);
+  if ((threads + 255) / 256 > 0x7fffffff) return SANA_ERR_SHAPE;
+  hipLaunchKernelGGL(dequant_w8_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), Wq, scale, static_cast<uint16_t*>(W), N, K, ldw, ldo);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }

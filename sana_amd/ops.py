@@ -275,12 +275,37 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
+# From this many rows on, an int8 weight is expanded to bf16 once per call (a streaming pass over N*K bytes) and
+# the bf16 GEMM runs; below it the GEMM converts inside its main loop.  Both give the same bits; the conversion
+# costs the main loop about 14 % at every M, the expansion a fixed 10-20 us.
+W8_EXPAND_MIN_ROWS = 4096
+
+
+def dequant_w8(wq: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """int8 [N, K] and fp32 [N] -> bf16 [N, K] = (wq.float() * scale[:, None]).bfloat16(), one kernel."""
+    _need_cuda(wq, scale)
+    if wq.dtype != torch.int8 or scale.dtype != torch.float32 or not scale.is_contiguous():
+        raise SanaHipError("dequant_w8 needs int8 weights and contiguous fp32 scales")
+    wq, ldw = _rows(wq, "wq")
+    N, K = wq.shape
+    if scale.numel() != N:
+        raise SanaHipError("one scale per weight row")
+    out = torch.empty(N, K, dtype=torch.bfloat16, device=wq.device)
+    code = _lib.load().sana_hip_dequant_w8(wq.data_ptr(), scale.data_ptr(), out.data_ptr(), N, K, ldw, K, _stream())
+    _lib.check(code, "sana_hip_dequant_w8")
+    return out
+
+
 def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """a: [M, K] bf16; wq: [N, K] int8; scale: [N] fp32.  Equals gemm_bf16 on (wq.float()*scale).bfloat16()."""
+               epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None,
+               expand: Optional[bool] = None) -> torch.Tensor:
+    """a: [M, K] bf16; wq: [N, K] int8; scale: [N] fp32.  Equals gemm_bf16 on (wq.float()*scale).bfloat16().
+    ``expand``: True = expand the weight to bf16 first, False = convert inside the GEMM, None = by M."""
     _need_cuda(a, wq, scale, bias)
     if a.dtype != torch.bfloat16 or wq.dtype != torch.int8 or scale.dtype != torch.float32:
         raise SanaHipError("gemm_w8a16 needs bf16 activations, int8 weights and fp32 scales")
+    if expand or (expand is None and a.shape[0] >= W8_EXPAND_MIN_ROWS):
+        return gemm_bf16(a, dequant_w8(wq, scale), bias, epilogue, out)
     a, lda = _rows(a, "a")
     wq, ldw = _rows(wq, "wq")
     M, K = a.shape
@@ -312,11 +337,14 @@ def _mod_rows(t: torch.Tensor, B: int, C: int, what: str) -> Tuple[torch.Tensor,
 
 
 def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], gate: torch.Tensor,
-                       residual: torch.Tensor, weight_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       residual: torch.Tensor, weight_scale: Optional[torch.Tensor] = None,
+                       expand: Optional[bool] = None) -> torch.Tensor:
     """residual + gate * (a @ weight.T + bias) with a: [B, N, K], residual: [B, N, C], gate: [B, 1, C].
-    weight is bf16 [C, K], or int8 with ``weight_scale`` (W8A16)."""
+    weight is bf16 [C, K], or int8 with ``weight_scale`` (W8A16; ``expand`` as in :func:`gemm_w8a16`)."""
     _need_cuda(a, weight, bias, gate, residual, weight_scale)
     B, Ntok, K = a.shape
+    if weight_scale is not None and (expand or (expand is None and B * Ntok >= W8_EXPAND_MIN_ROWS)):
+        weight, weight_scale = dequant_w8(weight.reshape(weight.shape[0], -1), weight_scale), None
     C = weight.shape[0]
     if a.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or gate.dtype != torch.bfloat16:
         raise SanaHipError("gemm_gate_residual is bf16 only")

@@ -155,10 +155,13 @@ def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilog
     wq, s = O.quantize_w8(w.bfloat16())
     wd = O.dequantize_w8(wq, s)
     bias = (torch.randn(N, generator=g) * 0.5).bfloat16().to(cuda) if epilogue else None
-    y8 = ops.gemm_w8a16(a, wq.to(cuda), s.to(cuda), bias, epilogue)
     y16 = ops.gemm_bf16(a, wd.to(cuda), bias, epilogue)
-    # in-register dequantisation reproduces (q.float()*s).bfloat16() exactly -> same kernel arithmetic
+    # both int8 routes -- conversion inside the GEMM's main loop, and the weight expanded to bf16 by a kernel of
+    # its own in front of the bf16 GEMM -- reproduce (q.float()*s).bfloat16() exactly -> same kernel arithmetic
+    y8 = ops.gemm_w8a16(a, wq.to(cuda), s.to(cuda), bias, epilogue, expand=False)
     assert torch.equal(y8, y16)
+    assert torch.equal(ops.dequant_w8(wq.to(cuda), s.to(cuda)).cpu(), wd)
+    assert torch.equal(ops.gemm_w8a16(a, wq.to(cuda), s.to(cuda), bias, epilogue, expand=True), y16)
     ref = _gemm_ref(a.cpu(), wd, None if bias is None else bias.cpu(), epilogue)
     assert rel_l2(y8.cpu(), ref) <= 4e-3
 
@@ -180,7 +183,8 @@ def test_gemm_gate_residual_matches_stock_op_chain(cuda, B, Ntok, C, K, w8):
     if w8:
         wq, s = O.quantize_w8(w)
         w = O.dequantize_w8(wq, s)
-        out = ops.gemm_gate_residual(a, wq.to(cuda), bias, gate, res, s.to(cuda))
+        out = ops.gemm_gate_residual(a, wq.to(cuda), bias, gate, res, s.to(cuda), expand=False)
+        assert torch.equal(out, ops.gemm_gate_residual(a, wq.to(cuda), bias, gate, res, s.to(cuda), expand=True))
     else:
         out = ops.gemm_gate_residual(a, w.to(cuda), bias, gate, res)
     # the reference's op chain in bf16: linear -> gate * y -> x + (.)
