@@ -134,13 +134,14 @@ def test_rotation_is_numerator_only_and_unit_rotation_is_identity(cuda):
 
 
 @pytest.mark.parametrize("qk_norm", [False, True])
-def test_chunk_causal_with_rope(cuda, qk_norm):
-    B, (f, h, w), C = 1, (5, 6, 8), 160
+@pytest.mark.parametrize("C,head_dim", [(160, 32), (224, 112)])
+def test_chunk_causal_with_rope(cuda, qk_norm, C, head_dim):
+    B, (f, h, w) = 1, (5, 6, 8)
     N = f * h * w
-    om, hm = make("ChunkCausalAttention", C, qk_norm, seed=4)
+    om, hm = make("ChunkCausalAttention", C, qk_norm, seed=4, head_dim=head_dim)
     hm = hm.to(cuda)
     x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(3)).bfloat16()
-    fr = freqs(N, 5)
+    fr = freqs(N, 5, head_dim=head_dim)
     with torch.no_grad():
         ref = ref64(om, x, HW=(f, h, w), rotary_emb=fr, chunk_index=[0, 1, 3])
         out = hm(x.to(cuda), HW=(f, h, w), rotary_emb=fr.to(cuda), chunk_index=[0, 1, 3])
