@@ -235,6 +235,16 @@ int sana_hip_layernorm_modulate(const void* x, const void* scale, const void* sh
                                 int64_t M, int C, int64_t ldx, int64_t ldo,
                                 int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
 
+/* The same with the residual update in front of the norm in the same pass:
+ *   sum[m][:] = x[m][:] + y[m][:]   (rounded to bf16, as the stock add stores it)
+ *   out[m][:] = LN(sum[m][:]) * (1 + scale[..]) + shift[..]
+ * replaces `x = x + self.cross_attn(x, y, mask)` followed by `t2i_modulate(self.norm2(x), shift_mlp,
+ * scale_mlp)` (sana_multi_scale.py:154-155).  y, sum: bf16 [M][C] with row strides ldy / lds; sum may alias x. */
+int sana_hip_add_layernorm_modulate(const void* x, const void* y, const void* scale, const void* shift,
+                                    void* sum, void* out, int64_t M, int C,
+                                    int64_t ldx, int64_t ldy, int64_t lds, int64_t ldo,
+                                    int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
+
 /* ---------------------------------------------------------------------------
  * int8 weight -> bf16: W[n][k] = bf16((float)Wq[n][k] * scale[n]), one rounding -- bit for bit the value
  * the int8 path of the GEMM feeds its MFMAs (and torch's `(Wq.float() * scale[:, None]).bfloat16()`).

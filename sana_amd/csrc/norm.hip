@@ -2,7 +2,9 @@
 //
 //   out[b, n, :] = LN(x[b, n, :]) * (1 + scale[b, :]) + shift[b, :]
 //
-// HBM bound: one read and one write of the activation (2 * M * C * 2 bytes).
+// HBM bound: one read and one write of the activation (2 * M * C * 2 bytes).  A second form takes the
+// residual sum in front of the norm along: sum = x + y is computed, stored and normalised in one pass
+// (2 reads + 2 writes instead of the 3 + 2 of a separate add).
 // One wave per token row; the row lives in registers as raw 16-byte chunks
 // (lane l holds chunks l, l+64, ...), so it is read from memory once: mean and
 // the centred variance are two register passes with wave reductions, the third
@@ -20,14 +22,17 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-// NCH: 16-byte chunks per lane (C <= 512 * NCH)
-template <int NCH>
+// NCH: 16-byte chunks per lane (C <= 512 * NCH).  ADD: the row is x + y (rounded to bf16, as the stock add
+// stores it) and is written to `sum` as well: the residual update in front of the norm, in the same pass.
+template <int NCH, bool ADD>
 __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __restrict__ x,
+                                                          const uint16_t* __restrict__ y,
                                                           const uint16_t* __restrict__ scale,
                                                           const uint16_t* __restrict__ shift,
+                                                          uint16_t* __restrict__ sum,
                                                           uint16_t* __restrict__ out, int64_t M, int C,
-                                                          int64_t ldx, int64_t ldo, int rows_per_mod,
-                                                          int64_t mod_stride, float eps) {
+                                                          int64_t ldx, int64_t ldy, int64_t lds, int64_t ldo,
+                                                          int rows_per_mod, int64_t mod_stride, float eps) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;
   if (row >= M) return;  // no barriers in this kernel
@@ -39,6 +44,21 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
   for (int i = 0; i < NCH; ++i) {
     const int ch = lane + 64 * i;
     raw[i] = ch < nchunks ? *reinterpret_cast<const u32x4_t*>(xr + 8 * ch) : zero4;
+  }
+  if (ADD) {
+    const uint16_t* yr = y + row * ldy;
+    uint16_t* sr = sum + row * lds;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int ch = lane + 64 * i;
+      if (ch < nchunks) {
+        const u32x4_t b = *reinterpret_cast<const u32x4_t*>(yr + 8 * ch);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          raw[i][e] = pack_bf16(bf16_lo(raw[i][e]) + bf16_lo(b[e]), bf16_hi(raw[i][e]) + bf16_hi(b[e]));
+        *reinterpret_cast<u32x4_t*>(sr + 8 * ch) = raw[i];
+      }
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -85,27 +105,32 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
 
 using namespace sana;
 
-extern "C" __attribute__((visibility("default"))) int sana_hip_layernorm_modulate(
-    const void* x, const void* scale, const void* shift, void* out, int64_t M, int C, int64_t ldx, int64_t ldo,
-    int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream) {
+template <bool ADD>
+static int ln_impl(const void* x, const void* y, const void* scale, const void* shift, void* sum, void* out, int64_t M,
+                   int C, int64_t ldx, int64_t ldy, int64_t lds, int64_t ldo, int rows_per_mod, int64_t mod_stride,
+                   float eps, int io_dtype, void* stream) {
   if (!x || !scale || !shift || !out || M <= 0 || C <= 0 || rows_per_mod <= 0) return SANA_ERR_ARG;
+  if (ADD && (!y || !sum)) return SANA_ERR_ARG;
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
   if (C % 8 || C > 8192) return SANA_ERR_SHAPE;
-  if (ldx < C || ldo < C || mod_stride < 0) return SANA_ERR_ARG;
+  if (ldx < C || ldo < C || mod_stride < 0 || (ADD && (ldy < C || lds < C))) return SANA_ERR_ARG;
   if (ldx % 8 || ldo % 8 || mod_stride % 8 || !aligned16(x) || !aligned16(out) || !aligned16(scale) ||
       !aligned16(shift))
     return SANA_ERR_ALIGN;
+  if (ADD && (ldy % 8 || lds % 8 || !aligned16(y) || !aligned16(sum))) return SANA_ERR_ALIGN;
   if ((M + 3) / 4 > 0x7fffffff) return SANA_ERR_SHAPE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid((unsigned)((M + 3) / 4)), block(256);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
+  const uint16_t* yp = static_cast<const uint16_t*>(y);
   const uint16_t* sc = static_cast<const uint16_t*>(scale);
   const uint16_t* sh = static_cast<const uint16_t*>(shift);
+  uint16_t* sp = static_cast<uint16_t*>(sum);
   uint16_t* op = static_cast<uint16_t*>(out);
   const int nch = (C / 8 + 63) / 64;
-#define SANA_LN(NCH) \
-  hipLaunchKernelGGL((ln_modulate_kernel<NCH>), grid, block, 0, s, xp, sc, sh, op, M, C, ldx, ldo, rows_per_mod, \
-                     mod_stride, eps)
+#define SANA_LN(NCH)                                                                                              \
+  hipLaunchKernelGGL((ln_modulate_kernel<NCH, ADD>), grid, block, 0, s, xp, yp, sc, sh, sp, op, M, C, ldx, ldy, lds, \
+                     ldo, rows_per_mod, mod_stride, eps)
   if (nch <= 2) SANA_LN(2);
   else if (nch <= 3) SANA_LN(3);
   else if (nch <= 5) SANA_LN(5);
@@ -113,4 +138,19 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_layernorm_modulat
   else SANA_LN(16);
 #undef SANA_LN
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_layernorm_modulate(
+    const void* x, const void* scale, const void* shift, void* out, int64_t M, int C, int64_t ldx, int64_t ldo,
+    int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream) {
+  return ln_impl<false>(x, nullptr, scale, shift, nullptr, out, M, C, ldx, 0, 0, ldo, rows_per_mod, mod_stride, eps,
+                        io_dtype, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_add_layernorm_modulate(
+    const void* x, const void* y, const void* scale, const void* shift, void* sum, void* out, int64_t M, int C,
+    int64_t ldx, int64_t ldy, int64_t lds, int64_t ldo, int rows_per_mod, int64_t mod_stride, float eps, int io_dtype,
+    void* stream) {
+  return ln_impl<true>(x, y, scale, shift, sum, out, M, C, ldx, ldy, lds, ldo, rows_per_mod, mod_stride, eps, io_dtype,
+                       stream);
 }

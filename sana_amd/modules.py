@@ -714,8 +714,8 @@ class SanaMSBlock(nn.Module):
                 x = x + gate_msa * self.attn(h, HW=HW, rotary_emb=image_rotary_emb)
             else:
                 x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
-            x = x + self.cross_attn(x, y, mask)
-            h = ops.layernorm_modulate(x, scale_mlp, shift_mlp, self.norm2.eps)
+            # the cross-attention's residual add and norm2 + modulate in one pass
+            x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask), scale_mlp, shift_mlp, self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)
         x = x + self.drop_path(
             gate_msa * self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), HW=HW, rotary_emb=image_rotary_emb))

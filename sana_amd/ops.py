@@ -403,3 +403,25 @@ def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor
                                                    B * Ntok, C, ldx, C, Ntok, s1, float(eps), _dt(x), _stream())
     _lib.check(code, "sana_hip_layernorm_modulate")
     return out.view(B, Ntok, C)
+
+
+def add_layernorm_modulate(x: torch.Tensor, y: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor,
+                           eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(x + y, LN(x + y) * (1 + scale) + shift) in one pass; x, y: [B, N, C] bf16, scale/shift: [B, 1, C]."""
+    _need_cuda(x, y, scale, shift)
+    if x.shape != y.shape or x.dtype != y.dtype:
+        raise SanaHipError("x and y must share shape and dtype")
+    B, Ntok, C = x.shape
+    x2, ldx = _rows(x.reshape(B * Ntok, C), "x")
+    y2, ldy = _rows(y.reshape(B * Ntok, C), "y")
+    sc, s1 = _mod_rows(scale, B, C, "scale")
+    sh, s2 = _mod_rows(shift, B, C, "shift")
+    if s1 != s2:
+        raise SanaHipError("scale and shift must share their batch stride")
+    total = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
+    out = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
+    code = _lib.load().sana_hip_add_layernorm_modulate(
+        x2.data_ptr(), y2.data_ptr(), sc.data_ptr(), sh.data_ptr(), total.data_ptr(), out.data_ptr(), B * Ntok, C,
+        ldx, ldy, C, C, Ntok, s1, float(eps), _dt(x), _stream())
+    _lib.check(code, "sana_hip_add_layernorm_modulate")
+    return total.view(B, Ntok, C), out.view(B, Ntok, C)

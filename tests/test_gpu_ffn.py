@@ -213,6 +213,20 @@ def test_layernorm_modulate_matches_stock_op_chain(cuda, B, Ntok, C):
     assert (diff == 0).float().mean().item() > 0.98
 
 
+@pytest.mark.parametrize("B,Ntok,C", [(1, 16384, 2240), (2, 77, 96), (3, 1024, 1152)])
+def test_add_layernorm_modulate_equals_add_then_norm(cuda, B, Ntok, C):
+    """x + y and LN(x + y) * (1 + scale) + shift in one pass: the sum is the stock bf16 add bit for bit, the
+    normalised output is the plain kernel's output on that sum bit for bit."""
+    g = torch.Generator().manual_seed(C + B)
+    x = (torch.randn(B, Ntok, C, generator=g) * 2 + 0.3).bfloat16().to(cuda)
+    y = torch.randn(B, Ntok, C, generator=g).bfloat16().to(cuda)
+    mod = (torch.randn(B, 6, C, generator=g) * 0.3).bfloat16().to(cuda)
+    shift, scale = mod[:, 3:4], mod[:, 4:5]
+    total, out = ops.add_layernorm_modulate(x, y, scale, shift, 1e-6)
+    assert torch.equal(total, x + y)
+    assert torch.equal(out, ops.layernorm_modulate(x + y, scale, shift, 1e-6))
+
+
 @pytest.mark.parametrize("C,T,P,B", [(64, 4, 30, 1), (128, 6, 35, 2), (2240, 3, 300, 1)])
 def test_temporal_conv_residual_matches_conv2d(cuda, C, T, P, B):
     """x + t_conv(x) over frames (zero frame in front, zeros behind) against F.conv2d in fp64, with the
