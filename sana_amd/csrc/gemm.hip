@@ -379,7 +379,9 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     const int base = total >> 3, rem = total & 7;
     pid = xcd * base + min(xcd, rem) + local;
   }
-  constexpr int GROUP = 8;
+  // tile rows per group: an XCD's 32 concurrent tiles are GROUP rows x 32/GROUP columns.  Measured: 4 is 1-2 % better
+  // for the short-K wide-N shapes (qkv, inverted conv), 8 is 2-3 % better for the long-K point conv.
+  const int GROUP = K >= 4096 ? 8 : 4;
   const int group_sz = GROUP * tiles_c;
   const int gid = pid / group_sz;
   const int first_t = gid * GROUP;
