@@ -4,14 +4,15 @@
 // problem of its own (3.5 x 3.5 MFMA tiles, padded to 4 x 4 with zero channels):
 //
 //   phase 1  workgroup = (batch, head, chunk, token split); each of its four waves takes interleaved
-//            32-token tiles and owns a whole 128 x 128 accumulator (256 registers).  Tiles go through
-//            wave-private LDS to become token-contiguous MFMA operands, as in the head_dim-32 kernel;
-//            the waves are summed in LDS in two rounds and a second kernel sums the splits in a
-//            fixed order.
-//   phase 2  workgroup = (batch, head, chunk, 64-token range); wave w produces output channels
-//            [32w, 32w+32) from its own slice of the state (two bf16 terms of the fp32 values as
-//            MFMA 16x16x32 A operands for bf16 output, three for fp32 output) plus a row block that
-//            carries ksum in every row, so each lane gets its token's denominator.
+//            32-token tiles (16 with on-load transforms) and owns a whole 128 x 128 accumulator (256
+//            registers).  Tiles go through wave-private LDS to become token-contiguous MFMA operands, as
+//            in the head_dim-32 kernel; the waves are summed in LDS (two padded accumulator images) and
+//            a second kernel sums the splits in a fixed order.
+//   phase 2  workgroup = (batch, head, chunk, range of 192..512 tokens), steps of 32 tokens through
+//            workgroup-shared LDS tiles; wave w produces output channels [32w, 32w+32) from its own slice
+//            of the state (two bf16 terms of the fp32 values as MFMA 16x16x32 A operands for bf16 output,
+//            three for fp32 output) plus a row block that carries ksum in every row, so each lane gets
+//            its token's denominator.
 #include "common.h"
 #include "linattn_common.h"
 
