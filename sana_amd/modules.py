@@ -685,8 +685,12 @@ class SanaMSBlock(nn.Module):
                  ffn_type="mlp", mlp_acts=("silu", "silu", None), linear_head_dim=32, cross_norm=False,
                  cross_attn_type="flash", **block_kwargs):
         super().__init__()
-        if attn_type != "linear" or ffn_type != "glumbconv":
+        # "triton_linear" is the reference's Triton twin of the same attention (TritonLiteMLA,
+        # fastlinear/modules/triton_lite_mla.py:104-121: qkv without bias, proj, no qk-norm): same math, same keys
+        if attn_type not in ("linear", "triton_linear") or ffn_type != "glumbconv":
             raise NotImplementedError("this block is the attn_type='linear' / ffn_type='glumbconv' hot path only")
+        if attn_type == "triton_linear":
+            qk_norm = False
         if cross_attn_type not in ("flash", "linear"):
             raise NotImplementedError(f"cross_attn_type={cross_attn_type!r}")
         if drop_path > 0.0:

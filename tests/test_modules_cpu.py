@@ -41,6 +41,14 @@ def test_qk_norm_keys():
     assert sorted(a.state_dict()) == sorted(b.state_dict())
 
 
+def test_triton_linear_is_the_same_attention():
+    """attn_type="triton_linear" (the reference's fused Triton twin) builds the same module with the same keys."""
+    a = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="triton_linear", ffn_type="glumbconv", qk_norm=True)
+    b = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv")
+    assert list(a.state_dict()) == list(b.state_dict())
+    assert isinstance(a.attn, S.LiteLA) and isinstance(a.attn.q_norm, torch.nn.Identity)
+
+
 def test_unsupported_options_fail_loudly():
     with pytest.raises(NotImplementedError):
         S.LiteLA(128, 128, dim=64)          # head dims with kernels: 32 and 112
