@@ -549,6 +549,93 @@ class CachedGLUMBConvTemp(GLUMBConvTemp):
 # --------------------------------------------------------------------------
 
 
+class LinearLayer(nn.Module):
+    """diffusion/model/nets/basic_modules_linear.py:32-58 (no norm)."""
+
+    def __init__(self, in_dim, out_dim, use_bias=True, norm=None, act=None):
+        super().__init__()
+        if norm is not None:
+            raise NotImplementedError("the hot path builds every LinearLayer with norm=None")
+        self.in_dim, self.out_dim, self.use_bias = in_dim, out_dim, use_bias
+        self.linear = nn.Linear(in_dim, out_dim, bias=use_bias)
+        self.norm = None
+        self.act = make_act(act)
+
+    def forward(self, x):
+        x = self.linear(x)
+        if self.act:
+            x = self.act(x)
+        return x
+
+
+class GLUMBConvLinear(nn.Module):
+    """diffusion/model/nets/basic_modules_linear.py:133-241: the Mix-FFN with its two 1x1 convolutions held as
+    ``nn.Linear`` over tokens (keys ``inverted_conv.linear.*``, ``point_conv.linear.*``); the depthwise 3x3 stays
+    a ConvLayer.  ``HW=None`` means a square grid (:206-207)."""
+
+    def __init__(self, in_features, hidden_features, out_feature=None, kernel_size=3, stride=1,
+                 padding=None, use_bias=False, norm=(None, None, None),
+                 act=("silu", "silu", None), dilation=1):
+        out_feature = out_feature or in_features
+        super().__init__()
+        use_bias = as_tuple(use_bias, 3)
+        norm = as_tuple(norm, 3)
+        act = as_tuple(act, 3)
+        self.hidden_features = hidden_features
+        self.out_feature = out_feature
+        self.glu_act = make_act(act[1], inplace=False)
+        self.inverted_conv = LinearLayer(in_features, hidden_features * 2, use_bias=use_bias[0], norm=norm[0],
+                                         act=act[0])
+        self.depth_conv = ConvLayer(hidden_features * 2, hidden_features * 2, kernel_size,
+                                    stride=stride, groups=hidden_features * 2, padding=padding,
+                                    use_bias=use_bias[1], norm=norm[1], act=None, dilation=dilation)
+        self.point_conv = LinearLayer(hidden_features, out_feature, use_bias=use_bias[2], norm=norm[2], act=act[2])
+
+    def _frames(self, x, HW):
+        """:204-236 up to the point conv: tokens [B, N, C] -> [frames, H*W, hidden]."""
+        B, N, C = x.shape
+        if HW is None:
+            H = W = int(N ** 0.5)
+            frames = B
+        elif len(HW) == 2:
+            (H, W), frames = HW, B
+        else:
+            T, H, W = HW
+            frames = B * T
+        x = self.inverted_conv(x)
+        x = x.reshape(frames, H, W, -1).permute(0, 3, 1, 2)
+        x = self.depth_conv(x)
+        a, g = torch.chunk(x, 2, dim=1)
+        x = a * self.glu_act(g)
+        return x.reshape(frames, self.hidden_features, H * W).permute(0, 2, 1)
+
+    def forward(self, x, HW=None):
+        B, N, C = x.shape
+        return self.point_conv(self._frames(x, HW).reshape(B, N, self.hidden_features))
+
+
+class GLUMBConvLinearTemp(GLUMBConvLinear):
+    """diffusion/model/nets/basic_modules_linear.py:243-311: GLUMBConvLinear per frame, then ``x + t_conv(x)``."""
+
+    def __init__(self, in_features, hidden_features, out_feature=None, kernel_size=3, stride=1, padding=None,
+                 use_bias=False, norm=(None, None, None), act=("silu", "silu", None), t_kernel_size=3):
+        super().__init__(in_features, hidden_features, out_feature=out_feature, kernel_size=kernel_size,
+                         stride=stride, padding=padding, use_bias=use_bias, norm=norm, act=act)
+        out_feature = out_feature or in_features
+        self.t_conv = nn.Conv2d(out_feature, out_feature, kernel_size=(t_kernel_size, 1), stride=1,
+                                padding=(t_kernel_size // 2, 0), bias=False)
+        nn.init.zeros_(self.t_conv.weight)
+
+    def forward(self, x, HW=None, **kwargs):
+        B, N, C = x.shape
+        assert len(HW) == 3, "HW must be a tuple of (T, H, W)"
+        T, H, W = HW
+        x = self.point_conv(self._frames(x, HW))                       # (B*T, H*W, out)
+        x = x.reshape(B, T, H * W, self.out_feature).permute(0, 3, 1, 2)
+        x_out = x + self.t_conv(x)
+        return x_out.permute(0, 2, 3, 1).reshape(B, N, self.out_feature)
+
+
 class MultiHeadCrossAttention(nn.Module):
     """diffusion/model/nets/sana_blocks.py:48-98, branch without xformers (:86-92)."""
 
@@ -591,16 +678,17 @@ class SanaMSBlock(nn.Module):
                  attn_type="flash", ffn_type="mlp", mlp_acts=("silu", "silu", None),
                  linear_head_dim=32, cross_norm=False, cross_attn_type="flash", **block_kwargs):
         super().__init__()
-        if attn_type != "linear" or ffn_type != "glumbconv":
-            raise NotImplementedError("oracle restates attn_type='linear', ffn_type='glumbconv' only")
+        if attn_type != "linear" or ffn_type not in ("glumbconv", "glumbconv_linear"):
+            raise NotImplementedError("oracle restates attn_type='linear', ffn_type='glumbconv[_linear]' only")
         self.hidden_size = hidden_size
         self.norm1 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
         self.attn = LiteLA(hidden_size, hidden_size, heads=hidden_size // linear_head_dim,
                            eps=1e-8, qk_norm=qk_norm)
         self.cross_attn = MultiHeadCrossAttention(hidden_size, num_heads, qk_norm=cross_norm)
         self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
-        self.mlp = GLUMBConv(hidden_size, int(hidden_size * mlp_ratio), use_bias=(True, True, False),
-                             norm=(None, None, None), act=mlp_acts)
+        ffn = GLUMBConv if ffn_type == "glumbconv" else GLUMBConvLinear          # :117-133
+        self.mlp = ffn(hidden_size, int(hidden_size * mlp_ratio), use_bias=(True, True, False),
+                       norm=(None, None, None), act=mlp_acts)
         self.drop_path = nn.Identity()
         self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
 

@@ -69,6 +69,43 @@ def blocks_state_dict(blocks: Iterable[torch.nn.Module], prefix: str = "blocks."
     return out
 
 
+_FFN_POINTWISE = ("inverted_conv", "point_conv")
+
+
+def ffn_conv_to_linear(state_dict: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """Keys of ``ffn_type="glumbconv"`` -> ``ffn_type="glumbconv_linear"``: ``<pointwise>.conv.weight``
+    [out, in, 1, 1] -> ``<pointwise>.linear.weight`` [out, in], biases renamed (the mapping stated at
+    basic_modules_linear.py:142-146).  Other keys pass through; tensors are views, not copies."""
+    out = {}
+    for k, v in unwrap(state_dict).items():
+        for base in _FFN_POINTWISE:
+            tag = base + ".conv."
+            if tag in k:
+                k = k.replace(tag, base + ".linear.")
+                if k.endswith("weight"):
+                    if v.dim() != 4 or v.shape[2:] != (1, 1):
+                        raise ValueError(f"{k}: expected a 1x1 convolution weight, got {tuple(v.shape)}")
+                    v = v[:, :, 0, 0]
+        out[k] = v
+    return out
+
+
+def ffn_linear_to_conv(state_dict: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """The inverse of :func:`ffn_conv_to_linear`."""
+    out = {}
+    for k, v in unwrap(state_dict).items():
+        for base in _FFN_POINTWISE:
+            tag = base + ".linear."
+            if tag in k:
+                k = k.replace(tag, base + ".conv.")
+                if k.endswith("weight"):
+                    if v.dim() != 2:
+                        raise ValueError(f"{k}: expected a linear weight, got {tuple(v.shape)}")
+                    v = v[:, :, None, None]
+        out[k] = v
+    return out
+
+
 def to_diffusers(state_dict: Dict[str, torch.Tensor], prefix: str = "blocks.") -> Dict[str, torch.Tensor]:
     """Block keys of a reference state dict -> ``transformer_blocks.{i}.*`` (convert_sana_to_diffusers.py:152-222)."""
     sd = unwrap(state_dict)

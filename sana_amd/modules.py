@@ -395,12 +395,24 @@ class GLUMBConv(nn.Module):
             raise NotImplementedError("GLUMBConv HIP path: norm must be (None, None, None)")
         if tuple(act) != ("silu", "silu", None):
             raise NotImplementedError("GLUMBConv HIP path: act must be ('silu', 'silu', None)")
+        self.hidden_features = hidden_features
+        self.out_feature = out_feature
         self.glu_act = nn.SiLU(inplace=False)
-        self.inverted_conv = ConvLayer(in_features, hidden_features * 2, 1, use_bias=use_bias[0], act="silu")
+        self.inverted_conv = self._pointwise_layer(in_features, hidden_features * 2, use_bias[0], "silu")
         self.depth_conv = ConvLayer(hidden_features * 2, hidden_features * 2, 3, groups=hidden_features * 2,
                                     use_bias=use_bias[1], act=None)
-        self.point_conv = ConvLayer(hidden_features, out_feature, 1, use_bias=use_bias[2], act=None)
+        self.point_conv = self._pointwise_layer(hidden_features, out_feature, use_bias[2], None)
         self.round_like_reference = True
+
+    # the two token-wise linears: 1x1 convolutions here (keys ``*.conv.weight`` [out, in, 1, 1]),
+    # nn.Linear in GLUMBConvLinear (keys ``*.linear.weight`` [out, in]); the same GEMM either way
+    @staticmethod
+    def _pointwise_layer(in_dim, out_dim, use_bias, act) -> nn.Module:
+        return ConvLayer(in_dim, out_dim, 1, use_bias=use_bias, act=act)
+
+    @staticmethod
+    def _pointwise_params(layer: nn.Module) -> nn.Module:
+        return layer.conv
 
     def forward(self, x: torch.Tensor, HW=None) -> torch.Tensor:
         return self.forward_gated(x, HW, None, None)
@@ -411,7 +423,7 @@ class GLUMBConv(nn.Module):
         _no_grad_only(x)
         B, N, C = x.shape
         if HW is None:
-            raise ValueError("GLUMBConv needs HW (the reference fails on HW=None too: basic_modules.py:193)")
+            HW = self._default_hw(N)
         if len(HW) == 2:
             frames, (H, W) = B, HW
         else:
@@ -419,15 +431,20 @@ class GLUMBConv(nn.Module):
             frames = B * T
         if frames * H * W != B * N:
             raise ValueError(f"HW={HW} does not match N={N}")
-        ic, dc, pc = self.inverted_conv.conv, self.depth_conv.conv, self.point_conv.conv
+        ic, pc = self._pointwise_params(self.inverted_conv), self._pointwise_params(self.point_conv)
+        dc = self.depth_conv.conv
         u = hip_linear(x, ic.weight, ic.bias, "silu", getattr(ic, "weight_q", None), getattr(ic, "weight_scale", None))
         y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
                                     round_like_reference=self.round_like_reference)
         return hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
                           getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual, out)
 
+    @staticmethod
+    def _default_hw(n_tokens: int):
+        raise ValueError("GLUMBConv needs HW (the reference fails on HW=None too: basic_modules.py:193)")
+
     def quantize_w8_(self) -> "GLUMBConv":
-        for conv in (self.inverted_conv.conv, self.point_conv.conv):
+        for conv in (self._pointwise_params(self.inverted_conv), self._pointwise_params(self.point_conv)):
             wq, scale = quantize_w8(conv.weight.data)
             conv.register_buffer("weight_q", wq.contiguous())
             conv.register_buffer("weight_scale", scale.contiguous())
@@ -438,8 +455,9 @@ class GLUMBConv(nn.Module):
 class GLUMBConvTemp(GLUMBConv):
     """Mix-FFN per frame plus a residual temporal conv (reference: basic_modules.py:200-264):
     ``x + t_conv(x)`` with ``t_conv`` a (t, 1) convolution over frames that mixes all channels,
-    zero-initialised.  The per-frame part runs the HIP kernels; the temporal conv stays a stock op
-    (it is outside the hot path), applied to a channels-last view of the token-major buffer."""
+    zero-initialised.  The per-frame part runs the HIP kernels; the temporal conv runs as one MFMA GEMM
+    over the token-major frames (bf16, 3 taps, C % 64 == 0, no frame mask) or as the stock convolution
+    on a channels-last view of the same buffer otherwise."""
 
     def __init__(self, in_features: int, hidden_features: int, out_feature=None, kernel_size=3, stride=1,
                  padding=None, use_bias=False, norm=(None, None, None), act=("silu", "silu", None), t_kernel_size=3):
@@ -597,6 +615,46 @@ class CachedGLUMBConvTemp(GLUMBConvTemp):
         return out
 
 
+class LinearLayer(nn.Module):
+    """Parameter holder with the reference's attribute names (basic_modules_linear.py:32-58):
+    ``linear`` (nn.Linear), ``norm`` (None), ``act``; its own forward is the stock op."""
+
+    def __init__(self, in_dim, out_dim, use_bias=True, act=None):
+        super().__init__()
+        self.in_dim, self.out_dim, self.use_bias = in_dim, out_dim, use_bias
+        self.linear = nn.Linear(in_dim, out_dim, bias=use_bias)
+        self.norm = None
+        self.act = nn.SiLU(inplace=True) if act == "silu" else None
+
+    def forward(self, x):
+        x = self.linear(x)
+        return self.act(x) if self.act else x
+
+
+class GLUMBConvLinear(GLUMBConv):
+    """The Mix-FFN with its 1x1 convolutions held as ``nn.Linear`` (reference: basic_modules_linear.py:133-241,
+    ``ffn_type="glumbconv_linear"``): keys ``inverted_conv.linear.{weight,bias}``, ``depth_conv.conv.*``,
+    ``point_conv.linear.weight``.  Same kernels as GLUMBConv; ``HW=None`` means a square grid (:206-207)."""
+
+    @staticmethod
+    def _pointwise_layer(in_dim, out_dim, use_bias, act) -> nn.Module:
+        return LinearLayer(in_dim, out_dim, use_bias=use_bias, act=act)
+
+    @staticmethod
+    def _pointwise_params(layer: nn.Module) -> nn.Module:
+        return layer.linear
+
+    @staticmethod
+    def _default_hw(n_tokens: int):
+        side = int(n_tokens ** 0.5)
+        return side, side
+
+
+class GLUMBConvLinearTemp(GLUMBConvLinear, GLUMBConvTemp):
+    """GLUMBConvLinear per frame plus the residual temporal conv (reference: basic_modules_linear.py:243-311);
+    constructor and forward of GLUMBConvTemp, parameters of GLUMBConvLinear."""
+
+
 # ------------------------------------------------------------------ the block
 
 
@@ -687,8 +745,8 @@ class SanaMSBlock(nn.Module):
         super().__init__()
         # "triton_linear" is the reference's Triton twin of the same attention (TritonLiteMLA,
         # fastlinear/modules/triton_lite_mla.py:104-121: qkv without bias, proj, no qk-norm): same math, same keys
-        if attn_type not in ("linear", "triton_linear") or ffn_type != "glumbconv":
-            raise NotImplementedError("this block is the attn_type='linear' / ffn_type='glumbconv' hot path only")
+        if attn_type not in ("linear", "triton_linear") or ffn_type not in ("glumbconv", "glumbconv_linear"):
+            raise NotImplementedError("this block is the attn_type='linear' / ffn_type='glumbconv[_linear]' hot path only")
         if attn_type == "triton_linear":
             qk_norm = False
         if cross_attn_type not in ("flash", "linear"):
@@ -700,8 +758,9 @@ class SanaMSBlock(nn.Module):
         self.attn = LiteLA(hidden_size, hidden_size, heads=hidden_size // linear_head_dim, eps=1e-8, qk_norm=qk_norm)
         self.cross_attn = MultiHeadCrossAttention(hidden_size, num_heads, qk_norm=cross_norm, **block_kwargs)
         self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
-        self.mlp = GLUMBConv(in_features=hidden_size, hidden_features=int(hidden_size * mlp_ratio),
-                             use_bias=(True, True, False), norm=(None, None, None), act=mlp_acts)
+        ffn = GLUMBConv if ffn_type == "glumbconv" else GLUMBConvLinear      # sana_multi_scale.py:117-133
+        self.mlp = ffn(in_features=hidden_size, hidden_features=int(hidden_size * mlp_ratio),
+                       use_bias=(True, True, False), norm=(None, None, None), act=mlp_acts)
         self.drop_path = nn.Identity()
         self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
 

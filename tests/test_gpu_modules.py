@@ -239,3 +239,38 @@ def test_guidance_processor_patched_over_attn_forward(cuda, mode):
         hb.attn.forward = pag.SelfAttnProcessorLiteLA(hb.attn)     # what the sampler leaves behind
         assert torch.equal(hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW), plain) or \
             (hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW).float() - plain.float()).abs().max().item() <= 2 ** -5
+
+
+def test_glumbconv_linear_block_and_temporal_variant(cuda):
+    """ffn_type="glumbconv_linear" (nn.Linear parameters, basic_modules_linear.py:133-311): the block, the module with
+    the HW=None square default, the W8A16 form and the temporal variant against the fp64 oracle."""
+    C, heads, B, HW = 256, 8, 2, (12, 12)
+    ob = O.init_block_(O.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv_linear"), 3)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(4)
+        for n, p in ob.named_parameters():
+            if n.endswith("bias"):
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+    ob = ob.bfloat16()
+    hb = S.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv_linear").bfloat16()
+    hb.load_state_dict(ob.state_dict(), strict=True)
+    hb = hb.to(cuda)
+    x, y, t = (a.bfloat16() for a in O.block_inputs(B, HW[0] * HW[1], C, seed=3))
+    with torch.no_grad():
+        check(hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW), _ref64(ob, x, y, t, HW=HW), "block, linear FFN", block=True)
+        ref = _ref64(ob.mlp, x, HW=HW)
+        check(hb.mlp(x.to(cuda), HW=HW), ref, "GLUMBConvLinear")
+        check(hb.mlp(x.to(cuda)), ref, "GLUMBConvLinear, HW=None")
+        check(hb.mlp(x.to(cuda), HW=(2, 12, 6)), _ref64(ob.mlp, x, HW=(2, 12, 6)), "GLUMBConvLinear, video HW")
+        # W8A16 against the oracle holding the dequantised weights
+        sd = dict(ob.mlp.state_dict())
+        for k in ("inverted_conv.linear.weight", "point_conv.linear.weight"):
+            sd[k] = O.dequantize_w8(*O.quantize_w8(sd[k]))
+        oq = O.GLUMBConvLinear(C, int(C * 2.5), use_bias=(True, True, False)).bfloat16()
+        oq.load_state_dict(sd, strict=True)
+        hb.mlp.quantize_w8_()
+        check(hb.mlp(x.to(cuda), HW=HW), _ref64(oq, x, HW=HW), "GLUMBConvLinear W8A16")
+        (T, H, W) = (4, 5, 6)
+        om, hm = _temp_pair("GLUMBConvLinearTemp", 128, 320, 7)
+        xt = torch.randn(1, T * H * W, 128, generator=torch.Generator().manual_seed(12)).bfloat16()
+        check(hm.to(cuda)(xt.to(cuda), HW=(T, H, W)), _ref64(om, xt, HW=(T, H, W)), "GLUMBConvLinearTemp")

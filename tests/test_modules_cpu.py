@@ -12,7 +12,7 @@ from oracle import sana_oracle as O
 
 @pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention", "LiteLAReLURope",
                                   "CachedCausalAttention", "GLUMBConvTemp", "ChunkGLUMBConvTemp",
-                                  "CachedGLUMBConvTemp"])
+                                  "CachedGLUMBConvTemp", "GLUMBConvLinear", "GLUMBConvLinearTemp"])
 def test_constructor_and_forward_signatures_match(name):
     a, b = getattr(S, name), getattr(O, name)
     pa = list(inspect.signature(a.__init__).parameters)
@@ -47,6 +47,29 @@ def test_triton_linear_is_the_same_attention():
     b = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv")
     assert list(a.state_dict()) == list(b.state_dict())
     assert isinstance(a.attn, S.LiteLA) and isinstance(a.attn.q_norm, torch.nn.Identity)
+
+
+def test_glumbconv_linear_keys_and_checkpoint_conversion():
+    """ffn_type="glumbconv_linear": the reference's key names, and a glumbconv checkpoint converts both ways."""
+    from sana_amd import checkpoint as ck
+    ob = O.init_block_(O.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv_linear"), 0)
+    hb = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv_linear")
+    assert isinstance(hb.mlp, S.GLUMBConvLinear) and hb.mlp.hidden_features == 160 and hb.mlp.out_feature == 64
+    assert list(ob.state_dict()) == list(hb.state_dict())
+    assert "mlp.inverted_conv.linear.weight" in hb.state_dict() and "mlp.point_conv.linear.bias" not in hb.state_dict()
+    hb.load_state_dict(ob.state_dict(), strict=True)
+    conv_blk = S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv")
+    conv_blk.load_state_dict(ck.ffn_linear_to_conv(hb.state_dict()), strict=True)
+    back = ck.ffn_conv_to_linear(conv_blk.state_dict())
+    assert list(back) == list(hb.state_dict())
+    for k, v in hb.state_dict().items():
+        assert torch.equal(back[k], v), k
+    with pytest.raises(ValueError):
+        ck.ffn_conv_to_linear({"mlp.inverted_conv.conv.weight": torch.zeros(4, 4, 3, 3)})
+    q = S.GLUMBConvLinear(64, 160, use_bias=(True, True, False)).bfloat16().quantize_w8_()
+    assert "inverted_conv.linear.weight_q" in q.state_dict() and "point_conv.linear.weight" not in q.state_dict()
+    t = S.GLUMBConvLinearTemp(64, 160, use_bias=(True, True, False))
+    assert isinstance(t.point_conv, S.modules.LinearLayer) and t.t_conv.weight.abs().max().item() == 0.0
 
 
 def test_unsupported_options_fail_loudly():

@@ -177,3 +177,49 @@ def test_cached_stream_equals_chunked_temporal_conv_and_frame_mask():
     wm = whole(x, HW=(T, Hh, Ww), frame_valid_mask=mask).view(2, T, P, C)
     assert wm[:, 5:].abs().max().item() == 0.0
     torch.testing.assert_close(wm[:, :4], w.view(2, T, P, C)[:, :4], rtol=1e-12, atol=1e-12)
+
+
+# ---- GLUMBConvLinear (basic_modules_linear.py:133-311): the same function with nn.Linear parameters
+
+
+def _linear_twin(conv_module, linear_cls, **kw):
+    """A *Linear module holding conv_module's weights under the mapping stated at basic_modules_linear.py:142-146."""
+    from sana_amd import checkpoint as ck
+    twin = linear_cls(**kw).double()
+    twin.load_state_dict(ck.ffn_conv_to_linear(conv_module.state_dict()), strict=True)
+    return twin
+
+
+def test_linear_variant_is_the_same_function_as_the_conv_variant():
+    """A 1x1 convolution over a channels-first image is a matmul over its pixels: with the stated weight mapping
+    GLUMBConvLinear must reproduce GLUMBConv (itself pinned by the brute-force taps above) on image and video HW,
+    and its HW=None default must be the square grid."""
+    kw = dict(in_features=24, hidden_features=40, use_bias=(True, True, False))
+    conv = O.GLUMBConv(**kw).double()
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        for p in conv.parameters():
+            p.copy_(torch.randn(p.shape, generator=g, dtype=torch.float64) * 0.3)
+    lin = _linear_twin(conv, O.GLUMBConvLinear, **kw)
+    assert sorted(lin.state_dict()) == ["depth_conv.conv.bias", "depth_conv.conv.weight", "inverted_conv.linear.bias",
+                                        "inverted_conv.linear.weight", "point_conv.linear.weight"]
+    assert lin.state_dict()["inverted_conv.linear.weight"].shape == (80, 24)
+    x = torch.randn(2, 36, 24, generator=g, dtype=torch.float64)
+    for hw in [(6, 6), (4, 9), (2, 3, 6), (3, 4, 3)]:
+        torch.testing.assert_close(lin(x, HW=hw), conv(x, HW=hw), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(lin(x), conv(x, HW=(6, 6)), rtol=1e-12, atol=1e-12)
+    # a non-square grid must differ from the square default (the reshape is not a no-op)
+    assert (lin(x, HW=(4, 9)) - lin(x)).abs().max() > 1e-3
+
+
+def test_linear_temporal_variant_matches_the_conv_temporal_variant():
+    kw = dict(in_features=16, hidden_features=24, use_bias=(True, True, False))
+    conv = O.GLUMBConvTemp(**kw).double()
+    g = torch.Generator().manual_seed(4)
+    with torch.no_grad():
+        for p in conv.parameters():
+            p.copy_(torch.randn(p.shape, generator=g, dtype=torch.float64) * 0.3)
+    lin = _linear_twin(conv, O.GLUMBConvLinearTemp, **kw)
+    assert "t_conv.weight" in lin.state_dict()
+    x = torch.randn(2, 5 * 12, 16, generator=g, dtype=torch.float64)
+    torch.testing.assert_close(lin(x, HW=(5, 3, 4)), conv(x, HW=(5, 3, 4)), rtol=1e-12, atol=1e-12)
