@@ -436,7 +436,7 @@ class GLUMBConv(nn.Module):
         u = hip_linear(x, ic.weight, ic.bias, "silu", getattr(ic, "weight_q", None), getattr(ic, "weight_scale", None))
         y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
                                     round_like_reference=self.round_like_reference)
-        return hip_linear(y.view(B, N, -1), pc.weight, pc.bias, None,
+        return hip_linear(y.view(B, N, y.shape[-1]), pc.weight, pc.bias, None,
                           getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual, out)
 
     @staticmethod

@@ -1,5 +1,7 @@
 """Tensor-level wrappers over the C ABI: shape/dtype/device checks, pointer and
 stride extraction, launch on torch's current stream.  Forward only, no autograd.
+Empty inputs (no batch entries or no tokens) are answered here, after the argument
+checks, without a launch: empty outputs, and an all-zero state for no tokens.
 """
 from __future__ import annotations
 
@@ -110,6 +112,8 @@ def qk_rms(q: torch.Tensor, k: torch.Tensor, eps: float) -> Tuple[torch.Tensor, 
     sb, sn = _token_major_view(q, "q")
     rq = torch.empty(B, N, dtype=torch.float32, device=q.device)
     rk = torch.empty(B, N, dtype=torch.float32, device=q.device)
+    if B * N == 0:
+        return rq, rk
     code = _lib.load().sana_hip_qk_rms(q.data_ptr(), k.data_ptr(), rq.data_ptr(), rk.data_ptr(), B, N, C, sb, sn,
                                        float(eps), _dt(q), _stream())
     _lib.check(code, "sana_hip_qk_rms")
@@ -151,6 +155,10 @@ def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: b
     tab, n_chunks, longest = chunk_table(chunk_tokens, N, k.device)
     lib = _lib.load()
     state = torch.empty(B, h, n_chunks, d + 1, d, dtype=torch.float32, device=k.device)
+    if B * N == 0:
+        if pre is not None:
+            pre.check(k, d)
+        return state.zero_()
     nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, d, n_chunks, longest, _dt(k))
     ws = _workspace(k.device, nbytes)
     args = (k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
@@ -198,6 +206,10 @@ def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens
     elif out.shape != q.shape or out.dtype != out_dtype:
         raise SanaHipError("out has the wrong shape or dtype")
     osb, osn = _token_major_view(out, "out")
+    if B * N == 0:
+        if pre is not None:
+            pre.check(q, d)
+        return out
     args = (q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, d, qsb, qsn, osb, osn,
             tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype])
     if pre is None:
@@ -231,6 +243,8 @@ def dwconv3x3_silu_gate(u: torch.Tensor, weight: torch.Tensor, bias: Optional[to
     if bias is not None and (bias.numel() != C2 or bias.dtype != u.dtype or not bias.is_contiguous()):
         raise SanaHipError("bias must be contiguous [2*Ch] in u's dtype")
     y = torch.empty(BT, H, W, C2 // 2, dtype=u.dtype, device=u.device)
+    if y.numel() == 0:
+        return y
     code = _lib.load().sana_hip_dwconv3x3_silu_gate(
         u.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(),
         BT, H, W, C2 // 2, 1 if round_like_reference else 0, _dt(u), _stream())
@@ -268,6 +282,10 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     if out is None:
         out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
     out, ldc = _rows(out, "out")
+    if tuple(out.shape) != (M, N) or out.dtype != torch.bfloat16:
+        raise SanaHipError("out has the wrong shape or dtype")
+    if M == 0:
+        return out
     code = _lib.load().sana_hip_gemm_bf16(a.data_ptr(), weight.data_ptr(),
                                           bias.data_ptr() if bias is not None else None, out.data_ptr(),
                                           M, N, K, lda, ldw, ldc, epi, _stream())
@@ -318,6 +336,10 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
     if out is None:
         out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
     out, ldc = _rows(out, "out")
+    if tuple(out.shape) != (M, N) or out.dtype != torch.bfloat16:
+        raise SanaHipError("out has the wrong shape or dtype")
+    if M == 0:
+        return out
     code = _lib.load().sana_hip_gemm_w8a16(a.data_ptr(), wq.data_ptr(), scale.data_ptr(),
                                            bias.data_ptr() if bias is not None else None, out.data_ptr(),
                                            M, N, K, lda, ldw, ldc, epi, _stream())
@@ -353,6 +375,8 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
     g2, gstride = _mod_rows(gate, B, C, "gate")
     out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=a.device)
+    if B * Ntok == 0:
+        return out.view(B, Ntok, C)
     code = _lib.load().sana_hip_gemm_gate_residual(
         a2.data_ptr(), w2.data_ptr(), weight_scale.data_ptr() if weight_scale is not None else None,
         bias.data_ptr() if bias is not None else None, g2.data_ptr(), r2.data_ptr(), out.data_ptr(),
@@ -383,6 +407,8 @@ def tconv_residual(xp: torch.Tensor, weight: torch.Tensor, n_rows: int, tap_rows
     o2, ldo = _rows(out, "out")
     if tuple(o2.shape) != (n_rows, C) or o2.dtype != torch.bfloat16:
         raise SanaHipError("out has the wrong shape or dtype")
+    if n_rows == 0:
+        return out
     code = _lib.load().sana_hip_tconv_residual(x2.data_ptr(), w2.data_ptr(), o2.data_ptr(), n_rows, C, taps,
                                                tap_rows, rows, ldx, ldw, ldo, _stream())
     _lib.check(code, "sana_hip_tconv_residual")
@@ -399,6 +425,8 @@ def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor
     if s1 != s2:
         raise SanaHipError("scale and shift must share their batch stride")
     out = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
+    if B * Ntok == 0:
+        return out.view(B, Ntok, C)
     code = _lib.load().sana_hip_layernorm_modulate(x2.data_ptr(), sc.data_ptr(), sh.data_ptr(), out.data_ptr(),
                                                    B * Ntok, C, ldx, C, Ntok, s1, float(eps), _dt(x), _stream())
     _lib.check(code, "sana_hip_layernorm_modulate")
@@ -420,6 +448,8 @@ def add_layernorm_modulate(x: torch.Tensor, y: torch.Tensor, scale: torch.Tensor
         raise SanaHipError("scale and shift must share their batch stride")
     total = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
     out = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
+    if B * Ntok == 0:
+        return total.view(B, Ntok, C), out.view(B, Ntok, C)
     code = _lib.load().sana_hip_add_layernorm_modulate(
         x2.data_ptr(), y2.data_ptr(), sc.data_ptr(), sh.data_ptr(), total.data_ptr(), out.data_ptr(), B * Ntok, C,
         ldx, ldy, C, C, Ntok, s1, float(eps), _dt(x), _stream())

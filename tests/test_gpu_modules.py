@@ -274,3 +274,27 @@ def test_glumbconv_linear_block_and_temporal_variant(cuda):
         om, hm = _temp_pair("GLUMBConvLinearTemp", 128, 320, 7)
         xt = torch.randn(1, T * H * W, 128, generator=torch.Generator().manual_seed(12)).bfloat16()
         check(hm.to(cuda)(xt.to(cuda), HW=(T, H, W)), _ref64(om, xt, HW=(T, H, W)), "GLUMBConvLinearTemp")
+
+
+def test_empty_inputs(cuda):
+    """No batch entries / no tokens: the stock ops of the reference return empty tensors (and a sum over no tokens
+    is zero); the drop-in answers the same way without a launch."""
+    from sana_amd import ops
+    C, heads = 128, 4
+    ob, hb = _pair(C, heads)
+    hb = hb.to(cuda)
+    with torch.no_grad():
+        # (the block itself cannot take B = 0: `t.reshape(B, 6, -1)` of sana_multi_scale.py:147 is ambiguous there)
+        x0 = torch.zeros(0, 16, C, dtype=torch.bfloat16, device=cuda)
+        assert hb.attn(x0, HW=(4, 4)).shape == (0, 16, C)
+        assert hb.mlp(x0, HW=(4, 4)).shape == (0, 16, C)
+        xn = torch.zeros(2, 0, C, dtype=torch.bfloat16, device=cuda)
+        assert hb.attn(xn, HW=(0, 0)).shape == (2, 0, C)
+        assert hb.mlp(xn, HW=(0, 0)).shape == (2, 0, C)
+        st = ops.linattn_state(xn, xn)
+        assert st.shape == (2, C // 32, 1, 33, 32) and st.abs().max().item() == 0.0
+        assert ops.linattn_apply(xn, st, 1e-8).shape == (2, 0, C)
+        rq, rk = ops.qk_rms(xn, xn, 1e-5)
+        assert rq.shape == (2, 0)
+        # the oracle agrees on the shapes
+        assert ob.attn(x0.cpu(), HW=(4, 4)).shape == (0, 16, C) and ob.mlp(x0.cpu(), HW=(4, 4)).shape == (0, 16, C)
