@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 3
+#define SANA_HIP_ABI_VERSION 4
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -191,10 +191,20 @@ int sana_hip_dwconv3x3_silu_gate(const void* u, const void* w, const void* bias,
  *   bias  [N] bf16 or NULL (must be non-NULL for SANA_EPI_BIAS*)
  *   C     [M][N] row-major with row stride ldc
  * K and N must be multiples of 8 (16-byte rows); lda, ldw, ldc multiples of 8.
+ *
+ * workspace (optional): a shape with too few output tiles to occupy the chip (few tokens, narrow N, long
+ * K: the proj and point-conv GEMMs of a single 1024 px image) runs faster as a split-k GEMM -- K cut into
+ * up to 8 ranges whose fp32 partial results go through the workspace and are summed in a fixed order by a
+ * second kernel that applies the epilogue.  sana_hip_gemm_workspace_bytes(M, N, K) is the size that
+ * needs (0: this shape is never split).  With workspace NULL, misaligned or smaller than that, the GEMM
+ * runs unsplit -- same result up to the fp32 summation order.  The plan depends on (M, N, K) only, so the
+ * int8-weight GEMM and the gated-residual GEMM split the same way and stay bit-identical to this one.
  */
+size_t sana_hip_gemm_workspace_bytes(int M, int N, int K);
+
 int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
-                       int epilogue, void* stream);
+                       int epilogue, void* workspace, size_t workspace_bytes, void* stream);
 
 /* W8A16: W is int8 [N][K] with a per-output-channel fp32 scale [N].  Each
  * weight is dequantised in registers as bf16_rne(float(q) * scale[n]) — the same
@@ -204,7 +214,7 @@ int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
  * benchmark configuration.  K and ldw must be multiples of 16. */
 int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias,
                         void* C, int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
-                        int epilogue, void* stream);
+                        int epilogue, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Fused seams around the two modules (the reference runs them as separate
@@ -219,12 +229,14 @@ int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, con
  *   rows_per_gate consecutive rows of C (= tokens per batch element);
  *   residual: bf16 [M][N] with row stride ldr (may alias C).  bias may be NULL.
  *   The linear output, the gate product and the sum are each rounded to bf16,
- *   as the reference's three ops do.
+ *   as the reference's three ops do.  workspace: as for sana_hip_gemm_bf16
+ *   (optional split-k).
  */
 int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_scale, const void* bias,
                                 const void* gate, const void* residual, void* C,
                                 int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc,
-                                int rows_per_gate, int64_t gate_stride, void* stream);
+                                int rows_per_gate, int64_t gate_stride,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* LayerNorm without affine (eps inside the rsqrt) + adaLN modulation:
  *   out[m][:] = LN(x[m][:]) * (1 + scale[m / rows_per_mod][:]) + shift[m / rows_per_mod][:]

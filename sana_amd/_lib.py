@@ -39,16 +39,17 @@ SIGNATURES = {
                                            c_void_p, c_void_p, c_void_p, c_void_p]),
     "sana_hip_dwconv3x3_silu_gate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                              c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "sana_hip_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "sana_hip_gemm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                   c_int64, c_int64, c_int64, c_int, c_void_p]),
+                                   c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "sana_hip_gemm_w8a16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                    c_int64, c_int64, c_int64, c_int, c_void_p]),
+                                    c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "sana_hip_dequant_w8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int64, c_void_p]),
     "sana_hip_tconv_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                         c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "sana_hip_gemm_gate_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64,
-                                            c_int, c_int64, c_void_p]),
+                                            c_int, c_int64, c_void_p, c_size_t, c_void_p]),
     "sana_hip_add_layernorm_modulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                 c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int64, c_float,
                                                 c_int, c_void_p]),

@@ -88,6 +88,9 @@ struct Taps {
   int kc;          // columns per tap, a multiple of the k-tile
   int64_t stride;  // rows between taps
   int64_t rows;
+  // split-k launches (SPLIT, never together with taps): grid row z works on k-tiles
+  // [z*split_tiles + min(z, split_rem), ...) -- split_tiles of them, one more for z < split_rem
+  int split_tiles, split_rem;
 };
 
 // 8 outputs of one row: accumulator (+bias) -> io dtype, per the epilogue kind (everything except
@@ -364,14 +367,28 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 // Rows past M / N read as zero (buffer range check) and only feed outputs that are
 // never stored; the last k-tile runs just the k-steps that exist.  Needs K % 16 == 0 and K >= 64.
 // ============================================================================
-template <bool W8, int EPI, int NI, bool TAPS = false>
-__global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
+// SPLIT (split-k, for shapes with too few tiles to fill the chip): grid row z multiplies its own range of
+// k-tiles and stores the raw fp32 accumulators to C taken as float [gridDim.y][M][N]; splitk_epilogue_kernel
+// adds the ranges up in order and applies the epilogue.
+template <bool W8, int EPI, int NI, bool TAPS = false, bool SPLIT = false>
+__global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A_, const void* __restrict__ Wv_,
                                                     const float* __restrict__ scale, const EpiArgs ep,
-                                                    uint16_t* __restrict__ C, int M, int N, int K, int64_t lda,
+                                                    uint16_t* __restrict__ C, int M, int N, int K_, int64_t lda,
                                                     int64_t ldw, int64_t ldc, int tiles_t, int tiles_c,
                                                     const Taps tp) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint16_t* A = A_;
+  const void* Wv = Wv_;
+  int K = K_;
+  if (SPLIT) {  // this grid row's k range becomes "the" K of everything below
+    const int z = blockIdx.y;
+    const int kb = (z * tp.split_tiles + min(z, tp.split_rem)) * BK;
+    const int kn = (tp.split_tiles + (z < tp.split_rem ? 1 : 0)) * BK;
+    A += kb;
+    Wv = static_cast<const char*>(Wv_) + (int64_t)kb * (W8 ? 1 : 2);
+    K = min(K_ - kb, kn);
+  }
   const int total = tiles_t * tiles_c;
   int pid = blockIdx.x;
   {
@@ -597,6 +614,32 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
   // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
   // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
+  if (SPLIT) {
+    // raw accumulators -> partial[z][M][N] (fp32, dense): a lane owns 16 consecutive channels of one token per
+    // MFMA tile, stored as four 16-byte pieces through a buffer resource over the wave's rows of this range's
+    // plane (rows past M fall outside it and are dropped; channel pieces past N get the idle offset)
+    const int prow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;
+    const int prows = max(0, min(128, M - prow0));
+    float* plane = reinterpret_cast<float*>(C) + ((int64_t)blockIdx.y * M + prow0) * N;
+    const __amdgpu_buffer_rsrc_t rsrc_p =
+        __builtin_amdgcn_make_buffer_rsrc(plane, 0, (int)((int64_t)prows * N * 4), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row_off = ((32 * j + fr) * N + n) * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2],
+                      v3 = acc[i][j][4 * q + 3];
+          const u32x4_t o = {__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)};
+          __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n + 4 * q < N ? row_off + 16 * q : (int)0x80000000u, 0, 0);
+        }
+      }
+    }
+    return;
+  }
   __syncthreads();  // every wave is done with the operand tiles
   unsigned char* stg = smem + wave * 32768;
   // Global accesses of the epilogue are buffer loads / stores on the wave's 128 rows of C (and of the
@@ -694,6 +737,38 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   }
 }
 
+// Second half of a split-k GEMM: partial[S][M][N] (fp32) -> C = epilogue(sum over the S k-ranges, added in
+// order).  One thread per row and 8 channels; the same epilogue functions as the fused path.
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_epilogue_kernel(const float* __restrict__ partial, int S,
+                                                               const EpiArgs ep, uint16_t* __restrict__ C, int M, int N,
+                                                               int64_t ldc) {
+  const int chunks = N >> 3;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (int64_t)M * chunks) return;
+  const int m = (int)(id / chunks), n = (int)(id - (int64_t)m * chunks) * 8;
+  const f32x4_t* p = reinterpret_cast<const f32x4_t*>(partial + (int64_t)m * N + n);
+  const int64_t plane = (int64_t)M * N / 4;
+  f32x4_t lo = p[0], hi = p[1];
+  for (int z = 1; z < S; ++z) {
+    lo += p[z * plane];
+    hi += p[z * plane + 1];
+  }
+  const float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  float bv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (EPI != SANA_EPI_NONE && ep.bias) {
+    const u32x4_t b = *reinterpret_cast<const u32x4_t*>(ep.bias + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      bv[2 * e] = bf16_lo(b[e]);
+      bv[2 * e + 1] = bf16_hi(b[e]);
+    }
+  }
+  u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a, bv);
+  if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
+  *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
+}
+
 int compute_units() {
   static int n = 0;  // same value from every thread that races here
   if (n == 0) {
@@ -706,12 +781,85 @@ int compute_units() {
   return n;
 }
 
+// Channel tile of the pipelined kernel (NI = 4: 256 channels, 3: 192).  One workgroup per compute unit at a
+// time, so the grid runs in rounds: the tile whose rounds x tile size is smaller wins; the narrower tile
+// re-reads a little more per MFMA, hence its 4 % handicap.
+int pick_ni(int M, int N) {
+  const int64_t cu = compute_units(), tiles_t = (M + BT - 1) / BT;
+  const int64_t t256 = tiles_t * ((N + 255) / 256), t192 = tiles_t * ((N + 191) / 192);
+  const double cost256 = (double)((t256 + cu - 1) / cu) * 4.0, cost192 = (double)((t192 + cu - 1) / cu) * 3.0 * 1.04;
+  return cost192 < cost256 ? 3 : 4;
+}
+
+// Split-k plan.  A grid of fewer tiles than half the compute units leaves most of the chip idle for a whole
+// K loop (M = 1024 tokens x N = 2240: 48 workgroups on 256 CUs), and a workgroup's K loop is a latency chain of
+// about 1.1 us per k-tile whatever the grid.  Cutting K into S ranges (>= 8 k-tiles each, S <= 8, S x tiles
+// <= CUs) shortens the chain to ceil(KT / S) k-tiles and costs the fp32 partial planes -- S x M x N x 4 bytes
+// written and read once, about 3 bytes/ns at these sizes -- plus a second launch (about 5 us).  S minimises
+// that estimate and is used when it beats the unsplit chain by 15 %: long-K narrow-N shapes (the point conv of
+// a few thousand tokens or less) split, wide-N or short-K ones do not.
+struct SplitPlan {
+  int S, tiles, rem;  // ranges; k-tiles per range; ranges that take one more
+};
+SplitPlan plan_split(int M, int N, int K) {
+  SplitPlan pl = {1, 0, 0};
+  if (K % 16 || K < 64) return pl;
+  const int ni = pick_ni(M, N);
+  const int64_t tiles = (int64_t)((M + BT - 1) / BT) * ((N + 64 * ni - 1) / (64 * ni));
+  const int KT = (K + BK - 1) / BK, cu = compute_units();
+  if (tiles * 2 > cu || KT < 16 || (int64_t)M * N * 4 >= ((int64_t)1 << 31)) return pl;
+  int smax = (int)(cu / tiles);
+  if (smax > KT / 8) smax = KT / 8;
+  if (smax > 8) smax = 8;
+  const double us_tile = 1.1, us_launch = 5.0, bytes_per_us = 3.0e6;
+  const double unsplit = KT * us_tile;
+  double best = unsplit * 0.85;
+  int S = 1;
+  for (int s = 2; s <= smax; ++s) {
+    const double t = (KT + s - 1) / s * us_tile + (double)s * M * N * 8.0 / bytes_per_us + us_launch;
+    if (t < best) {
+      best = t;
+      S = s;
+    }
+  }
+  if (S < 2) return pl;
+  pl.S = S;
+  pl.tiles = KT / S;
+  pl.rem = KT % S;
+  return pl;
+}
+size_t split_bytes(const SplitPlan& pl, int M, int N) { return pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0; }
+
 template <bool W8, int NI>
 int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N, int K,
-            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr) {
+            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr,
+            float* ws = nullptr, size_t ws_bytes = 0) {
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + 64 * NI - 1) / (64 * NI);
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
-  const Taps none = {0, 0, 0};
+  const Taps none = {0, 0, 0, 0, 0};
+  if (!taps && ws) {  // split-k when it pays and the caller's workspace holds the partial planes
+    const SplitPlan pl = plan_split(M, N, K);
+    if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
+      const Taps split = {0, 0, 0, pl.tiles, pl.rem};
+      hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, false, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
+                         a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
+                         split);
+      if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+      const int64_t threads = (int64_t)M * (N / 8);
+      dim3 egrid((unsigned)((threads + 255) / 256));
+#define SANA_SPLIT_EPI(EPI) \
+  hipLaunchKernelGGL((splitk_epilogue_kernel<EPI>), egrid, block, 0, s, ws, pl.S, ep, c, M, N, ldc)
+      switch (epilogue) {
+        case SANA_EPI_NONE: SANA_SPLIT_EPI(SANA_EPI_NONE); break;
+        case SANA_EPI_BIAS: SANA_SPLIT_EPI(SANA_EPI_BIAS); break;
+        case SANA_EPI_BIAS_SILU: SANA_SPLIT_EPI(SANA_EPI_BIAS_SILU); break;
+        case SANA_EPI_GATE_RES: SANA_SPLIT_EPI(SANA_EPI_GATE_RES); break;
+        default: return SANA_ERR_ARG;
+      }
+#undef SANA_SPLIT_EPI
+      return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+    }
+  }
   if (taps) {  // only the bf16 gated-residual instance exists with taps
     if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
     hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, true>), grid, block, 0, s, a, W, scale, ep, c, M, N,
@@ -734,20 +882,17 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
 
 template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
-           int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr) {
+           int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr,
+           void* workspace = nullptr, size_t workspace_bytes = 0) {
   const int64_t tiles_t = (M + BT - 1) / BT;
   if (tiles_t * ((N + 127) / 128) > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
   if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
-    // One workgroup per compute unit at a time, so the grid runs in rounds: pick the channel tile
-    // (256 or 192) whose rounds x tile size is smaller; the narrower tile re-reads a little more
-    // per MFMA, hence its 4 % handicap.
-    const int64_t cu = compute_units();
-    const int64_t t256 = tiles_t * ((N + 255) / 256), t192 = tiles_t * ((N + 191) / 192);
-    const double cost256 = (double)((t256 + cu - 1) / cu) * 4.0, cost192 = (double)((t192 + cu - 1) / cu) * 3.0 * 1.04;
-    return cost192 < cost256 ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps)
-                             : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps);
+    float* ws = aligned16(workspace) ? static_cast<float*>(workspace) : nullptr;
+    return pick_ni(M, N) == 3
+               ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes)
+               : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes);
   }
   if (taps) return SANA_ERR_SHAPE;
   const int tiles_c = (N + BC - 1) / BC;
@@ -797,29 +942,36 @@ using namespace sana;
 
 #define SANA_API extern "C" __attribute__((visibility("default")))
 
+SANA_API size_t sana_hip_gemm_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || N % 8) return 0;
+  return split_bytes(plan_split(M, N, K), M, N);
+}
+
 SANA_API int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,
-                                int64_t lda, int64_t ldw, int64_t ldc, int epilogue, void* stream) {
+                                int64_t lda, int64_t ldw, int64_t ldc, int epilogue, void* workspace,
+                                size_t workspace_bytes, void* stream) {
   if (epilogue == SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   const int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, epilogue, 8, 8);
   if (rc != SANA_OK) return rc;
   return launch<false>(A, W, nullptr, plain_epi(bias), C, M, N, K, lda, ldw, ldc, epilogue,
-                       static_cast<hipStream_t>(stream));
+                       static_cast<hipStream_t>(stream), nullptr, workspace, workspace_bytes);
 }
 
 SANA_API int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias, void* C,
                                  int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
-                                 void* stream) {
+                                 void* workspace, size_t workspace_bytes, void* stream) {
   if (!scale || epilogue == SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   const int rc = check_common(A, Wq, bias, C, M, N, K, lda, ldw, ldc, epilogue, 16, 16);
   if (rc != SANA_OK) return rc;
   return launch<true>(A, Wq, scale, plain_epi(bias), C, M, N, K, lda, ldw, ldc, epilogue,
-                      static_cast<hipStream_t>(stream));
+                      static_cast<hipStream_t>(stream), nullptr, workspace, workspace_bytes);
 }
 
 SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_scale, const void* bias,
                                          const void* gate, const void* residual, void* C, int M, int N, int K,
                                          int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc, int rows_per_gate,
-                                         int64_t gate_stride, void* stream) {
+                                         int64_t gate_stride, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
   const bool w8 = w8_scale != nullptr;
   int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, w8 ? 16 : 8, w8 ? 16 : 8);
   if (rc != SANA_OK) return rc;
@@ -828,8 +980,10 @@ SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const flo
   const EpiArgs e = {static_cast<const uint16_t*>(bias), static_cast<const uint16_t*>(gate),
                      static_cast<const uint16_t*>(residual), ldr, gate_stride, rows_per_gate};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return w8 ? launch<true>(A, W, w8_scale, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s)
-            : launch<false>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s);
+  return w8 ? launch<true>(A, W, w8_scale, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s, nullptr, workspace,
+                           workspace_bytes)
+            : launch<false>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s, nullptr, workspace,
+                            workspace_bytes);
 }
 
 SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,
@@ -843,7 +997,7 @@ SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, in
   if (x_rows * ldx * 2 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;  // 32-bit byte offsets inside the buffer
   const uint16_t* x = static_cast<const uint16_t*>(X);
   const EpiArgs e = {nullptr, nullptr, x + (taps / 2) * tap_rows * ldx, ldx, 0, M};
-  const Taps tp = {C, tap_rows, x_rows};
+  const Taps tp = {C, tap_rows, x_rows, 0, 0};
   return launch<false>(X, W, nullptr, e, out, M, C, taps * C, ldx, ldw, ldo, SANA_EPI_GATE_RES,
                        static_cast<hipStream_t>(stream), &tp);
 }

@@ -262,6 +262,17 @@ def _rows(t: torch.Tensor, what: str) -> Tuple[torch.Tensor, int]:
     return t, t.stride(0)
 
 
+SPLIT_K = True   # False: never hand the GEMMs a workspace (they then run unsplit; used by tests)
+
+
+def _gemm_workspace(lib, device, M: int, N: int, K: int) -> Tuple[Optional[int], int]:
+    """(pointer, bytes) of the split-k workspace this shape wants, or (None, 0): shapes with few output tiles
+    run as a split-k GEMM through fp32 partial planes in the per-device workspace."""
+    nbytes = lib.sana_hip_gemm_workspace_bytes(M, N, K) if SPLIT_K else 0
+    ws = _workspace(device, nbytes)
+    return (ws.data_ptr(), nbytes) if ws is not None else (None, 0)
+
+
 def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
               epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a: [M, K] bf16; weight: [N, K] bf16 (nn.Linear layout).  Returns epilogue(a @ weight.T) [M, N] bf16."""
@@ -286,9 +297,10 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
         raise SanaHipError("out has the wrong shape or dtype")
     if M == 0:
         return out
-    code = _lib.load().sana_hip_gemm_bf16(a.data_ptr(), weight.data_ptr(),
-                                          bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                                          M, N, K, lda, ldw, ldc, epi, _stream())
+    lib = _lib.load()
+    ws, nbytes = _gemm_workspace(lib, a.device, M, N, K)
+    code = lib.sana_hip_gemm_bf16(a.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                  out.data_ptr(), M, N, K, lda, ldw, ldc, epi, ws, nbytes, _stream())
     _lib.check(code, "sana_hip_gemm_bf16")
     return out
 
@@ -340,9 +352,11 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
         raise SanaHipError("out has the wrong shape or dtype")
     if M == 0:
         return out
-    code = _lib.load().sana_hip_gemm_w8a16(a.data_ptr(), wq.data_ptr(), scale.data_ptr(),
-                                           bias.data_ptr() if bias is not None else None, out.data_ptr(),
-                                           M, N, K, lda, ldw, ldc, epi, _stream())
+    lib = _lib.load()
+    ws, nbytes = _gemm_workspace(lib, a.device, M, N, K)
+    code = lib.sana_hip_gemm_w8a16(a.data_ptr(), wq.data_ptr(), scale.data_ptr(),
+                                   bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                                   M, N, K, lda, ldw, ldc, epi, ws, nbytes, _stream())
     _lib.check(code, "sana_hip_gemm_w8a16")
     return out
 
@@ -377,10 +391,12 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=a.device)
     if B * Ntok == 0:
         return out.view(B, Ntok, C)
-    code = _lib.load().sana_hip_gemm_gate_residual(
+    lib = _lib.load()
+    ws, nbytes = _gemm_workspace(lib, a.device, B * Ntok, C, K)
+    code = lib.sana_hip_gemm_gate_residual(
         a2.data_ptr(), w2.data_ptr(), weight_scale.data_ptr() if weight_scale is not None else None,
         bias.data_ptr() if bias is not None else None, g2.data_ptr(), r2.data_ptr(), out.data_ptr(),
-        B * Ntok, C, K, lda, ldw, ldr, C, Ntok, gstride, _stream())
+        B * Ntok, C, K, lda, ldw, ldr, C, Ntok, gstride, ws, nbytes, _stream())
     _lib.check(code, "sana_hip_gemm_gate_residual")
     return out.view(B, Ntok, C)
 

@@ -32,7 +32,7 @@ def test_exports_every_declared_symbol():
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.sana_hip_abi_version() == 3
+    assert lib.sana_hip_abi_version() == 4
     assert b"aligned" in lib.sana_hip_strerror(-3)
     assert b"unknown" in lib.sana_hip_strerror(-99)
 
@@ -54,9 +54,9 @@ def test_argument_validation_needs_no_gpu():
     assert lib.sana_hip_linattn_state(16, 16, 16, 16, 1 << 30, 1, 16, 1, 112, 0, 96, None, 1, 16, 0, BF16, None) == -1
     assert lib.sana_hip_linattn_apply(16, 16, 16, 1, 16, 1, 112, 0, 112, 0, 112, None, 1, 16, 1e-8, F16, F16, None) == -6
     assert lib.sana_hip_dwconv3x3_silu_gate(16, 16, None, 16, 1, 4, 4, 3, 1, 1, None) == -2  # odd Ch
-    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 20, 24, 24, 8, 0, None) == -2      # K % 8
-    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None) == -1      # bias epilogue, no bias
-    assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None) == -1  # no scale
+    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 20, 24, 24, 8, 0, None, 0, None) == -2      # K % 8
+    assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None, 0, None) == -1      # bias epilogue, no bias
+    assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None, 0, None) == -1  # no scale
     # temporal conv: C % 64, odd taps, the centre tap must exist for every output row
     assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 96, 3, 16, 80, 96, 288, 96, None) == -2
     assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 2, 16, 80, 64, 128, 64, None) == -1
@@ -75,6 +75,20 @@ def test_workspace_query():
     # head_dim 112 always goes through per-split partial states: 20 heads at the video shape -> 12 splits
     assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 1, 32760, 1) == 20 * 12 * 113 * 112 * 4
     assert lib.sana_hip_linattn_workspace_bytes(1, 20, 64, 1, 32760, 1) == 0   # no kernel for this head dim
+
+
+def test_gemm_split_k_workspace_query():
+    """Shapes with fewer output tiles than half the compute units (256 assumed without a device) are split
+    along K through fp32 partial planes; shapes that fill the chip, short K loops and int8-only shapes are not."""
+    lib = _lib.load()
+    # one 1024 px image at Sana-1.6B: point conv 1024 x 2240 x 5600 -> 4 x 12 tiles of 256 x 192, 88 k-tiles, 4 ranges
+    assert lib.sana_hip_gemm_workspace_bytes(1024, 2240, 5600) == 4 * 1024 * 2240 * 4
+    # 256 tokens through the proj GEMM (35 k-tiles): at most one range per 8 k-tiles
+    assert lib.sana_hip_gemm_workspace_bytes(256, 2240, 2240) == 4 * 256 * 2240 * 4
+    # not split: grids that fill the chip, wide N or short K (the partial planes would cost more than the loop saves)
+    for M, N, K in ((16384, 2240, 5600), (16384, 11200, 2240), (1024, 11200, 2240), (1024, 2240, 2240),
+                    (1024, 3456, 1152), (1024, 2240, 512), (0, 8, 64), (256, 2244, 5600)):
+        assert lib.sana_hip_gemm_workspace_bytes(M, N, K) == 0, (M, N, K)
 
 
 def test_ops_refuse_cpu_tensors():

@@ -166,6 +166,53 @@ def test_gemm_w8a16_equals_bf16_gemm_on_dequantised_weight(cuda, M, N, K, epilog
     assert rel_l2(y8.cpu(), ref) <= 4e-3
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 2240, 5600),    # point conv of one 1024 px image: 4 k ranges
+                                   (256, 2240, 2240),     # 4 ranges of 9, 9, 9 and 8 k-tiles
+                                   (1000, 1152, 2880),    # ragged rows, 600M widths
+                                   (300, 72, 1168),       # two tiles, k ranges of 10 and 9 k-tiles, a k tail of one k-step
+                                   (2048, 2240, 5600)])   # 2 ranges
+def test_gemm_split_k(cuda, monkeypatch, M, N, K):
+    """Shapes with too few output tiles run as split-k through the workspace: against the fp64 oracle to the same
+    bounds as the fused path, against the unsplit kernel to fp32 summation-order noise, bit-identical between the
+    bf16, int8 and gated-residual entry points (they share the plan), and exact on integer inputs."""
+    from sana_amd import _lib
+    assert _lib.load().sana_hip_gemm_workspace_bytes(M, N, K) > 0
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(cuda)
+    w = torch.empty(N, K)
+    torch.nn.init.trunc_normal_(w, std=0.03, generator=g)
+    wq, s = O.quantize_w8(w.bfloat16())
+    wd = O.dequantize_w8(wq, s).to(cuda)
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16().to(cuda)
+    outs = {}
+    for epilogue in (None, "bias", "bias_silu"):
+        b = bias if epilogue else None
+        y = ops.gemm_bf16(a, wd, b, epilogue)
+        ref = _gemm_ref(a.cpu(), wd.cpu(), None if b is None else b.cpu(), epilogue)
+        assert rel_l2(y.cpu(), ref) <= 4e-3
+        assert ((y.cpu().double() - ref).abs() > 2e-2 + 2 ** -7 * ref.abs()).sum().item() == 0
+        assert torch.equal(ops.gemm_w8a16(a, wq.to(cuda), s.to(cuda), b, epilogue, expand=False), y)
+        outs[epilogue] = y
+    mod = (torch.randn(1, 6, N, generator=g) * 0.5).bfloat16().to(cuda)
+    res = torch.randn(1, M, N, generator=g).bfloat16().to(cuda)
+    gated = ops.gemm_gate_residual(a.view(1, M, K), wd, bias, mod[:, 2:3], res)
+    assert torch.equal(gated, res + mod[:, 2:3] * outs["bias"].view(1, M, N))
+    monkeypatch.setattr(ops, "SPLIT_K", False)
+    for epilogue, y in outs.items():
+        y1 = ops.gemm_bf16(a, wd, bias if epilogue else None, epilogue)
+        # same products, another fp32 summation order: the linear output moves by at most one bf16 ulp (plus fp32
+        # noise where it cancels to ~0), and only on a few outputs; SiLU of an output that moved by one ulp moves by
+        # up to ~|x| ulps of its own small value in the negative tail, hence the absolute term there
+        diff = (y.float() - y1.float()).abs()
+        floor = 2e-2 if epilogue == "bias_silu" else 1e-4
+        assert (diff > 2 ** -7 * y1.float().abs() + floor).sum().item() == 0
+        assert (diff > 0).float().mean().item() < 0.05
+    monkeypatch.setattr(ops, "SPLIT_K", True)
+    ai = torch.randint(-2, 3, (M, K), generator=g).bfloat16()
+    wi = torch.randint(-1, 2, (N, K), generator=g).bfloat16()
+    assert torch.equal(ops.gemm_bf16(ai.to(cuda), wi.to(cuda)).cpu(), (ai.float() @ wi.float().T).bfloat16())
+
+
 # ---------------------------------------------------------------- fused seams of the block
 
 
