@@ -298,3 +298,32 @@ def test_empty_inputs(cuda):
         assert rq.shape == (2, 0)
         # the oracle agrees on the shapes
         assert ob.attn(x0.cpu(), HW=(4, 4)).shape == (0, 16, C) and ob.mlp(x0.cpu(), HW=(4, 4)).shape == (0, 16, C)
+
+
+def test_block_replays_from_a_hip_graph(cuda):
+    """The whole block (hand-written kernels, stock cross-attention, the cached workspace) captured once into a HIP
+    graph: every replay, with eager launches and synchronisations between them, reproduces the eager result bit
+    for bit, also after the input buffer's contents change."""
+    C, heads, B, HW = 256, 8, 2, (16, 16)
+    ob, hb = _pair(C, heads, seed=5)
+    hb = hb.to(cuda)
+    x, y, t = (a.bfloat16().to(cuda) for a in O.block_inputs(B, HW[0] * HW[1], C, seed=5))
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):           # warm-up off the default stream, as capture requires
+            for _ in range(2):
+                hb(x, y, t, HW=HW)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = hb(x, y, t, HW=HW)
+        for r in range(3):
+            if r == 2:
+                x.copy_(torch.randn(x.shape, generator=torch.Generator().manual_seed(9)).bfloat16())
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = hb(x, y, t, HW=HW)
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {r}"
+        check(out, _ref64(ob, x.cpu(), y.cpu(), t.cpu(), HW=HW), "graph replay vs fp64 oracle", block=True)
