@@ -174,13 +174,23 @@ __device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m,
   return o;
 }
 
-template <bool W8, int EPI>
-__global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
+// Compiler-scheduled kernel, any K % 8 == 0 (int8: K % 16 == 0).  Workgroup tile 64*TT tokens x 64*TC channels,
+// four waves in 2x2, each TT x TC MFMA tiles.  <4, 4>: the 256 x 256 tile of the pipelined kernel, for the K
+// values that one does not take.  <2, 2>: 128 x 128 with 64 accumulators and 64 KB of LDS, two workgroups per
+// CU -- a quarter of the work per k-tile, so a much shorter latency chain for shapes whose 256-wide grid would
+// leave the chip mostly idle (a few hundred to a few thousand tokens); its k-tiles are requested three ahead
+// (three register sets in rotation), because with so little math per k-tile the chain is otherwise one global
+// load latency per k-tile.  Every output sums its k products in the same order in all of these kernels, so
+// they agree bit for bit.
+template <bool W8, int EPI, int TT = 4, int TC = 4>
+__global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
                                                    const float* __restrict__ scale, const EpiArgs ep,
                                                    uint16_t* __restrict__ C,
                                                    int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                                                    int tiles_t, int tiles_c) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE_BYTES];  // [stage][A | W]
+  constexpr int BT = 64 * TT, BC = 64 * TC;              // shadow the file-scope 256 x 256
+  constexpr int A_BYTES = BT * ROW_BYTES, STAGE_BYTES = (BT + BC) * ROW_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE_BYTES];  // [stage][A | W]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
   // ---- workgroup -> tile, XCD aware: ids are dealt round-robin to the 8 XCDs, so
@@ -202,56 +212,58 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
   const int m0 = tile_t * BT, n0 = tile_c * BC;
 
   // ---- global -> register staging
-  // A tile: 256 rows x 8 chunks(16 B); thread -> chunk tid%8, rows tid/8 + 32*i
+  // A tile: BT rows x 8 chunks(16 B); thread -> chunk tid%8, rows tid/8 + 32*i
   const int a_chunk = tid & 7, a_row = tid >> 3;
-  u32x4_t ra[8];
-  // W tile bf16: same shape.  W8: 256 rows x 4 chunks of 16 int8; thread -> chunk tid%4, rows tid/4 + 64*i
-  u32x4_t rw[W8 ? 4 : 8];
+  constexpr int NA = 2 * TT, NW = W8 ? TC : 2 * TC;
+  constexpr int DEPTH = TT * TC <= 4 ? 3 : 1;  // k-tiles in flight in registers
+  u32x4_t ra[DEPTH][NA];
+  // W tile bf16: same shape.  W8: BC rows x 4 chunks of 16 int8; thread -> chunk tid%4, rows tid/4 + 64*i
+  u32x4_t rw[DEPTH][NW];
   const int w_chunk = W8 ? (tid & 3) : (tid & 7), w_row = W8 ? (tid >> 2) : (tid >> 3);
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 
-  auto load_tile = [&](int k0) {
+  // Operand tiles are read with buffer loads, one resource per operand over the tile's valid rows (ending with
+  // the last valid row's K-th element): rows past M / N fall outside it and read as zero, and a k chunk past K
+  // gets an offset outside it -- no branches around the loads, so that several k-tiles can stay in flight.
+  // (The whole offset is the vector offset: only that one is range-checked.)
+  const int a_last = min(BT, M - m0) - 1, w_last = min(BC, N - n0) - 1;
+  constexpr int WB = W8 ? 1 : 2;  // bytes per weight
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(A + (int64_t)m0 * lda), 0, (int)(((int64_t)a_last * lda + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * WB), 0,
+      (int)(((int64_t)w_last * ldw + K) * WB), 0x00020000);
+  const int idle_off = (int)0x80000000u;
+  const int voff_a = (a_row * (int)lda + a_chunk * 8) * 2, step_a = 32 * (int)lda * 2;
+  const int voff_w = (w_row * (int)ldw + w_chunk * (W8 ? 16 : 8)) * WB, step_w = (W8 ? 64 : 32) * (int)ldw * WB;
+  auto load_tile = [&](int set, int k0) {  // k chunks past K load zeros
+    const int off_a = k0 + a_chunk * 8 < K ? voff_a + k0 * 2 : idle_off;
+    const int off_w = k0 + w_chunk * (W8 ? 16 : 8) < K ? voff_w + k0 * WB : idle_off;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int m = m0 + a_row + 32 * i, k = k0 + a_chunk * 8;
-      ra[i] = (m < M && k < K) ? *reinterpret_cast<const u32x4_t*>(A + (int64_t)m * lda + k) : zero4;
-    }
-    if (W8) {
-      const int8_t* Wq = static_cast<const int8_t*>(Wv);
+    for (int i = 0; i < NA; ++i)
+      ra[set][i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off_a + i * step_a, 0, 0));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + w_row + 64 * i, k = k0 + w_chunk * 16;
-        // rows are 16-byte aligned and K % 16 == 0 on this path
-        rw[i] = (n < N && k < K) ? *reinterpret_cast<const u32x4_t*>(Wq + (int64_t)n * ldw + k) : zero4;
-      }
-    } else {
-      const uint16_t* Wb = static_cast<const uint16_t*>(Wv);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int n = n0 + w_row + 32 * i, k = k0 + w_chunk * 8;
-        rw[i] = (n < N && k < K) ? *reinterpret_cast<const u32x4_t*>(Wb + (int64_t)n * ldw + k) : zero4;
-      }
-    }
+    for (int i = 0; i < NW; ++i)
+      rw[set][i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, off_w + i * step_w, 0, 0));
   };
-  float wscale[4], woff[4];
+  float wscale[TC], woff[TC];
   if (W8) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < TC; ++i) {
       const int n = n0 + w_row + 64 * i;
       wscale[i] = n < N ? scale[n] : 0.f;
       woff[i] = -128.f * wscale[i];
     }
   }
-  auto store_tile = [&](int stage) {
-    unsigned char* sa = smem + stage * 2 * TILE_BYTES;
-    unsigned char* sw = sa + TILE_BYTES;
+  auto store_tile = [&](int set, int stage) {
+    unsigned char* sa = smem + stage * STAGE_BYTES;
+    unsigned char* sw = sa + A_BYTES;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(sa + swz(a_row + 32 * i, a_chunk)) = ra[i];
+    for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4_t*>(sa + swz(a_row + 32 * i, a_chunk)) = ra[set][i];
     if (W8) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < NW; ++i) {
         const int lrow = wrow_to_lds(w_row + 64 * i);
-        u32x4_t q = rw[i];
+        u32x4_t q = rw[set][i];
         q.x ^= 0x80808080u;
         q.y ^= 0x80808080u;
         q.z ^= 0x80808080u;
@@ -270,65 +282,74 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<u32x4_t*>(sw + swz(wrow_to_lds(w_row + 32 * i), w_chunk)) = rw[i];
+      for (int i = 0; i < NW; ++i)
+        *reinterpret_cast<u32x4_t*>(sw + swz(wrow_to_lds(w_row + 32 * i), w_chunk)) = rw[set][i];
     }
   };
 
-  // ---- MFMA tiling: wave (wc, wt) owns channels [wc*128, +128) x tokens [wt*128, +128)
+  // ---- MFMA tiling: wave (wc, wt) owns channels [wc*32*TC, +32*TC) x tokens [wt*32*TT, +32*TT)
   const int wc = wave & 1, wt = wave >> 1;
   const int fr = lane & 31, fg = lane >> 5;
-  f32x16_t acc[4][4];
+  f32x16_t acc[TC][TT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TC; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < TT; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int KT = (K + BK - 1) / BK;
-  load_tile(0);
-  store_tile(0);
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_tile(d, d * BK);
+  store_tile(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
+  // k-tile kt is multiplied from LDS stage kt % 2 while register set kt % DEPTH (which held it) is refilled with
+  // k-tile kt + DEPTH and set (kt + 1) % DEPTH goes to the other stage; unrolled by DEPTH so the set is static.
+  // The loop runs whole rounds of DEPTH: k-tiles past K are all zeros (they add nothing), and a body without
+  // exits keeps the compiler's count of outstanding loads exact.
+  for (int kt0 = 0; kt0 < KT; kt0 += DEPTH) {
+#pragma unroll
+   for (int d = 0; d < DEPTH; ++d) {
+    const int kt = kt0 + d;
     const int cur = kt & 1;
-    if (kt + 1 < KT) load_tile((kt + 1) * BK);
-    const unsigned char* sa = smem + cur * 2 * TILE_BYTES;
-    const unsigned char* sw = sa + TILE_BYTES;
+    load_tile(d, (kt + DEPTH) * BK);
+    const unsigned char* sa = smem + cur * STAGE_BYTES;
+    const unsigned char* sw = sa + A_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      u32x4_t fw[4], fa[4];
+      u32x4_t fw[TC], fa[TT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        fw[i] = *reinterpret_cast<const u32x4_t*>(sw + swz(wc * 128 + 32 * i + fr, 2 * ks + fg));
+      for (int i = 0; i < TC; ++i)
+        fw[i] = *reinterpret_cast<const u32x4_t*>(sw + swz(wc * 32 * TC + 32 * i + fr, 2 * ks + fg));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        fa[j] = *reinterpret_cast<const u32x4_t*>(sa + swz(wt * 128 + 32 * j + fr, 2 * ks + fg));
+      for (int j = 0; j < TT; ++j)
+        fa[j] = *reinterpret_cast<const u32x4_t*>(sa + swz(wt * 32 * TT + 32 * j + fr, 2 * ks + fg));
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < TC; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TT; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[i]),
                                                              __builtin_bit_cast(bf16x8_t, fa[j]), acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < KT) store_tile(cur ^ 1);
+    store_tile((d + 1) % DEPTH, cur ^ 1);
     __syncthreads();
+   }
   }
 
-  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 32*j + lane%32,
-  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r
+  // ---- epilogue.  acc[i][j][r]: token m0 + wt*32*TT + 32*j + lane%32,
+  // channel n0 + wc*32*TC + 32*i + 16*(lane/32) + r
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = n0 + wc * 128 + 32 * i + 16 * fg;
+  for (int i = 0; i < TC; ++i) {
+    const int n = n0 + wc * 32 * TC + 32 * i + 16 * fg;
     float bv[16];
     if (HAS_BIAS) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int m = m0 + wt * 128 + 32 * j + fr;
+    for (int j = 0; j < TT; ++j) {
+      const int m = m0 + wt * 32 * TT + 32 * j + fr;
       if (m >= M) continue;
       uint16_t* cp = C + (int64_t)m * ldc + n;
 #pragma unroll
@@ -791,44 +812,54 @@ int pick_ni(int M, int N) {
   return cost192 < cost256 ? 3 : 4;
 }
 
-// Split-k plan.  A grid of fewer tiles than half the compute units leaves most of the chip idle for a whole
-// K loop (M = 1024 tokens x N = 2240: 48 workgroups on 256 CUs), and a workgroup's K loop is a latency chain of
-// about 1.1 us per k-tile whatever the grid.  Cutting K into S ranges (>= 8 k-tiles each, S <= 8, S x tiles
-// <= CUs) shortens the chain to ceil(KT / S) k-tiles and costs the fp32 partial planes -- S x M x N x 4 bytes
-// written and read once, about 3 bytes/ns at these sizes -- plus a second launch (about 5 us).  S minimises
-// that estimate and is used when it beats the unsplit chain by 15 %: long-K narrow-N shapes (the point conv of
-// a few thousand tokens or less) split, wide-N or short-K ones do not.
-struct SplitPlan {
-  int S, tiles, rem;  // ranges; k-tiles per range; ranges that take one more
+// Which kernel, and whether K is split.  A workgroup's K loop is a latency chain whatever the grid: about
+// 1.1 us per k-tile for the 256-wide pipelined kernel, 0.8 us for the 128 x 128 one (a quarter of the math, but
+// the same load / LDS / barrier round trip).  A grid that covers the chip keeps the 256-wide kernel (throughput
+// is what counts, and that kernel has twice the math per byte).  A grid of fewer tiles than half the compute
+// units (M = 1024 tokens x N = 2240: 48 workgroups on 256 CUs) leaves most of the chip idle for the whole
+// chain; two remedies, by estimate:
+//  * split-k: S ranges of >= 8 k-tiles (S <= 8, S x tiles <= CUs) shorten the chain to ceil(KT / S) k-tiles and
+//    cost the fp32 partial planes (S x M x N x 4 bytes written and read once, about 3 bytes/ns at these sizes)
+//    plus a second launch (about 5 us); taken when that beats the unsplit chain by 15 %.  Long-K narrow-N
+//    shapes (the point conv of a few thousand tokens or less) split, wide-N or short-K ones do not.
+//  * the 128 x 128 kernel, when its grid still fits one workgroup per CU and its chain beats the above.
+struct GemmPlan {
+  bool small;         // the 128 x 128 kernel
+  int S, tiles, rem;  // k ranges; k-tiles per range; ranges that take one more
 };
-SplitPlan plan_split(int M, int N, int K) {
-  SplitPlan pl = {1, 0, 0};
-  if (K % 16 || K < 64) return pl;
-  const int ni = pick_ni(M, N);
-  const int64_t tiles = (int64_t)((M + BT - 1) / BT) * ((N + 64 * ni - 1) / (64 * ni));
+GemmPlan plan_gemm(int M, int N, int K, bool w8) {
+  GemmPlan pl = {false, 1, 0, 0};
   const int KT = (K + BK - 1) / BK, cu = compute_units();
-  if (tiles * 2 > cu || KT < 16 || (int64_t)M * N * 4 >= ((int64_t)1 << 31)) return pl;
-  int smax = (int)(cu / tiles);
-  if (smax > KT / 8) smax = KT / 8;
-  if (smax > 8) smax = 8;
-  const double us_tile = 1.1, us_launch = 5.0, bytes_per_us = 3.0e6;
-  const double unsplit = KT * us_tile;
-  double best = unsplit * 0.85;
-  int S = 1;
-  for (int s = 2; s <= smax; ++s) {
-    const double t = (KT + s - 1) / s * us_tile + (double)s * M * N * 8.0 / bytes_per_us + us_launch;
-    if (t < best) {
-      best = t;
-      S = s;
+  const bool pipelined = K % 16 == 0 && K >= 64;
+  const double us_tile = pipelined ? 1.1 : 1.4, us_tile_small = 0.8, us_launch = 5.0, bytes_per_us = 3.0e6;
+  double best = KT * us_tile;
+  if (pipelined) {
+    const int ni = pick_ni(M, N);
+    const int64_t tiles = (int64_t)((M + BT - 1) / BT) * ((N + 64 * ni - 1) / (64 * ni));
+    if (tiles * 2 <= cu && KT >= 16 && (int64_t)M * N * 4 < ((int64_t)1 << 31)) {
+      int smax = (int)(cu / tiles);
+      if (smax > KT / 8) smax = KT / 8;
+      if (smax > 8) smax = 8;
+      double bound = best * 0.85;
+      for (int s = 2; s <= smax; ++s) {
+        const double t = (KT + s - 1) / s * us_tile + (double)s * M * N * 8.0 / bytes_per_us + us_launch;
+        if (t < bound) {
+          bound = best = t;
+          pl.S = s;
+        }
+      }
     }
   }
-  if (S < 2) return pl;
-  pl.S = S;
-  pl.tiles = KT / S;
-  pl.rem = KT % S;
+  const int64_t tiles128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles128 <= cu && K % (w8 ? 16 : 8) == 0 && KT * us_tile_small + 3.0 < best) {
+    pl.small = true;
+    pl.S = 1;
+  }
+  pl.tiles = KT / pl.S;
+  pl.rem = KT % pl.S;
   return pl;
 }
-size_t split_bytes(const SplitPlan& pl, int M, int N) { return pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0; }
+size_t split_bytes(const GemmPlan& pl, int M, int N) { return pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0; }
 
 template <bool W8, int NI>
 int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N, int K,
@@ -838,7 +869,7 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
   const Taps none = {0, 0, 0, 0, 0};
   if (!taps && ws) {  // split-k when it pays and the caller's workspace holds the partial planes
-    const SplitPlan pl = plan_split(M, N, K);
+    const GemmPlan pl = plan_gemm(M, N, K, W8);
     if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
       const Taps split = {0, 0, 0, pl.tiles, pl.rem};
       hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, false, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
@@ -881,6 +912,25 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
 }
 
 template <bool W8>
+int launch_small(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N,
+                 int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
+  const int tiles_t = (M + 127) / 128, tiles_c = (N + 127) / 128;
+  dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
+#define SANA_LAUNCH_S(EPI)                                                                                          \
+  hipLaunchKernelGGL((gemm_kernel<W8, EPI, 2, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+                     tiles_t, tiles_c)
+  switch (epilogue) {
+    case SANA_EPI_NONE: SANA_LAUNCH_S(SANA_EPI_NONE); break;
+    case SANA_EPI_BIAS: SANA_LAUNCH_S(SANA_EPI_BIAS); break;
+    case SANA_EPI_BIAS_SILU: SANA_LAUNCH_S(SANA_EPI_BIAS_SILU); break;
+    case SANA_EPI_GATE_RES: SANA_LAUNCH_S(SANA_EPI_GATE_RES); break;
+    default: return SANA_ERR_ARG;
+  }
+#undef SANA_LAUNCH_S
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+template <bool W8>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr,
            void* workspace = nullptr, size_t workspace_bytes = 0) {
@@ -888,6 +938,8 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
   if (tiles_t * ((N + 127) / 128) > (1 << 30)) return SANA_ERR_SHAPE;
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
+  if (!taps && plan_gemm(M, N, K, W8).small)
+    return launch_small<W8>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
   if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
     float* ws = aligned16(workspace) ? static_cast<float*>(workspace) : nullptr;
     return pick_ni(M, N) == 3
@@ -918,6 +970,7 @@ int check_common(const void* A, const void* W, const void* bias, const void* C, 
   if (epilogue < SANA_EPI_NONE || epilogue > SANA_EPI_GATE_RES) return SANA_ERR_ARG;
   if (K % kmult || N % 8) return SANA_ERR_SHAPE;
   if (lda < K || ldw < K || ldc < N) return SANA_ERR_ARG;
+  if (lda >= (1 << 22) || ldw >= (1 << 22) || ldc >= (1 << 22)) return SANA_ERR_SHAPE;  // 32-bit offsets inside a tile's rows
   if (lda % 8 || ldw % ldw_mult || ldc % 8 || !aligned16(A) || !aligned16(W) || !aligned16(C)) return SANA_ERR_ALIGN;
   return SANA_OK;
 }
@@ -944,7 +997,7 @@ using namespace sana;
 
 SANA_API size_t sana_hip_gemm_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0 || N % 8) return 0;
-  return split_bytes(plan_split(M, N, K), M, N);
+  return split_bytes(plan_gemm(M, N, K, false), M, N);
 }
 
 SANA_API int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,

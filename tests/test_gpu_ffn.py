@@ -95,6 +95,9 @@ GEMM_SHAPES = [
     (31, 24, 80),         # two k-tiles, the second with one k-step; fewer than 32 rows either side
     (260, 520, 136),      # K % 16 != 0: the generic kernel
     (129, 1000, 208),     # k tail of one k-step after three full tiles
+    (1024, 2240, 2240),   # proj of one 1024 px image: the 128 x 128 kernel (144 tiles, one per CU)
+    (520, 264, 1160),     # the 128 x 128 kernel with K % 16 != 0, ragged rows and channels, 19 k-tiles (not a multiple of 3)
+    (200, 136, 1024),     # the 128 x 128 kernel, 16 k-tiles
 ]
 
 
@@ -218,7 +221,8 @@ def test_gemm_split_k(cuda, monkeypatch, M, N, K):
 
 @pytest.mark.parametrize("B,Ntok,C,K,w8", [(1, 16384, 2240, 2240, False), (2, 1024, 2240, 5600, False),
                                           (3, 100, 96, 240, False), (2, 1024, 2240, 5600, True),
-                                          (7, 20, 96, 128, False)])   # several gate rows inside one 32-token group
+                                          (7, 20, 96, 128, False),    # several gate rows inside one 32-token group
+                                          (2, 512, 1152, 1152, False), (3, 100, 264, 1152, True)])  # the 128 x 128 kernel
 def test_gemm_gate_residual_matches_stock_op_chain(cuda, B, Ntok, C, K, w8):
     g = torch.Generator().manual_seed(B + K)
     a = torch.randn(B, Ntok, K, generator=g).bfloat16().to(cuda)
