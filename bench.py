@@ -249,11 +249,11 @@ def kernel_rooflines(dev, iters=50, warmup=10):
     return rows, round(copy_gbs, 1)
 
 
-def images_per_s(dev, w8: bool, steps: int, warmup: int) -> float:
-    """1024px shape of Sana-1.6B: B=16, N=1024; DiT blocks of one denoising step only."""
+def images_per_s(dev, w8: bool, steps: int, warmup: int, B: int = 16) -> float:
+    """1024px shape of Sana-1.6B: B images of N=1024 tokens; DiT blocks of one denoising step only."""
     import sana_amd as S
 
-    B, HW = 16, (32, 32)
+    HW = (32, 32)
     blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
     blk.load_state_dict(make_state(0))
     blk = blk.to(dev)
@@ -349,6 +349,7 @@ def main():
         kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev)
         ips_bf16 = images_per_s(dev, False, 20, 5)
         ips_w8 = images_per_s(dev, True, 20, 5)
+        one_image_ms = 1e3 / images_per_s(dev, False, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
     del blocks
     torch.cuda.empty_cache()
 
@@ -366,8 +367,10 @@ def main():
         "config": {"workload": "cfg3: Sana-1.6B, 20 SanaMSBlocks chained = one denoising step, B=1, N=128x128=16384, "
                                "C=2240, 70x32 heads, Mix-FFN hidden 5600, 300 text tokens, random init"},
         "images_per_s_1024px": {"bf16": round(ips_bf16, 2), "w8a16": round(ips_w8, 2),
+                                "one_image_step_ms_bf16": round(one_image_ms, 3),
                                 "note": "B=16, N=1024: B / (20 x block latency); DiT blocks of one denoising step only "
-                                        "(no text encoder, VAE, embedders, step count or CFG doubling)"},
+                                        "(no text encoder, VAE, embedders, step count or CFG doubling); "
+                                        "one_image_step_ms: the same 20 blocks at B=1"},
         "roofline": roofline,
         "kernels": kernels,
         "copy_GBps_this_box": copy_gbs,
