@@ -327,3 +327,26 @@ def test_block_replays_from_a_hip_graph(cuda):
             torch.cuda.synchronize()
             assert torch.equal(out, eager), f"replay {r}"
         check(out, _ref64(ob, x.cpu(), y.cpu(), t.cpu(), HW=HW), "graph replay vs fp64 oracle", block=True)
+
+
+def test_four_images_at_the_full_shape_equal_one_at_a_time(cuda):
+    """B = 4 at the cfg3 shape (65536 tokens x 2240 channels, 4x the benchmark size: 1.5 GB hidden activation, row
+    offsets past 2^31 bytes): images do not interact, so the batched block must reproduce the per-image calls --
+    the GEMMs, depthwise conv and norms bit for bit per element, the attention up to the fp32 summation order of
+    its token splits (which depends on the grid)."""
+    C, heads, B, HW = 2240, 20, 4, (128, 128)
+    hb = S.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").bfloat16()
+    hb.load_state_dict(O.init_block_(O.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv"),
+                                     7).bfloat16().state_dict())
+    hb = hb.to(cuda)
+    x, y, t = (a.bfloat16().to(cuda) for a in O.block_inputs(B, HW[0] * HW[1], C, seed=7))
+    with torch.no_grad():
+        full = hb(x, y, t, HW=HW)
+        ffn = hb.mlp(x, HW=HW)
+        for b in range(B):
+            one = hb(x[b:b + 1], y[b:b + 1], t[b:b + 1], HW=HW)
+            assert rel_l2(full[b:b + 1], one) <= 2e-3
+            # a one-ulp flip of an attention output travels through two more GEMMs: a few bf16 ulps at the end
+            assert ((full[b:b + 1].float() - one.float()).abs() > 2 ** -5 * one.float().abs() + 4e-3).sum().item() == 0
+            assert torch.equal(ffn[b:b + 1], hb.mlp(x[b:b + 1], HW=HW))
+        assert torch.isfinite(full.float()).all()
