@@ -286,10 +286,14 @@ int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, int N, in
  *   W     bf16 [C][taps*C], row stride ldw: W[o][t*C + i] = t_conv.weight[o][i][t][0]
  *   out   bf16 [M][C], row stride ldo (must not overlap X)
  *   taps  odd; C % 64 == 0; x_rows * ldx * 2 < 2^31
+ *   zero_last_tap  NULL, or one byte per block of tap_rows output rows (per frame): non-zero = the last tap of
+ *         these rows reads zeros instead of the rows behind them.  That is the zero padding ChunkGLUMBConvTemp
+ *         puts behind every chunk (:302-349: a chunk sees the previous chunk's last frame in front and zeros
+ *         behind), so all chunks of a sequence run as one launch.  taps >= 3 when given.
  */
 int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,
-                            int64_t tap_rows, int64_t x_rows, int64_t ldx, int64_t ldw, int64_t ldo,
-                            void* stream);
+                            int64_t tap_rows, int64_t x_rows, const unsigned char* zero_last_tap,
+                            int64_t ldx, int64_t ldw, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

@@ -46,7 +46,7 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "sana_hip_dequant_w8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int64, c_void_p]),
     "sana_hip_tconv_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]),
+                                        c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "sana_hip_gemm_gate_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64,
                                             c_int, c_int64, c_void_p, c_size_t, c_void_p]),

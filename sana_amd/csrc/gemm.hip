@@ -91,6 +91,9 @@ struct Taps {
   // split-k launches (SPLIT, never together with taps): grid row z works on k-tiles
   // [z*split_tiles + min(z, split_rem), ...) -- split_tiles of them, one more for z < split_rem
   int split_tiles, split_rem;
+  // taps only, may be null: one byte per block of `stride` output rows; non-zero = the LAST tap reads zeros for
+  // these rows (a chunk boundary behind the block: the convolution's zero padding inside the buffer)
+  const unsigned char* zero_last;
 };
 
 // 8 outputs of one row: accumulator (+bias) -> io dtype, per the epilogue kind (everything except
@@ -480,6 +483,18 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int tap_b = TAPS ? (int)(tp.stride * lda * 2) : 0;
   auto a_koff = [&](int k0) { return TAPS ? (k0 / tp.kc) * tap_b + (k0 % tp.kc) * 2 : k0 * 2; };
   int a_kb = 0, a_kin = 0;  // offset of the k-tile being requested, and its column inside the tap
+  // rows of this thread (bit q: row g_row + 32*q) whose last tap is zero padding, and the same mask while the
+  // k-tile being requested belongs to the last tap (else 0)
+  uint32_t zlast = 0, a_zmask = 0;
+  int a_tap = 0;
+  const int last_tap = TAPS ? K / tp.kc - 1 : 0;
+  if (TAPS && tp.zero_last) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int r = m0 + (tid >> 3) + 32 * q;
+      if (r < M && tp.zero_last[r / tp.stride]) zlast |= 1u << q;
+    }
+  }
   const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * (W8 ? 1 : 2)), 0,
       (int)(((int64_t)w_last * ldw + K) * (W8 ? 1 : 2)), 0x00020000);
@@ -488,7 +503,9 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int step_a = 32 * (int)ulda * 2, step_w = W8 ? 64 * (int)uldw : 32 * (int)uldw * 2;
   auto gload = [&](int q, int k0) {
     if (q < 8) {
-      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff_a + (q * step_a + (TAPS ? a_kb : k0 * 2)), 0, 0);
+      int off = voff_a + (q * step_a + (TAPS ? a_kb : k0 * 2));
+      if (TAPS) off = ((a_zmask >> q) & 1u) ? (int)0x80000000u : off;  // outside the resource: reads zeros
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0);
       rs[q] = __builtin_bit_cast(u32x4_t, v);
     } else {
       const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w + ((q - 8) * step_w + k0 * (W8 ? 1 : 2)), 0, 0);
@@ -525,7 +542,10 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // prologue: k-tile 0 -> stage 0, k-tile 1 in flight
 #pragma unroll
   for (int q = 0; q < NQ; ++q) gload(q, 0);
-  if (TAPS) a_kb = a_koff(BK);
+  if (TAPS) {
+    a_kb = a_koff(BK);
+    a_zmask = BK / tp.kc == last_tap ? zlast : 0u;
+  }
 #pragma unroll
   for (int q = 0; q < (W8 ? 8 : NQ); ++q) lstore(q, 0);
   if (W8) {
@@ -537,6 +557,8 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   if (TAPS) {
     a_kb = a_koff(2 * BK);
     a_kin = (2 * BK) % tp.kc;
+    a_tap = (2 * BK) / tp.kc;
+    a_zmask = a_tap == last_tap ? zlast : 0u;
   }
   __syncthreads();
 #pragma unroll
@@ -591,6 +613,8 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       if (a_kin >= tp.kc) {
         a_kin -= tp.kc;
         a_kb += tap_b - tp.kc * 2;
+        ++a_tap;
+        a_zmask = a_tap == last_tap ? zlast : 0u;
       }
     }
   }
@@ -867,11 +891,11 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
             float* ws = nullptr, size_t ws_bytes = 0) {
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + 64 * NI - 1) / (64 * NI);
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
-  const Taps none = {0, 0, 0, 0, 0};
+  const Taps none = {0, 0, 0, 0, 0, nullptr};
   if (!taps && ws) {  // split-k when it pays and the caller's workspace holds the partial planes
     const GemmPlan pl = plan_gemm(M, N, K, W8);
     if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
-      const Taps split = {0, 0, 0, pl.tiles, pl.rem};
+      const Taps split = {0, 0, 0, pl.tiles, pl.rem, nullptr};
       hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, false, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
                          a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
                          split);
@@ -1040,9 +1064,10 @@ SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const flo
 }
 
 SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,
-                                     int64_t tap_rows, int64_t x_rows, int64_t ldx, int64_t ldw, int64_t ldo,
-                                     void* stream) {
+                                     int64_t tap_rows, int64_t x_rows, const unsigned char* zero_last_tap,
+                                     int64_t ldx, int64_t ldw, int64_t ldo, void* stream) {
   if (!X || !W || !out || M <= 0 || C <= 0 || taps <= 0 || !(taps & 1) || tap_rows <= 0) return SANA_ERR_ARG;
+  if (zero_last_tap && taps < 3) return SANA_ERR_ARG;
   if (C % 64) return SANA_ERR_SHAPE;  // a tap is a whole number of k-tiles
   if (x_rows < (taps / 2) * tap_rows + M) return SANA_ERR_ARG;  // the centre tap (= the residual) must exist for every row
   if (ldx < C || ldw < (int64_t)taps * C || ldo < C) return SANA_ERR_ARG;
@@ -1050,7 +1075,7 @@ SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, in
   if (x_rows * ldx * 2 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;  // 32-bit byte offsets inside the buffer
   const uint16_t* x = static_cast<const uint16_t*>(X);
   const EpiArgs e = {nullptr, nullptr, x + (taps / 2) * tap_rows * ldx, ldx, 0, M};
-  const Taps tp = {C, tap_rows, x_rows, 0, 0};
+  const Taps tp = {C, tap_rows, x_rows, 0, 0, zero_last_tap};
   return launch<false>(X, W, nullptr, e, out, M, C, taps * C, ldx, ldw, ldo, SANA_EPI_GATE_RES,
                        static_cast<hipStream_t>(stream), &tp);
 }

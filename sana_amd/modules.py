@@ -530,9 +530,11 @@ class GLUMBConvTemp(GLUMBConv):
             buf[:, :P].copy_(left)
         out = buf.new_empty(B, T * P, C)
         w2 = self._tconv_weight()
+        # one launch per batch entry for all chunks: the frame behind a chunk's last frame reads as zeros
+        # (the last frame of the sequence has nothing behind it in the buffer anyway)
+        ends = ops.frame_flags(T, [f1 - 1 for f1 in bounds[1:-1]], buf.device)
         for b in range(B):
-            for f0, f1 in zip(bounds[:-1], bounds[1:]):
-                ops.tconv_residual(buf[b, f0 * P:(f1 + 1) * P], w2, (f1 - f0) * P, P, out=out[b, f0 * P:f1 * P])
+            ops.tconv_residual(buf[b], w2, T * P, P, out=out[b], zero_last_tap=ends)
         return out
 
     def forward(self, x: torch.Tensor, HW=None, **kwargs) -> torch.Tensor:

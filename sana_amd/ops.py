@@ -401,15 +401,37 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     return out.view(B, Ntok, C)
 
 
+_frame_flags = {}    # (device index, n_frames, tuple of flagged frames) -> uint8 tensor
+
+
+def frame_flags(n_frames: int, flagged: Sequence[int], device) -> Optional[torch.Tensor]:
+    """uint8 [n_frames] with ones at ``flagged`` (cached per device), or None when nothing is flagged."""
+    flagged = tuple(sorted(set(int(f) for f in flagged)))
+    if not flagged:
+        return None
+    if flagged[0] < 0 or flagged[-1] >= n_frames:
+        raise SanaHipError(f"flagged frames {flagged} outside 0..{n_frames - 1}")
+    key = (torch.device(device).index, n_frames, flagged)
+    t = _frame_flags.get(key)
+    if t is None:
+        host = torch.zeros(n_frames, dtype=torch.uint8)
+        host[list(flagged)] = 1
+        t = host.to(device)
+        _frame_flags[key] = t
+    return t
+
+
 def tconv_residual(xp: torch.Tensor, weight: torch.Tensor, n_rows: int, tap_rows: int,
-                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   out: Optional[torch.Tensor] = None, zero_last_tap: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Temporal conv over frames plus its residual, as one GEMM over a virtual im2col.
 
     xp: [rows, C] bf16 (unit channel stride), the frame in front of the first output frame followed by the
     frames themselves (``rows >= n_rows + tap_rows``; rows past the end read as zero: the right padding);
     weight: [C, taps*C] bf16 with ``weight[o, t*C + i] = t_conv.weight[o, i, t, 0]``.  Returns
-    ``out[m] = xp[m + (taps//2)*tap_rows] + sum_t weight[:, t*C:(t+1)*C] @ xp[m + t*tap_rows]``, m < n_rows."""
-    _need_cuda(xp, weight, out)
+    ``out[m] = xp[m + (taps//2)*tap_rows] + sum_t weight[:, t*C:(t+1)*C] @ xp[m + t*tap_rows]``, m < n_rows.
+    ``zero_last_tap``: uint8 [ceil(n_rows / tap_rows)] from :func:`frame_flags`; a flagged frame's last tap reads
+    zeros (a chunk ends behind it), so all chunks of a sequence are one launch."""
+    _need_cuda(xp, weight, out, zero_last_tap)
     if xp.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise SanaHipError("tconv_residual is bf16 only")
     x2, ldx = _rows(xp, "xp")
@@ -425,8 +447,13 @@ def tconv_residual(xp: torch.Tensor, weight: torch.Tensor, n_rows: int, tap_rows
         raise SanaHipError("out has the wrong shape or dtype")
     if n_rows == 0:
         return out
+    if zero_last_tap is not None and (zero_last_tap.dtype != torch.uint8 or not zero_last_tap.is_contiguous()
+                                      or zero_last_tap.numel() < (n_rows + tap_rows - 1) // tap_rows):
+        raise SanaHipError("zero_last_tap must be a contiguous uint8 tensor with one entry per frame")
     code = _lib.load().sana_hip_tconv_residual(x2.data_ptr(), w2.data_ptr(), o2.data_ptr(), n_rows, C, taps,
-                                               tap_rows, rows, ldx, ldw, ldo, _stream())
+                                               tap_rows, rows,
+                                               zero_last_tap.data_ptr() if zero_last_tap is not None else None,
+                                               ldx, ldw, ldo, _stream())
     _lib.check(code, "sana_hip_tconv_residual")
     return out
 

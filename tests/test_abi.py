@@ -58,10 +58,11 @@ def test_argument_validation_needs_no_gpu():
     assert lib.sana_hip_gemm_bf16(16, 16, None, 16, 8, 8, 32, 32, 32, 8, 1, None, 0, None) == -1      # bias epilogue, no bias
     assert lib.sana_hip_gemm_w8a16(16, 16, None, None, 16, 8, 8, 32, 32, 32, 8, 0, None, 0, None) == -1  # no scale
     # temporal conv: C % 64, odd taps, the centre tap must exist for every output row
-    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 96, 3, 16, 80, 96, 288, 96, None) == -2
-    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 2, 16, 80, 64, 128, 64, None) == -1
-    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 64, 64, 192, 64, None) == -1
-    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 80, 64, 128, 64, None) == -1   # ldw < taps * C
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 96, 3, 16, 80, None, 96, 288, 96, None) == -2
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 2, 16, 80, None, 64, 128, 64, None) == -1
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 64, None, 64, 192, 64, None) == -1
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 3, 16, 80, None, 64, 128, 64, None) == -1   # ldw < taps * C
+    assert lib.sana_hip_tconv_residual(16, 16, 32, 64, 64, 1, 16, 80, 16, 64, 64, 64, None) == -1   # chunk flags need >= 3 taps
 
 
 def test_workspace_query():

@@ -304,6 +304,26 @@ def test_temporal_conv_residual_matches_conv2d(cuda, C, T, P, B):
         assert (out_c.cpu().double() - ref_c).abs().max().item() <= 2e-2 and rel_l2(out_c.cpu(), ref_c) <= 3e-3
 
 
+@pytest.mark.parametrize("C,T,P,ends", [(128, 7, 37, [0, 3, 4]), (64, 5, 300, [1]), (2240, 6, 260, [2, 4])])
+def test_temporal_conv_chunk_flags_equal_per_chunk_launches(cuda, C, T, P, ends):
+    """All chunks in one launch (`zero_last_tap` flags on each chunk's last frame) against one launch per chunk,
+    whose buffer simply ends behind the chunk: the same products in the same order, so the same bits; and the flags
+    must matter (the unflagged launch differs on exactly the flagged frames)."""
+    g = torch.Generator().manual_seed(C + T)
+    y = torch.randn(T * P, C, generator=g).bfloat16().to(cuda)
+    w2 = (torch.randn(C, 3 * C, generator=g) * (1.0 / (3 * C)) ** 0.5).bfloat16().to(cuda)
+    buf = torch.cat([torch.randn(P, C, generator=g).bfloat16().to(cuda), y])     # a real frame in front (a cache tail)
+    flags = ops.frame_flags(T, ends, cuda)
+    one = ops.tconv_residual(buf, w2, T * P, P, zero_last_tap=flags)
+    bounds = [0] + [e + 1 for e in sorted(ends)] + ([T] if sorted(ends)[-1] + 1 < T else [])
+    parts = [ops.tconv_residual(buf[f0 * P:(f1 + 1) * P], w2, (f1 - f0) * P, P) for f0, f1 in zip(bounds[:-1], bounds[1:])]
+    assert torch.equal(one, torch.cat(parts))
+    plain = ops.tconv_residual(buf, w2, T * P, P)
+    differs = (plain != one).view(T, P * C).any(1).cpu().tolist()
+    assert differs == [f in ends and f != T - 1 for f in range(T)]
+    assert ops.frame_flags(T, [], cuda) is None
+
+
 def test_temporal_conv_zero_weight_is_identity(cuda):
     """t_conv is zero-initialised in the reference: x + 0 must come back bit for bit."""
     C, T, P = 128, 3, 50
