@@ -16,8 +16,21 @@ _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 HEAD_DIM = 32
 HEAD_DIMS = (32, 112)   # head dims with kernels: 32 (all dtypes), 112 (bf16; the video configurations)
 
-_workspaces = {}     # (device index) -> uint8 tensor, grown on demand
+# One scratch buffer per device, grown on demand and shared by every call on that device (attention partial
+# states, split-k planes): calls are ordered by the stream they run on, so launching from two streams at once
+# on one device needs one process (or one copy of this module) per stream.
+_workspaces = {}     # (device index) -> uint8 tensor
 _chunk_tables = {}   # (device index, tuple) -> int32 tensor
+_CACHE_LIMIT = 256   # small derived device tensors (chunk tables, frame flags) kept per process
+
+
+def _remember(cache: dict, key, make):
+    t = cache.get(key)
+    if t is None:
+        t = make()
+        if len(cache) < _CACHE_LIMIT:   # ever-changing chunkings must not grow the cache without bound; entries
+            cache[key] = t              # are never dropped (a captured graph may hold their addresses)
+    return t
 
 
 def _stream() -> int:
@@ -57,10 +70,7 @@ def chunk_table(chunk_tokens: Optional[Sequence[int]], N: int, device) -> Tuple[
     if starts[0] != 0 or any(b <= a for a, b in zip(starts[:-1], starts[1:])):
         raise SanaHipError(f"chunk starts must begin at 0 and increase strictly below N={N}: {chunk_tokens}")
     key = (torch.device(device).index, tuple(starts))
-    tab = _chunk_tables.get(key)
-    if tab is None:
-        tab = torch.tensor(starts, dtype=torch.int32, device=device)
-        _chunk_tables[key] = tab
+    tab = _remember(_chunk_tables, key, lambda: torch.tensor(starts, dtype=torch.int32, device=device))
     return tab, len(starts) - 1, max(b - a for a, b in zip(starts[:-1], starts[1:]))
 
 
@@ -411,14 +421,12 @@ def frame_flags(n_frames: int, flagged: Sequence[int], device) -> Optional[torch
         return None
     if flagged[0] < 0 or flagged[-1] >= n_frames:
         raise SanaHipError(f"flagged frames {flagged} outside 0..{n_frames - 1}")
-    key = (torch.device(device).index, n_frames, flagged)
-    t = _frame_flags.get(key)
-    if t is None:
+    def make():
         host = torch.zeros(n_frames, dtype=torch.uint8)
         host[list(flagged)] = 1
-        t = host.to(device)
-        _frame_flags[key] = t
-    return t
+        return host.to(device)
+
+    return _remember(_frame_flags, (torch.device(device).index, n_frames, flagged), make)
 
 
 def tconv_residual(xp: torch.Tensor, weight: torch.Tensor, n_rows: int, tap_rows: int,
