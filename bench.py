@@ -163,6 +163,17 @@ def kernel_rooflines(dev, iters=50, warmup=10):
     add("linattn_apply_chunk_causal_cfg5", "hbm", la5,
         event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st5, 1e-8, starts, out=out5), iters, warmup),
         "cfg5: Q read + out write + 21 states")
+    # the reference's own chunking of that shape: two chunks, frames [0, 11) and [11, 21)
+    starts2 = [0, 11 * hw]
+    st5b = ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts2, causal=True)
+    la5b = 2 * Nv * C * 2 + 2 * (C // 32) * 33 * 32 * 4
+    add("linattn_state_chunk_causal_cfg5_chunks_0_11", "hbm", la5b,
+        event_time_us(lambda: ops.linattn_state(qkv5[:, :, 1], qkv5[:, :, 2], starts2, causal=True), iters, warmup),
+        "cfg5: N=32760, chunk_index [0, 11]; K,V read + 2 states")
+    add("linattn_apply_chunk_causal_cfg5_chunks_0_11", "hbm", la5b,
+        event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st5b, 1e-8, starts2, out=out5), iters, warmup),
+        "cfg5: chunk_index [0, 11]; Q read + out write + 2 states")
+    del st5b
     # the same video shape with 112-wide heads (linear_head_dim = 112: 20 heads at C = 2240), q/k RMSNorm and rotary
     # embedding on load as the video blocks use them; whole sequence as one chunk, and 21 causal chunks
     D2 = 112
