@@ -279,7 +279,7 @@ def images_per_s(dev, w8: bool, steps: int, warmup: int, B: int = 16) -> float:
     return B / (DEPTH * t_us * 1e-6)
 
 
-def cpu_baseline(iters: int = 2):
+def cpu_baseline(iters: int = 5):
     """The oracle (stock PyTorch restatement of the reference block) on the host
     cores: one block of the cfg3 workload in fp32 (bf16 GEMM/conv on CPU is not a
     fair or stable baseline), same seeded weights and inputs."""
