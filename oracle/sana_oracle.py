@@ -704,6 +704,116 @@ class SanaMSBlock(nn.Module):
         return x
 
 
+class ChunkedLiteLAReLURope(LiteLAReLURope):
+    """diffusion/model/nets/sana_blocks.py:1790-1802 onwards: LiteLAReLURope evaluated in token chunks of
+    ``chunk_size`` to bound memory; the same function of its inputs (restated as the unchunked call)."""
+
+    def __init__(self, *args, chunk_size=200_000, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.chunk_size = chunk_size
+
+
+class SanaVideoMSBlock(nn.Module):
+    """diffusion/model/nets/sana_multi_scale_video.py:66-333: the video DiT block, the caller of the chunk-causal /
+    cached attention and of the temporal Mix-FFN variants.  Restated for the linear-attention ``attn_type`` values
+    and the GLUMBConv family of ``ffn_type`` values, without the optional extra flash attention, image-embedding
+    cross-attention and drop-path (all off in the released SANA-Video configurations)."""
+
+    ATTN = {"chunkcausal": "ChunkCausalAttention", "cachedcausal": "CachedCausalAttention", "linear": "LiteLA",
+            "LiteLAReLURope": "LiteLAReLURope", "ChunkedLiteLAReLURope": "ChunkedLiteLAReLURope"}
+    FFN = ("glumbconv", "GLUMBConvTemp", "ChunkGLUMBConvTemp", "CachedGLUMBConvTemp")
+
+    def __init__(self, hidden_size, num_heads, mlp_ratio=4.0, drop_path=0.0, qk_norm=False, attn_type="flash",
+                 ffn_type="mlp", mlp_acts=("silu", "silu", None), linear_head_dim=32, cross_norm=False,
+                 cross_attn_image_embeds=False, t_kernel_size=3, additional_flash_attn=False,
+                 flash_attn_window_count=None, **block_kwargs):
+        super().__init__()
+        if attn_type not in self.ATTN or ffn_type not in self.FFN or additional_flash_attn or \
+                cross_attn_image_embeds or drop_path > 0.0:
+            raise NotImplementedError("oracle restates the linear-attention / GLUMBConv-family video block only")
+        self.hidden_size = hidden_size
+        self.norm1 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        attn_cls = globals()[self.ATTN[attn_type]]
+        self.attn = attn_cls(hidden_size, hidden_size, heads=hidden_size // linear_head_dim, eps=1e-8,
+                             qk_norm=qk_norm)                                                    # :101-119
+        self.flash_attn_additional = None
+        self.cross_attn_image_embeds = cross_attn_image_embeds
+        self.cross_attn = MultiHeadCrossAttention(hidden_size, num_heads, qk_norm=cross_norm)
+        self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        ffn_kw = dict(in_features=hidden_size, hidden_features=int(hidden_size * mlp_ratio),
+                      use_bias=(True, True, False), norm=(None, None, None), act=mlp_acts)
+        if ffn_type == "glumbconv":                                                              # :156-191
+            self.mlp = GLUMBConv(**ffn_kw)
+        else:
+            self.mlp = globals()[ffn_type](t_kernel_size=t_kernel_size, **ffn_kw)
+        self.drop_path = nn.Identity()
+        self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
+        self.block_hook = None
+
+    def forward_frame_aware(self, x, y, t, mask=None, THW=None, rotary_emb=None, chunk_index=None, **kwargs):
+        """:204-254: one modulation row per frame, t = [B, 1, F, 6C]."""
+        B, N, C = x.shape
+        num_frames = t.shape[2]
+        t = t.reshape(B, num_frames, 6, -1)
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+            self.scale_shift_table[None, None, :, :] + t).chunk(6, dim=-2)            # each B, F, 1, C
+        attn_kw = {"HW": THW, "rotary_emb": rotary_emb}
+        if chunk_index is not None:
+            attn_kw["chunk_index"] = chunk_index[:]
+        h = t2i_modulate(self.norm1(x).reshape(B, num_frames, -1, C), shift_msa, scale_msa).reshape(B, N, C)
+        x = x + (gate_msa * self.attn(h, **attn_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+        x = x + self.cross_attn(x, y, mask=mask)
+        mlp_kw = {"HW": THW}
+        if chunk_index is not None:
+            mlp_kw["chunk_index"] = chunk_index[:]
+        h = t2i_modulate(self.norm2(x).reshape(B, num_frames, -1, C), shift_mlp, scale_mlp).reshape(B, N, C)
+        x = x + (gate_mlp * self.mlp(h, **mlp_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+        return x
+
+    def forward(self, x, y, t, mask=None, THW=None, rotary_emb=None, chunk_index=None, **kwargs):
+        """:256-333."""
+        if len(t.shape) > 2:
+            return self.forward_frame_aware(x, y, t, mask=mask, THW=THW, rotary_emb=rotary_emb,
+                                            chunk_index=chunk_index, **kwargs)
+        B, N, C = x.shape
+        feats = {"x_in": x, "x_self_attn": None, "x_cross_attn": None, "x_ffn": None}
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+            self.scale_shift_table[None] + t.reshape(B, 6, -1)).chunk(6, dim=1)
+        attn_kw = {"HW": THW, "rotary_emb": rotary_emb}
+        if chunk_index is not None:
+            attn_kw["chunk_index"] = chunk_index[:]
+        save_kv_cache = kwargs.get("save_kv_cache", None)
+        if save_kv_cache is not None:
+            attn_kw["save_kv_cache"] = save_kv_cache
+        kv_cache = kwargs.get("kv_cache", None)
+        if kv_cache is not None:
+            attn_kw["kv_cache"] = kv_cache
+        x_sa = self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), **attn_kw)
+        if kv_cache is not None:
+            x_sa, kv_cache = x_sa
+        feats["x_self_attn"] = x_sa
+        x = x + gate_msa * x_sa
+        x = x + self.cross_attn(x, y, mask=mask)
+        feats["x_cross_attn"] = x
+        mlp_kw = {"HW": THW}
+        if chunk_index is not None:
+            mlp_kw["chunk_index"] = chunk_index[:]
+        if save_kv_cache is not None:
+            mlp_kw["save_kv_cache"] = save_kv_cache
+        if kv_cache is not None:
+            mlp_kw["kv_cache"] = kv_cache
+        mlp_out = self.mlp(t2i_modulate(self.norm2(x), shift_mlp, scale_mlp), **mlp_kw)
+        if kv_cache is not None:
+            mlp_out, kv_cache = mlp_out
+        x = x + gate_mlp * mlp_out
+        feats["x_ffn"] = x
+        if self.block_hook is not None:
+            self.block_hook(**feats)
+        if kv_cache is not None:
+            return x, kv_cache
+        return x
+
+
 # --------------------------------------------------------------------------
 # A8: W8A16 quantiser (defined by the benchmark configuration, not by the
 # reference, which has no W8A16 code)

@@ -794,3 +794,132 @@ class SanaMSBlock(nn.Module):
         self.attn.quantize_w8_()
         self.mlp.quantize_w8_()
         return self
+
+
+class ChunkedLiteLAReLURope(LiteLAReLURope):
+    """The reference's memory-bounded evaluation of LiteLAReLURope in token chunks (sana_blocks.py:1790-1802):
+    the same function; the kernels here stream any N, so ``chunk_size`` is kept as an attribute only."""
+
+    def __init__(self, *args, chunk_size=200_000, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.chunk_size = chunk_size
+
+
+class SanaVideoMSBlock(nn.Module):
+    """The video DiT block (reference: sana_multi_scale_video.py:66-333), the caller of the chunk-causal / cached
+    attention and of the temporal Mix-FFN variants: same constructor, ``forward(x, y, t, mask, THW, rotary_emb,
+    chunk_index, save_kv_cache=, kv_cache=)``, per-frame conditioning (``t`` [B, 1, F, 6C], :204-254), ``block_hook``
+    and ``state_dict`` keys.  LayerNorm + modulation run as the fused kernel (one modulation row per batch entry or
+    per frame); attention and Mix-FFN are the HIP modules; cross-attention, gates and residual sums are stock ops."""
+
+    ATTN = {"chunkcausal": ChunkCausalAttention, "cachedcausal": CachedCausalAttention, "linear": LiteLA,
+            "LiteLAReLURope": LiteLAReLURope, "ChunkedLiteLAReLURope": ChunkedLiteLAReLURope}
+    FFN = {"glumbconv": GLUMBConv, "GLUMBConvTemp": GLUMBConvTemp, "ChunkGLUMBConvTemp": ChunkGLUMBConvTemp,
+           "CachedGLUMBConvTemp": CachedGLUMBConvTemp}
+
+    def __init__(self, hidden_size, num_heads, mlp_ratio=4.0, drop_path=0.0, qk_norm=False, attn_type="flash",
+                 ffn_type="mlp", mlp_acts=("silu", "silu", None), linear_head_dim=32, cross_norm=False,
+                 cross_attn_image_embeds=False, t_kernel_size=3, additional_flash_attn=False,
+                 flash_attn_window_count=None, **block_kwargs):
+        super().__init__()
+        if attn_type not in self.ATTN or ffn_type not in self.FFN:
+            raise NotImplementedError(f"this block is the linear-attention / GLUMBConv hot path only: attn_type in "
+                                      f"{sorted(self.ATTN)}, ffn_type in {sorted(self.FFN)}")
+        if additional_flash_attn or cross_attn_image_embeds:
+            raise NotImplementedError("additional_flash_attn / cross_attn_image_embeds are outside this path")
+        if drop_path > 0.0:
+            raise NotImplementedError("drop_path > 0 is a training-time option; this block is forward-only")
+        self.hidden_size = hidden_size
+        self.norm1 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        self.attn = self.ATTN[attn_type](hidden_size, hidden_size, heads=hidden_size // linear_head_dim, eps=1e-8,
+                                         qk_norm=qk_norm)
+        self.flash_attn_additional = None
+        self.cross_attn_image_embeds = cross_attn_image_embeds
+        self.cross_attn = MultiHeadCrossAttention(hidden_size, num_heads, qk_norm=cross_norm, **block_kwargs)
+        self.norm2 = nn.LayerNorm(hidden_size, elementwise_affine=False, eps=1e-6)
+        ffn_kw = dict(in_features=hidden_size, hidden_features=int(hidden_size * mlp_ratio),
+                      use_bias=(True, True, False), norm=(None, None, None), act=mlp_acts)
+        if ffn_type != "glumbconv":
+            ffn_kw["t_kernel_size"] = t_kernel_size
+        self.mlp = self.FFN[ffn_type](**ffn_kw)
+        self.drop_path = nn.Identity()
+        self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
+        self.block_hook = None
+
+    def _norm_modulate(self, norm, x, shift, scale, groups: int):
+        """t2i_modulate(norm(x), shift, scale) with ``groups`` modulation rows per batch entry (1, or one per
+        frame): shift / scale are [B, groups, 1, C] or [B, 1, C]."""
+        B, N, C = x.shape
+        if x.is_cuda and x.dtype == torch.bfloat16 and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
+            h = ops.layernorm_modulate(x.reshape(B * groups, N // groups, C), scale.reshape(B * groups, 1, C),
+                                       shift.reshape(B * groups, 1, C), norm.eps)
+            return h.view(B, N, C)
+        if groups == 1:
+            return t2i_modulate(norm(x), shift, scale)
+        return t2i_modulate(norm(x).reshape(B, groups, -1, C), shift, scale).reshape(B, N, C)
+
+    def forward_frame_aware(self, x, y, t, mask=None, THW=None, rotary_emb=None, chunk_index=None, **kwargs):
+        B, N, C = x.shape
+        num_frames = t.shape[2]
+        t = t.reshape(B, num_frames, 6, -1)
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+            self.scale_shift_table[None, None, :, :] + t).chunk(6, dim=-2)            # each [B, F, 1, C]
+        attn_kw = {"HW": THW, "rotary_emb": rotary_emb}
+        if chunk_index is not None:
+            attn_kw["chunk_index"] = chunk_index[:]
+        h = self._norm_modulate(self.norm1, x, shift_msa, scale_msa, num_frames)
+        x = x + (gate_msa * self.attn(h, **attn_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+        x = x + self.cross_attn(x, y, mask=mask)
+        mlp_kw = {"HW": THW}
+        if chunk_index is not None:
+            mlp_kw["chunk_index"] = chunk_index[:]
+        h = self._norm_modulate(self.norm2, x, shift_mlp, scale_mlp, num_frames)
+        x = x + (gate_mlp * self.mlp(h, **mlp_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+        return x
+
+    def forward(self, x, y, t, mask=None, THW=None, rotary_emb=None, chunk_index=None, **kwargs):
+        if len(t.shape) > 2:
+            return self.forward_frame_aware(x, y, t, mask=mask, THW=THW, rotary_emb=rotary_emb,
+                                            chunk_index=chunk_index, **kwargs)
+        B, N, C = x.shape
+        feats = {"x_in": x, "x_self_attn": None, "x_cross_attn": None, "x_ffn": None}
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+            self.scale_shift_table[None] + t.reshape(B, 6, -1)).chunk(6, dim=1)
+        attn_kw = {"HW": THW, "rotary_emb": rotary_emb}
+        if chunk_index is not None:
+            attn_kw["chunk_index"] = chunk_index[:]      # the callee may edit its list
+        save_kv_cache = kwargs.get("save_kv_cache", None)
+        if save_kv_cache is not None:
+            attn_kw["save_kv_cache"] = save_kv_cache
+        kv_cache = kwargs.get("kv_cache", None)
+        if kv_cache is not None:
+            attn_kw["kv_cache"] = kv_cache
+        x_sa = self.attn(self._norm_modulate(self.norm1, x, shift_msa, scale_msa, 1), **attn_kw)
+        if kv_cache is not None:
+            x_sa, kv_cache = x_sa
+        feats["x_self_attn"] = x_sa
+        x = x + gate_msa * x_sa
+        x = x + self.cross_attn(x, y, mask=mask)
+        feats["x_cross_attn"] = x
+        mlp_kw = {"HW": THW}
+        if chunk_index is not None:
+            mlp_kw["chunk_index"] = chunk_index[:]
+        if save_kv_cache is not None:
+            mlp_kw["save_kv_cache"] = save_kv_cache
+        if kv_cache is not None:
+            mlp_kw["kv_cache"] = kv_cache
+        mlp_out = self.mlp(self._norm_modulate(self.norm2, x, shift_mlp, scale_mlp, 1), **mlp_kw)
+        if kv_cache is not None:
+            mlp_out, kv_cache = mlp_out
+        x = x + gate_mlp * mlp_out
+        feats["x_ffn"] = x
+        if self.block_hook is not None:
+            self.block_hook(**feats)
+        if kv_cache is not None:
+            return x, kv_cache
+        return x
+
+    def quantize_w8_(self) -> "SanaVideoMSBlock":
+        self.attn.quantize_w8_()
+        self.mlp.quantize_w8_()
+        return self

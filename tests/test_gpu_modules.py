@@ -350,3 +350,81 @@ def test_four_images_at_the_full_shape_equal_one_at_a_time(cuda):
             assert ((full[b:b + 1].float() - one.float()).abs() > 2 ** -5 * one.float().abs() + 4e-3).sum().item() == 0
             assert torch.equal(ffn[b:b + 1], hb.mlp(x[b:b + 1], HW=HW))
         assert torch.isfinite(full.float()).all()
+
+
+def _video_blocks(C, heads, attn_type, ffn_type, seed, **kw):
+    ob = O.SanaVideoMSBlock(C, heads, mlp_ratio=2.5, attn_type=attn_type, ffn_type=ffn_type, **kw)
+    O.init_block_(ob, seed)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(seed + 1)
+        for n, p in ob.named_parameters():
+            if n.endswith("bias"):
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+            elif n.endswith("t_conv.weight"):
+                p.copy_(torch.randn(p.shape, generator=g) * (0.3 / p.shape[1]) ** 0.5)
+    ob = ob.bfloat16()
+    hb = S.SanaVideoMSBlock(C, heads, mlp_ratio=2.5, attn_type=attn_type, ffn_type=ffn_type, **kw).bfloat16()
+    hb.load_state_dict(ob.state_dict(), strict=True)
+    return ob, hb
+
+
+def _freqs(N, d, seed):
+    theta = torch.rand(N, d // 2, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * 6.283
+    return torch.polar(torch.ones_like(theta), theta)[None, None]
+
+
+@pytest.mark.parametrize("attn_type,ffn_type,d,C", [("chunkcausal", "ChunkGLUMBConvTemp", 32, 128),
+                                                    ("LiteLAReLURope", "GLUMBConvTemp", 112, 224),
+                                                    ("ChunkedLiteLAReLURope", "glumbconv", 32, 96)])
+def test_video_block_matches_oracle(cuda, attn_type, ffn_type, d, C):
+    """SanaVideoMSBlock (sana_multi_scale_video.py:66-333) against the fp64 oracle: flat conditioning, one
+    modulation row per frame, text mask, block_hook."""
+    B, (T, H, W) = 2, (4, 5, 6)
+    N = T * H * W
+    ob, hb = _video_blocks(C, 4, attn_type, ffn_type, seed=d, qk_norm=True, linear_head_dim=d)
+    hb = hb.to(cuda)
+    x, y, t = (a.bfloat16() for a in O.block_inputs(B, N, C, n_text=40, seed=d))
+    freqs = _freqs(N, d, 3)
+    kw = {"chunk_index": [0, 1, 3]} if attn_type == "chunkcausal" else {}
+    with torch.no_grad():
+        ref = _ref64(ob, x, y, t, THW=(T, H, W), rotary_emb=freqs, **kw)
+        seen = {}
+        hb.block_hook = lambda **feats: seen.update(feats)
+        out = hb(x.to(cuda), y.to(cuda), t.to(cuda), THW=(T, H, W), rotary_emb=freqs.to(cuda), **kw)
+        check(out, ref, f"{attn_type}/{ffn_type}", block=True)
+        assert set(seen) == {"x_in", "x_self_attn", "x_cross_attn", "x_ffn"} and torch.equal(seen["x_ffn"], out)
+        hb.block_hook = None
+        tf = (torch.randn(B, 1, T, 6 * C, generator=torch.Generator().manual_seed(8)) * 0.3).bfloat16()
+        mask = torch.ones(B, 40, dtype=torch.long)
+        mask[:, 25:] = 0
+        ref = _ref64(ob, x, y, tf, mask=mask, THW=(T, H, W), rotary_emb=freqs, **kw)
+        out = hb(x.to(cuda), y.to(cuda), tf.to(cuda), mask=mask.to(cuda), THW=(T, H, W), rotary_emb=freqs.to(cuda), **kw)
+        check(out, ref, f"{attn_type}/{ffn_type}, per-frame conditioning", block=True)
+
+
+def test_video_block_streaming_cache_equals_chunked_block(cuda):
+    """cachedcausal + CachedGLUMBConvTemp fed chunk by chunk with the accumulated cache against chunkcausal +
+    ChunkGLUMBConvTemp on the whole sequence (both on the HIP path), and the whole against the fp64 oracle."""
+    C, d, B, (T, H, W) = 128, 32, 1, (5, 4, 6)
+    P = H * W
+    ob, hb = _video_blocks(C, 4, "chunkcausal", "ChunkGLUMBConvTemp", seed=11, linear_head_dim=d)
+    hc = S.SanaVideoMSBlock(C, 4, mlp_ratio=2.5, attn_type="cachedcausal", ffn_type="CachedGLUMBConvTemp",
+                            linear_head_dim=d).bfloat16()
+    hc.load_state_dict(hb.state_dict(), strict=True)
+    hb, hc = hb.to(cuda), hc.to(cuda)
+    x, y, t = (a.bfloat16() for a in O.block_inputs(B, T * P, C, n_text=20, seed=11))
+    freqs = _freqs(T * P, d, 4)
+    with torch.no_grad():
+        whole = hb(x.to(cuda), y.to(cuda), t.to(cuda), THW=(T, H, W), rotary_emb=freqs.to(cuda), chunk_index=[0, 2, 3])
+        check(whole, _ref64(ob, x, y, t, THW=(T, H, W), rotary_emb=freqs, chunk_index=[0, 2, 3]), "chunked video block",
+              block=True)
+        acc, outs = None, []
+        for a, b in ((0, 2), (2, 3), (3, 5)):
+            cache = [None, None, None] if acc is None else list(acc)
+            o, saved = hc(x[:, a * P:b * P].to(cuda), y.to(cuda), t.to(cuda), THW=(b - a, H, W),
+                          rotary_emb=freqs[:, :, a * P:b * P].to(cuda), save_kv_cache=True, kv_cache=cache)
+            outs.append(o)
+            acc = S.accumulate_kv_cache(acc, saved)
+        stream = torch.cat(outs, 1)
+        assert rel_l2(stream, whole) <= 3e-3
+        assert ((stream.float() - whole.float()).abs() > 2 ** -5 * whole.float().abs() + 4e-3).sum().item() == 0

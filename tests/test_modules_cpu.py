@@ -12,7 +12,8 @@ from oracle import sana_oracle as O
 
 @pytest.mark.parametrize("name", ["LiteLA", "GLUMBConv", "SanaMSBlock", "ChunkCausalAttention", "LiteLAReLURope",
                                   "CachedCausalAttention", "GLUMBConvTemp", "ChunkGLUMBConvTemp",
-                                  "CachedGLUMBConvTemp", "GLUMBConvLinear", "GLUMBConvLinearTemp"])
+                                  "CachedGLUMBConvTemp", "GLUMBConvLinear", "GLUMBConvLinearTemp", "SanaVideoMSBlock",
+                                  "ChunkedLiteLAReLURope"])
 def test_constructor_and_forward_signatures_match(name):
     a, b = getattr(S, name), getattr(O, name)
     pa = list(inspect.signature(a.__init__).parameters)
@@ -70,6 +71,22 @@ def test_glumbconv_linear_keys_and_checkpoint_conversion():
     assert "inverted_conv.linear.weight_q" in q.state_dict() and "point_conv.linear.weight" not in q.state_dict()
     t = S.GLUMBConvLinearTemp(64, 160, use_bias=(True, True, False))
     assert isinstance(t.point_conv, S.modules.LinearLayer) and t.t_conv.weight.abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("attn_type,ffn_type", [("chunkcausal", "ChunkGLUMBConvTemp"), ("cachedcausal", "CachedGLUMBConvTemp"),
+                                                ("LiteLAReLURope", "GLUMBConvTemp"), ("ChunkedLiteLAReLURope", "glumbconv"),
+                                                ("linear", "glumbconv")])
+def test_video_block_keys(attn_type, ffn_type):
+    kw = dict(mlp_ratio=2.5, attn_type=attn_type, ffn_type=ffn_type, qk_norm=True, cross_norm=True, linear_head_dim=32)
+    ob, hb = O.SanaVideoMSBlock(64, 4, **kw), S.SanaVideoMSBlock(64, 4, **kw)
+    assert list(ob.state_dict()) == list(hb.state_dict())
+    hb.load_state_dict(ob.state_dict(), strict=True)
+    assert type(hb.attn).__name__ == type(ob.attn).__name__ and type(hb.mlp).__name__ == type(ob.mlp).__name__
+    assert hb.block_hook is None and hb.flash_attn_additional is None and hb.cross_attn_image_embeds is False
+    for bad in (dict(attn_type="flash"), dict(ffn_type="mlp"), dict(additional_flash_attn="flash"),
+                dict(cross_attn_image_embeds=True)):
+        with pytest.raises(NotImplementedError):
+            S.SanaVideoMSBlock(64, 4, **{**kw, **bad})
 
 
 def test_unsupported_options_fail_loudly():

@@ -184,3 +184,74 @@ def test_dequantized_block_state_touches_only_the_four_gemm_weights():
             assert ((sd[key].float() - dq[key].float()).abs().max() <= sd[key].float().abs().max() / 127 * 0.51 + 1e-3)
         else:
             assert torch.equal(sd[key], dq[key])
+
+
+# ---- SanaVideoMSBlock (sana_multi_scale_video.py:66-333): pinned by reductions to what is already pinned
+
+
+def _video_pair(attn_type, ffn_type, seed=0, **kw):
+    blk = O.SanaVideoMSBlock(64, 4, mlp_ratio=2.5, attn_type=attn_type, ffn_type=ffn_type, **kw).double()
+    O.init_block_(blk, seed)
+    with torch.no_grad():
+        for n, p in blk.named_parameters():
+            if n.endswith("bias") or n.endswith("t_conv.weight"):
+                p.copy_(torch.randn(p.shape, generator=torch.Generator().manual_seed(seed + 7), dtype=torch.float64) * 0.05)
+    return blk
+
+
+def test_video_block_with_image_options_is_the_image_block():
+    """attn_type="linear", ffn_type="glumbconv", flat t: the video block's forward is SanaMSBlock's (same wiring,
+    same keys), so the two restatements must agree exactly on the same weights."""
+    vb = _video_pair("linear", "glumbconv")
+    ib = O.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").double()
+    assert list(ib.state_dict()) == list(vb.state_dict())
+    ib.load_state_dict(vb.state_dict(), strict=True)
+    x, y, t = (a.double() for a in O.block_inputs(2, 6 * 5, 64, n_text=9, seed=1))
+    torch.testing.assert_close(vb(x, y, t, THW=(6, 5)), ib(x, y, t, HW=(6, 5)), rtol=0, atol=0)
+
+
+def test_video_block_frame_aware_conditioning():
+    """One modulation row per frame ([B, 1, F, 6C]): equal rows reduce to the flat-t forward; different rows act on
+    their own frames only through the modulation (zero gates for one frame leave that frame's residual stream with
+    the cross-attention update alone)."""
+    vb = _video_pair("chunkcausal", "ChunkGLUMBConvTemp", seed=2, qk_norm=True)
+    B, (T, H, W), C = 2, (4, 3, 5), 64
+    x, y, t = (a.double() for a in O.block_inputs(B, T * H * W, C, n_text=9, seed=2))
+    flat = vb(x, y, t, THW=(T, H, W), chunk_index=[0, 2])
+    tf = t.view(B, 1, 1, 6 * C).expand(B, 1, T, 6 * C).contiguous()
+    torch.testing.assert_close(vb(x, y, tf, THW=(T, H, W), chunk_index=[0, 2]), flat, rtol=1e-12, atol=1e-12)
+    # frame 1 gets gates that cancel the table's: its tokens then only receive x + cross_attn(x, y)
+    tf2 = tf.clone().view(B, 1, T, 6, C)
+    tf2[:, :, 1, 2] = -vb.scale_shift_table[2]
+    tf2[:, :, 1, 5] = -vb.scale_shift_table[5]
+    out = vb(x, y, tf2.view(B, 1, T, 6 * C), THW=(T, H, W), chunk_index=[0, 2])
+    P = H * W
+    want = (x + vb.cross_attn(x, y))[:, P:2 * P]
+    torch.testing.assert_close(out[:, P:2 * P], want, rtol=1e-12, atol=1e-12)
+    assert (out[:, :P] - (x + vb.cross_attn(x, y))[:, :P]).abs().max() > 1e-3
+
+
+def test_video_block_streaming_cache_equals_the_chunked_block():
+    """cachedcausal + CachedGLUMBConvTemp fed chunk by chunk with the accumulated cache (the pipeline's bookkeeping,
+    sana_inference_pipeline.py:242-263) reproduces chunkcausal + ChunkGLUMBConvTemp on the whole sequence, given
+    rotary factors that depend on the absolute token position."""
+    chunked = _video_pair("chunkcausal", "ChunkGLUMBConvTemp", seed=3)
+    cached = O.SanaVideoMSBlock(64, 4, mlp_ratio=2.5, attn_type="cachedcausal", ffn_type="CachedGLUMBConvTemp").double()
+    cached.load_state_dict(chunked.state_dict(), strict=True)
+    B, (T, H, W), C = 1, (5, 2, 3), 64
+    P = H * W
+    x, y, t = (a.double() for a in O.block_inputs(B, T * P, C, n_text=9, seed=3))
+    theta = torch.rand(T * P, 16, generator=torch.Generator().manual_seed(5), dtype=torch.float64) * 6.283
+    freqs = torch.polar(torch.ones_like(theta), theta)[None, None]
+    whole = chunked(x, y, t, THW=(T, H, W), rotary_emb=freqs, chunk_index=[0, 2, 3])
+    acc, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 5)):
+        cache = [None, None, None] if acc is None else [acc[0], acc[1], acc[2]]
+        o, saved = cached(x[:, a * P:b * P], y, t, THW=(b - a, H, W), rotary_emb=freqs[:, :, a * P:b * P],
+                          save_kv_cache=True, kv_cache=cache)
+        outs.append(o)
+        if acc is None:
+            acc = [saved[0], saved[1], saved[2]]
+        else:   # states add up, the temporal-conv tail is replaced
+            acc = [acc[0] + saved[0], acc[1] + saved[1], saved[2]]
+    torch.testing.assert_close(torch.cat(outs, 1), whole, rtol=1e-9, atol=1e-9)
