@@ -216,7 +216,7 @@ class LiteLA(nn.Module):
                 block_mask=None) -> torch.Tensor:
         return self.forward_gated(x, None, None, rotary_emb=rotary_emb)
 
-    def forward_gated(self, x, gate, residual, rotary_emb=None) -> torch.Tensor:
+    def forward_gated(self, x, gate, residual, rotary_emb=None, **kwargs) -> torch.Tensor:
         """forward(x), or residual + gate * forward(x) with the update fused into the proj GEMM."""
         _no_grad_only(x)
         if rotary_emb is None and x.dtype == torch.bfloat16:   # qk-norm (if any) on load inside the kernels
@@ -225,7 +225,20 @@ class LiteLA(nn.Module):
         else:
             qkv = self._qkv_tokens(x, rotary_emb)
             out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps, head_dim=self.dim)
-        return self.proj(out, gate=gate, residual=residual)
+        return self._proj_gated(out, gate, residual)
+
+    def _proj_gated(self, out, gate, residual):
+        """proj(out), or residual + gate * proj(out) in the GEMM epilogue; gate is [B, 1, C] or one row per
+        group of consecutive tokens, [B, G, 1, C] (per-frame conditioning)."""
+        if gate is None:
+            return self.proj(out)
+        B, N, C = out.shape
+        groups = gate.numel() // (B * gate.shape[-1])
+        if groups == 1:
+            return self.proj(out, gate=gate.reshape(B, 1, -1), residual=residual)
+        y = self.proj(out.view(B * groups, N // groups, C), gate=gate.reshape(B * groups, 1, -1),
+                      residual=residual.reshape(B * groups, N // groups, -1))
+        return y.view(B, N, -1)
 
     def _pre(self, qkv: torch.Tensor, rotary_emb):
         """(QkPre for q, QkPre for k) for a fused [B, N, 3, C] buffer, or (None, None)."""
@@ -280,11 +293,11 @@ class LiteLAReLURope(LiteLA):
     def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None, **kwargs) -> torch.Tensor:
         return self.forward_gated(x, None, None, rotary_emb=rotary_emb)
 
-    def forward_gated(self, x, gate, residual, rotary_emb=None) -> torch.Tensor:
+    def forward_gated(self, x, gate, residual, rotary_emb=None, **kwargs) -> torch.Tensor:
         _no_grad_only(x)
         B, N, C = x.shape
         qkv = self.qkv(x).view(B, N, 3, C)
-        return self.proj(self._attend(qkv, rotary_emb), gate=gate, residual=residual)
+        return self._proj_gated(self._attend(qkv, rotary_emb), gate, residual)
 
 
 class ChunkCausalAttention(LiteLAReLURope):
@@ -295,6 +308,9 @@ class ChunkCausalAttention(LiteLAReLURope):
 
     def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None,
                 chunk_index: Optional[List[int]] = None) -> torch.Tensor:
+        return self.forward_gated(x, None, None, HW=HW, rotary_emb=rotary_emb, chunk_index=chunk_index)
+
+    def forward_gated(self, x, gate, residual, HW=None, rotary_emb=None, chunk_index=None, **kwargs) -> torch.Tensor:
         _no_grad_only(x)
         if HW is None or len(HW) != 3:
             raise ValueError("ChunkCausalAttention needs HW = (frames, h, w)")
@@ -305,7 +321,7 @@ class ChunkCausalAttention(LiteLAReLURope):
         starts = list(chunk_index) if chunk_index is not None else [0]
         qkv = self.qkv(x).view(B, N, 3, C)
         out = self._attend(qkv, rotary_emb, chunk_tokens=[s * hh * ww for s in starts])
-        return self.proj(out)
+        return self._proj_gated(out, gate, residual)
 
 
 class CachedCausalAttention(LiteLAReLURope):
@@ -318,6 +334,10 @@ class CachedCausalAttention(LiteLAReLURope):
 
     def forward(self, x: torch.Tensor, mask=None, HW=None, rotary_emb=None, block_mask=None,
                 save_kv_cache: bool = False, kv_cache: Optional[list] = None, **kwargs):
+        return self.forward_gated(x, None, None, rotary_emb=rotary_emb, save_kv_cache=save_kv_cache, kv_cache=kv_cache)
+
+    def forward_gated(self, x, gate, residual, rotary_emb=None, save_kv_cache: bool = False,
+                      kv_cache: Optional[list] = None, **kwargs):
         _no_grad_only(x)
         B, N, C = x.shape
         qkv = self.qkv(x).view(B, N, 3, C)
@@ -332,7 +352,7 @@ class CachedCausalAttention(LiteLAReLURope):
             if past_vk is not None and past_ks is not None:
                 state[:, :, 0, :d] += past_vk.to(state)
                 state[:, :, 0, d:] += past_ks.to(state)
-        out = self.proj(ops.linattn_apply(qkv[:, :, 0], state, self.eps, pre=pre_q))
+        out = self._proj_gated(ops.linattn_apply(qkv[:, :, 0], state, self.eps, pre=pre_q), gate, residual)
         if kv_cache is not None:
             return out, kv_cache
         return out
@@ -846,6 +866,11 @@ class SanaVideoMSBlock(nn.Module):
         self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
         self.block_hook = None
 
+    def _fused(self, x) -> bool:
+        """bf16 device inference with the attention's own forward (no processor patched over it)."""
+        return (x.is_cuda and x.dtype == torch.bfloat16 and not torch.is_grad_enabled()
+                and "forward" not in self.attn.__dict__)
+
     def _norm_modulate(self, norm, x, shift, scale, groups: int):
         """t2i_modulate(norm(x), shift, scale) with ``groups`` modulation rows per batch entry (1, or one per
         frame): shift / scale are [B, groups, 1, C] or [B, 1, C]."""
@@ -868,7 +893,10 @@ class SanaVideoMSBlock(nn.Module):
         if chunk_index is not None:
             attn_kw["chunk_index"] = chunk_index[:]
         h = self._norm_modulate(self.norm1, x, shift_msa, scale_msa, num_frames)
-        x = x + (gate_msa * self.attn(h, **attn_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+        if self._fused(x):
+            x = self.attn.forward_gated(h, gate_msa, x, **attn_kw)
+        else:
+            x = x + (gate_msa * self.attn(h, **attn_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
         x = x + self.cross_attn(x, y, mask=mask)
         mlp_kw = {"HW": THW}
         if chunk_index is not None:
@@ -894,11 +922,18 @@ class SanaVideoMSBlock(nn.Module):
         kv_cache = kwargs.get("kv_cache", None)
         if kv_cache is not None:
             attn_kw["kv_cache"] = kv_cache
-        x_sa = self.attn(self._norm_modulate(self.norm1, x, shift_msa, scale_msa, 1), **attn_kw)
-        if kv_cache is not None:
-            x_sa, kv_cache = x_sa
-        feats["x_self_attn"] = x_sa
-        x = x + gate_msa * x_sa
+        h = self._norm_modulate(self.norm1, x, shift_msa, scale_msa, 1)
+        if self.block_hook is None and self._fused(x):
+            # x + gate * attn(h) inside the attention's proj GEMM (a hook wants the attention output itself)
+            x = self.attn.forward_gated(h, gate_msa, x, **attn_kw)
+            if kv_cache is not None:
+                x, kv_cache = x
+        else:
+            x_sa = self.attn(h, **attn_kw)
+            if kv_cache is not None:
+                x_sa, kv_cache = x_sa
+            feats["x_self_attn"] = x_sa
+            x = x + gate_msa * x_sa
         x = x + self.cross_attn(x, y, mask=mask)
         feats["x_cross_attn"] = x
         mlp_kw = {"HW": THW}

@@ -375,7 +375,8 @@ def _freqs(N, d, seed):
 
 @pytest.mark.parametrize("attn_type,ffn_type,d,C", [("chunkcausal", "ChunkGLUMBConvTemp", 32, 128),
                                                     ("LiteLAReLURope", "GLUMBConvTemp", 112, 224),
-                                                    ("ChunkedLiteLAReLURope", "glumbconv", 32, 96)])
+                                                    ("ChunkedLiteLAReLURope", "glumbconv", 32, 96),
+                                                    ("linear", "glumbconv", 32, 128)])
 def test_video_block_matches_oracle(cuda, attn_type, ffn_type, d, C):
     """SanaVideoMSBlock (sana_multi_scale_video.py:66-333) against the fp64 oracle: flat conditioning, one
     modulation row per frame, text mask, block_hook."""
@@ -384,13 +385,15 @@ def test_video_block_matches_oracle(cuda, attn_type, ffn_type, d, C):
     ob, hb = _video_blocks(C, 4, attn_type, ffn_type, seed=d, qk_norm=True, linear_head_dim=d)
     hb = hb.to(cuda)
     x, y, t = (a.bfloat16() for a in O.block_inputs(B, N, C, n_text=40, seed=d))
-    freqs = _freqs(N, d, 3)
+    # LiteLA takes the real-valued (cos, sin) form of the rotary embedding, applied before the ReLU: none here
+    freqs = _freqs(N, d, 3) if attn_type != "linear" else None
     kw = {"chunk_index": [0, 1, 3]} if attn_type == "chunkcausal" else {}
     with torch.no_grad():
         ref = _ref64(ob, x, y, t, THW=(T, H, W), rotary_emb=freqs, **kw)
         seen = {}
         hb.block_hook = lambda **feats: seen.update(feats)
-        out = hb(x.to(cuda), y.to(cuda), t.to(cuda), THW=(T, H, W), rotary_emb=freqs.to(cuda), **kw)
+        dfreqs = None if freqs is None else freqs.to(cuda)
+        out = hb(x.to(cuda), y.to(cuda), t.to(cuda), THW=(T, H, W), rotary_emb=dfreqs, **kw)
         check(out, ref, f"{attn_type}/{ffn_type}", block=True)
         assert set(seen) == {"x_in", "x_self_attn", "x_cross_attn", "x_ffn"} and torch.equal(seen["x_ffn"], out)
         hb.block_hook = None
@@ -398,7 +401,7 @@ def test_video_block_matches_oracle(cuda, attn_type, ffn_type, d, C):
         mask = torch.ones(B, 40, dtype=torch.long)
         mask[:, 25:] = 0
         ref = _ref64(ob, x, y, tf, mask=mask, THW=(T, H, W), rotary_emb=freqs, **kw)
-        out = hb(x.to(cuda), y.to(cuda), tf.to(cuda), mask=mask.to(cuda), THW=(T, H, W), rotary_emb=freqs.to(cuda), **kw)
+        out = hb(x.to(cuda), y.to(cuda), tf.to(cuda), mask=mask.to(cuda), THW=(T, H, W), rotary_emb=dfreqs, **kw)
         check(out, ref, f"{attn_type}/{ffn_type}, per-frame conditioning", block=True)
 
 
