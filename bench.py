@@ -279,6 +279,29 @@ def images_per_s(dev, w8: bool, steps: int, warmup: int, B: int = 16) -> float:
     return B / (DEPTH * t_us * 1e-6)
 
 
+def video_block_ms(dev, steps: int = 10, warmup: int = 3) -> float:
+    """One SanaVideoMSBlock forward at the video shape (21 x 30 x 52 tokens, C = 2240, 20 heads of 112, q/k norm,
+    rotary embedding, chunk_index [0, 11], temporal Mix-FFN): the reference's released video configuration."""
+    import sana_amd as S
+
+    T, H, W, d = 21, 30, 52, 112
+    N = T * H * W
+    g = torch.Generator().manual_seed(5)
+    blk = S.SanaVideoMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="chunkcausal", ffn_type="ChunkGLUMBConvTemp",
+                             qk_norm=True, linear_head_dim=d).bfloat16()
+    with torch.no_grad():
+        for n, p in blk.named_parameters():
+            if n != "scale_shift_table" and p.dim() > 1:
+                p.copy_(torch.nn.init.trunc_normal_(torch.empty(p.shape), std=0.02, generator=g))
+    blk = blk.to(dev)
+    x, y, t = (a.bfloat16().to(dev) for a in make_inputs(1, N))
+    theta = torch.rand(N, d // 2, generator=g, dtype=torch.float64) * 6.283
+    freqs = torch.polar(torch.ones_like(theta), theta)[None, None].to(dev)
+    with torch.no_grad():
+        t_us = event_time_us(lambda: blk(x, y, t, THW=(T, H, W), rotary_emb=freqs, chunk_index=[0, 11]), steps, warmup)
+    return t_us / 1e3
+
+
 def cpu_baseline(iters: int = 5):
     """The oracle (stock PyTorch restatement of the reference block) on the host
     cores: one block of the cfg3 workload in fp32 (bf16 GEMM/conv on CPU is not a
@@ -364,6 +387,7 @@ def main():
         ips_bf16 = images_per_s(dev, False, 20, 5)
         ips_w8 = images_per_s(dev, True, 20, 5)
         one_image_ms = 1e3 / images_per_s(dev, False, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
+        video_ms = video_block_ms(dev)
     del blocks
     torch.cuda.empty_cache()
 
@@ -385,6 +409,9 @@ def main():
                                 "note": "B=16, N=1024: B / (20 x block latency); DiT blocks of one denoising step only "
                                         "(no text encoder, VAE, embedders, step count or CFG doubling); "
                                         "one_image_step_ms: the same 20 blocks at B=1"},
+        "video_block_ms": {"value": round(video_ms, 3),
+                           "note": "one SanaVideoMSBlock forward, bf16: N=21x30x52=32760 tokens, C=2240, 20 heads of 112, "
+                                   "q/k RMSNorm + rotary embedding, chunk_index [0, 11], ChunkGLUMBConvTemp, 300 text tokens"},
         "roofline": roofline,
         "kernels": kernels,
         "copy_GBps_this_box": copy_gbs,
