@@ -268,6 +268,18 @@ int sana_hip_add_layernorm_modulate(const void* x, const void* y, const void* sc
 int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, int N, int K,
                         int64_t ldw, int64_t ldo, void* stream);
 
+/* Gated residual update as one elementwise pass:
+ *   out[m][:] = residual[m][:] + gate[m / rows_per_gate][:] * y[m][:]
+ * with the product and the sum each rounded to bf16, as the reference's two ops do.  Replaces
+ * `x + self.drop_path(gate_mlp * mlp_out)` (diffusion/model/nets/sana_multi_scale_video.py:321; per frame
+ * :247-252) where the module's last op is not a GEMM of this library (the temporal Mix-FFN variants), and
+ * `x + gate_msa * attn(...)` when a guidance processor or hook needs the attention output itself.
+ *   y, residual, out: bf16 [M][C] with row strides ldy / ldr / ldo (out may alias residual or y);
+ *   gate: bf16 rows of C values, gate_stride elements apart.  C % 8 == 0.  bf16 only. */
+int sana_hip_gate_residual(const void* y, const void* gate, const void* residual, void* out,
+                           int64_t M, int C, int64_t ldy, int64_t ldr, int64_t ldo,
+                           int rows_per_gate, int64_t gate_stride, int io_dtype, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Temporal (t, 1) convolution over frames with full channel mixing, plus its residual, as ONE GEMM over a
  * virtual im2col of the token-major buffer (no copy of the activations):

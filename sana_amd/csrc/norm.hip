@@ -100,6 +100,32 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
   }
 }
 
+// out = res + gate[row / rows_per_gate] * y with the two roundings of the stock op pair (product, then sum):
+// the gated residual update behind a module whose last op is not one of this library's GEMMs.  One thread per
+// 8 channels; three streams (y, res, out), HBM bound.
+__global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __restrict__ y,
+                                                            const uint16_t* __restrict__ gate,
+                                                            const uint16_t* __restrict__ res,
+                                                            uint16_t* __restrict__ out, int64_t M, int C, int64_t ldy,
+                                                            int64_t ldr, int64_t ldo, int rows_per_gate,
+                                                            int64_t gate_stride) {
+  const int chunks = C >> 3;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= M * chunks) return;
+  const int64_t m = id / chunks;
+  const int n = (int)(id - m * chunks) * 8;
+  const u32x4_t yv = *reinterpret_cast<const u32x4_t*>(y + m * ldy + n);
+  const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(res + m * ldr + n);
+  const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gate + (m / rows_per_gate) * gate_stride + n);
+  u32x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t t = pack_bf16(bf16_lo(gv[e]) * bf16_lo(yv[e]), bf16_hi(gv[e]) * bf16_hi(yv[e]));
+    o[e] = pack_bf16(bf16_lo(rv[e]) + bf16_lo(t), bf16_hi(rv[e]) + bf16_hi(t));
+  }
+  *reinterpret_cast<u32x4_t*>(out + m * ldo + n) = o;
+}
+
 }  // namespace
 }  // namespace sana
 
@@ -153,4 +179,23 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_add_layernorm_mod
     void* stream) {
   return ln_impl<true>(x, y, scale, shift, sum, out, M, C, ldx, ldy, lds, ldo, rows_per_mod, mod_stride, eps, io_dtype,
                        stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_gate_residual(
+    const void* y, const void* gate, const void* residual, void* out, int64_t M, int C, int64_t ldy, int64_t ldr,
+    int64_t ldo, int rows_per_gate, int64_t gate_stride, int io_dtype, void* stream) {
+  if (!y || !gate || !residual || !out || M <= 0 || C <= 0 || rows_per_gate <= 0) return SANA_ERR_ARG;
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (C % 8) return SANA_ERR_SHAPE;
+  if (ldy < C || ldr < C || ldo < C || gate_stride < 0) return SANA_ERR_ARG;
+  if (ldy % 8 || ldr % 8 || ldo % 8 || gate_stride % 8 || !aligned16(y) || !aligned16(gate) || !aligned16(residual) ||
+      !aligned16(out))
+    return SANA_ERR_ALIGN;
+  const int64_t threads = M * (C / 8);
+  if ((threads + 255) / 256 > 0x7fffffff) return SANA_ERR_SHAPE;
+  hipLaunchKernelGGL(gate_residual_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(y),
+                     static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(residual),
+                     static_cast<uint16_t*>(out), M, C, ldy, ldr, ldo, rows_per_gate, gate_stride);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }

@@ -796,7 +796,7 @@ class SanaMSBlock(nn.Module):
             h = ops.layernorm_modulate(x, scale_msa, shift_msa, self.norm1.eps)
             if "forward" in self.attn.__dict__:
                 # a guidance processor was patched over attn.forward (dpm_solver.py:486-524): call it
-                x = x + gate_msa * self.attn(h, HW=HW, rotary_emb=image_rotary_emb)
+                x = ops.gate_residual(self.attn(h, HW=HW, rotary_emb=image_rotary_emb), gate_msa, x)
             else:
                 x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
             # the cross-attention's residual add and norm2 + modulate in one pass
@@ -871,6 +871,17 @@ class SanaVideoMSBlock(nn.Module):
         return (x.is_cuda and x.dtype == torch.bfloat16 and not torch.is_grad_enabled()
                 and "forward" not in self.attn.__dict__)
 
+    @staticmethod
+    def _gate_residual(x, gate, y):
+        """x + gate * y (gate [B, 1, C] or per frame [B, F, 1, C]); one fused pass on the bf16 device path."""
+        if x.is_cuda and x.dtype == torch.bfloat16 and y.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 \
+                and not torch.is_grad_enabled():
+            return ops.gate_residual(y, gate, x)
+        B, N, C = x.shape
+        if gate.dim() == 4:
+            return x + (gate * y.reshape(B, gate.shape[1], -1, C)).reshape(B, N, C)
+        return x + gate * y
+
     def _norm_modulate(self, norm, x, shift, scale, groups: int):
         """t2i_modulate(norm(x), shift, scale) with ``groups`` modulation rows per batch entry (1, or one per
         frame): shift / scale are [B, groups, 1, C] or [B, 1, C]."""
@@ -896,14 +907,13 @@ class SanaVideoMSBlock(nn.Module):
         if self._fused(x):
             x = self.attn.forward_gated(h, gate_msa, x, **attn_kw)
         else:
-            x = x + (gate_msa * self.attn(h, **attn_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
+            x = self._gate_residual(x, gate_msa, self.attn(h, **attn_kw))
         x = x + self.cross_attn(x, y, mask=mask)
         mlp_kw = {"HW": THW}
         if chunk_index is not None:
             mlp_kw["chunk_index"] = chunk_index[:]
         h = self._norm_modulate(self.norm2, x, shift_mlp, scale_mlp, num_frames)
-        x = x + (gate_mlp * self.mlp(h, **mlp_kw).reshape(B, num_frames, -1, C)).reshape(B, N, C)
-        return x
+        return self._gate_residual(x, gate_mlp, self.mlp(h, **mlp_kw))
 
     def forward(self, x, y, t, mask=None, THW=None, rotary_emb=None, chunk_index=None, **kwargs):
         if len(t.shape) > 2:
@@ -933,7 +943,7 @@ class SanaVideoMSBlock(nn.Module):
             if kv_cache is not None:
                 x_sa, kv_cache = x_sa
             feats["x_self_attn"] = x_sa
-            x = x + gate_msa * x_sa
+            x = self._gate_residual(x, gate_msa, x_sa)
         x = x + self.cross_attn(x, y, mask=mask)
         feats["x_cross_attn"] = x
         mlp_kw = {"HW": THW}
@@ -946,7 +956,7 @@ class SanaVideoMSBlock(nn.Module):
         mlp_out = self.mlp(self._norm_modulate(self.norm2, x, shift_mlp, scale_mlp, 1), **mlp_kw)
         if kv_cache is not None:
             mlp_out, kv_cache = mlp_out
-        x = x + gate_mlp * mlp_out
+        x = self._gate_residual(x, gate_mlp, mlp_out)
         feats["x_ffn"] = x
         if self.block_hook is not None:
             self.block_hook(**feats)

@@ -506,3 +506,26 @@ def add_layernorm_modulate(x: torch.Tensor, y: torch.Tensor, scale: torch.Tensor
         ldx, ldy, C, C, Ntok, s1, float(eps), _dt(x), _stream())
     _lib.check(code, "sana_hip_add_layernorm_modulate")
     return total.view(B, Ntok, C), out.view(B, Ntok, C)
+
+
+def gate_residual(y: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+    """residual + gate * y in one pass with the stock op pair's two roundings; y, residual: [B, N, C] bf16;
+    gate: [B, 1, C], or one row per group of consecutive tokens, [B, G, 1, C]."""
+    _need_cuda(y, gate, residual)
+    if y.shape != residual.shape or y.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or \
+            gate.dtype != torch.bfloat16:
+        raise SanaHipError("gate_residual needs bf16 y and residual of one shape and a bf16 gate")
+    B, Ntok, C = y.shape
+    groups = gate.numel() // max(B * C, 1)
+    if groups < 1 or gate.numel() != B * groups * C or Ntok % groups:
+        raise SanaHipError(f"gate {tuple(gate.shape)} does not divide the {Ntok} tokens of {B} batch entries")
+    y2, ldy = _rows(y.reshape(B * Ntok, C), "y")
+    r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
+    g2, gstride = _mod_rows(gate.reshape(B * groups, 1, C), B * groups, C, "gate")
+    out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=y.device)
+    if B * Ntok == 0:
+        return out.view(B, Ntok, C)
+    code = _lib.load().sana_hip_gate_residual(y2.data_ptr(), g2.data_ptr(), r2.data_ptr(), out.data_ptr(), B * Ntok, C,
+                                              ldy, ldr, C, Ntok // groups, gstride, _dt(y), _stream())
+    _lib.check(code, "sana_hip_gate_residual")
+    return out.view(B, Ntok, C)

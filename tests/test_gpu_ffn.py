@@ -331,3 +331,16 @@ def test_temporal_conv_zero_weight_is_identity(cuda):
     buf = torch.cat([torch.zeros(P, C, dtype=torch.bfloat16, device=cuda), y])
     out = ops.tconv_residual(buf, torch.zeros(C, 3 * C, dtype=torch.bfloat16, device=cuda), T * P, P)
     assert torch.equal(out, y)
+
+
+@pytest.mark.parametrize("B,Ntok,C,groups", [(1, 32760, 2240, 1), (2, 120, 96, 4), (3, 77, 1152, 1), (1, 60, 128, 60)])
+def test_gate_residual_equals_the_stock_op_pair(cuda, B, Ntok, C, groups):
+    """res + gate * y as one pass: the bits of the two stock ops (product rounded to bf16, then the sum), with one
+    gate row per batch entry or per group of consecutive tokens (per-frame conditioning)."""
+    g = torch.Generator().manual_seed(C + groups)
+    y = torch.randn(B, Ntok, C, generator=g).bfloat16().to(cuda)
+    res = torch.randn(B, Ntok, C, generator=g).bfloat16().to(cuda)
+    mod = (torch.randn(B, groups, 6, C, generator=g) * 0.7).bfloat16().to(cuda)
+    gate = mod[:, :, 2:3]                                          # [B, G, 1, C], a strided view as in the blocks
+    want = res + (gate * y.view(B, groups, -1, C)).view(B, Ntok, C)
+    assert torch.equal(ops.gate_residual(y, gate if groups > 1 else gate[:, 0], res), want)
