@@ -394,7 +394,8 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
 // SPLIT (split-k, for shapes with too few tiles to fill the chip): grid row z multiplies its own range of
 // k-tiles and stores the raw fp32 accumulators to C taken as float [gridDim.y][M][N]; splitk_epilogue_kernel
 // adds the ranges up in order and applies the epilogue.
-template <bool W8, int EPI, int NI, bool TAPS = false, bool SPLIT = false>
+// TAPS: 0 = plain A operand, 1 = tap-concatenated A operand, 2 = the same with per-row-block zero_last flags.
+template <bool W8, int EPI, int NI, int TAPS = 0, bool SPLIT = false>
 __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A_, const void* __restrict__ Wv_,
                                                     const float* __restrict__ scale, const EpiArgs ep,
                                                     uint16_t* __restrict__ C, int M, int N, int K_, int64_t lda,
@@ -483,18 +484,30 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int tap_b = TAPS ? (int)(tp.stride * lda * 2) : 0;
   auto a_koff = [&](int k0) { return TAPS ? (k0 / tp.kc) * tap_b + (k0 % tp.kc) * 2 : k0 * 2; };
   int a_kb = 0, a_kin = 0;  // offset of the k-tile being requested, and its column inside the tap
-  // rows of this thread (bit q: row g_row + 32*q) whose last tap is zero padding, and the same mask while the
-  // k-tile being requested belongs to the last tap (else 0)
-  uint32_t zlast = 0, a_zmask = 0;
+  // rows of this thread (bit q: row g_row + 32*q) whose last tap is zero padding.  While the k-tile being
+  // requested belongs to the last tap, those rows' vector offsets carry 2^31 -- outside the resource, so the
+  // loads return zeros -- at no cost in the loop: the per-row offsets live in registers and change with the tap.
+  uint32_t zlast = 0;
+  int voffq[8];
   int a_tap = 0;
   const int last_tap = TAPS ? K / tp.kc - 1 : 0;
-  if (TAPS && tp.zero_last) {
+  if (TAPS == 2 && tp.zero_last) {
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int r = m0 + (tid >> 3) + 32 * q;
       if (r < M && tp.zero_last[r / tp.stride]) zlast |= 1u << q;
     }
   }
+  const int voff_a0 = ((tid >> 3) * (int)lda + 8 * (tid & 7)) * 2;  // the thread's (row, k chunk) inside the tile
+  auto poison = [&](bool last) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) voffq[q] = voff_a0;
+    if (TAPS == 2 && last) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) voffq[q] = voff_a0 + (((zlast >> q) & 1u) ? (int)0x80000000u : 0);
+    }
+  };
+  poison(false);
   const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * (W8 ? 1 : 2)), 0,
       (int)(((int64_t)w_last * ldw + K) * (W8 ? 1 : 2)), 0x00020000);
@@ -503,8 +516,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int step_a = 32 * (int)ulda * 2, step_w = W8 ? 64 * (int)uldw : 32 * (int)uldw * 2;
   auto gload = [&](int q, int k0) {
     if (q < 8) {
-      int off = voff_a + (q * step_a + (TAPS ? a_kb : k0 * 2));
-      if (TAPS) off = ((a_zmask >> q) & 1u) ? (int)0x80000000u : off;  // outside the resource: reads zeros
+      const int off = (TAPS == 2 ? voffq[q] : voff_a) + (q * step_a + (TAPS ? a_kb : k0 * 2));
       const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0);
       rs[q] = __builtin_bit_cast(u32x4_t, v);
     } else {
@@ -544,7 +556,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   for (int q = 0; q < NQ; ++q) gload(q, 0);
   if (TAPS) {
     a_kb = a_koff(BK);
-    a_zmask = BK / tp.kc == last_tap ? zlast : 0u;
+    if (TAPS == 2 && zlast) poison(BK / tp.kc == last_tap);
   }
 #pragma unroll
   for (int q = 0; q < (W8 ? 8 : NQ); ++q) lstore(q, 0);
@@ -558,7 +570,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     a_kb = a_koff(2 * BK);
     a_kin = (2 * BK) % tp.kc;
     a_tap = (2 * BK) / tp.kc;
-    a_zmask = a_tap == last_tap ? zlast : 0u;
+    if (TAPS == 2 && zlast) poison(a_tap == last_tap);
   }
   __syncthreads();
 #pragma unroll
@@ -614,7 +626,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
         a_kin -= tp.kc;
         a_kb += tap_b - tp.kc * 2;
         ++a_tap;
-        a_zmask = a_tap == last_tap ? zlast : 0u;
+        if (TAPS == 2 && zlast) poison(a_tap == last_tap);
       }
     }
   }
@@ -896,7 +908,7 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
     const GemmPlan pl = plan_gemm(M, N, K, W8);
     if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
       const Taps split = {0, 0, 0, pl.tiles, pl.rem, nullptr};
-      hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, false, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
+      hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, 0, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
                          a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
                          split);
       if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
@@ -917,8 +929,12 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
   }
   if (taps) {  // only the bf16 gated-residual instance exists with taps
     if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
-    hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, true>), grid, block, 0, s, a, W, scale, ep, c, M, N,
-                       K, lda, ldw, ldc, tiles_t, tiles_c, *taps);
+    if (taps->zero_last)
+      hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
+                         lda, ldw, ldc, tiles_t, tiles_c, *taps);
+    else
+      hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 1>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
+                         lda, ldw, ldc, tiles_t, tiles_c, *taps);
     return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
   }
 #define SANA_LAUNCH4(EPI)                                                                                         \
