@@ -42,7 +42,7 @@ if ROOT not in sys.path:
 
 # HBM bytes per launch of the dominant kernel (inverted-conv GEMM at cfg3), from the pmc summary
 # profiles/kernels_cfg3_hbm_traffic.txt: FETCH_SIZE x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE x 1.0.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 1641817292  # 1274.8 MB read + 367.0 MB written
+DOMINANT_KERNEL_TRAFFIC_BYTES = 1640357273  # 1274.8 MB read + 367.0 MB written
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
