@@ -738,56 +738,76 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
           bv[i][8 * half + 2 * e + 1] = bf16_hi(bpk[i][half][e]);
         }
   }
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  // Software-pipelined over the four groups of 32 tokens: step s of phase j converts piece s of group j
+  // (accumulators -> activation -> LDS) and stores row chunk s of group j - 1 (LDS -> gate / residual -> global).
+  // Handing a 16-byte-per-lane store to the memory pipeline keeps it busy for ~130 clocks, during which the
+  // wave can issue VALU work but not another store: one store between two pieces of arithmetic costs a
+  // fraction of what eight stores in a row cost.
+  auto convert_piece = [&](int j, int p) {  // p = 2 * i + half
+    const int i = p >> 1, half = p & 1;
     const int tok = 32 * j + fr;
+    float a8[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
+    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[i] + 8 * half);
+    const int chunk = 4 * i + 2 * fg + half;
+    *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
+  };
+  auto read_row = [&](int j, int it) {
+    const int row = 32 * j + it * 4 + o_rsub;
+    return *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
+  };
+#pragma unroll
+  for (int j = 0; j <= 4; ++j) {
+    const int js = j - 1;  // the group whose rows are stored in this phase
     // The lane's eight gate values, as floats.  One gate row serves the whole group of 32 tokens unless a
     // batch boundary runs through it: then the rows from m_switch on take the next gate row (gates are per
     // batch entry; entries shorter than 32 tokens take the slow way, a division per row).
-    const int m_first = wrow0 + 32 * j;
-    const int g_first = m_first / ep.rows_per_gate;
-    const int m_switch = (g_first + 1) * ep.rows_per_gate;
-    const bool two_gates = EPI == SANA_EPI_GATE_RES && ep.gate && m_switch < min(m_first + 32, M);
+    const int m_first = wrow0 + 32 * js;
+    int m_switch = 0;
+    bool two_gates = false;
     float gf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // no gate: 1.0, a plain residual add
-    if (EPI == SANA_EPI_GATE_RES && ep.gate && o_live && m_first < M) {
-      const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
+    u32x4_t o_next = {0u, 0u, 0u, 0u};
+    if (js >= 0) {
+      if (EPI == SANA_EPI_GATE_RES) {
+        const int g_first = m_first / ep.rows_per_gate;
+        m_switch = (g_first + 1) * ep.rows_per_gate;
+        two_gates = ep.gate && m_switch < min(m_first + 32, M);
+        if (ep.gate && o_live && m_first < M) {
+          const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        gf[2 * e] = bf16_lo(gate[e]);
-        gf[2 * e + 1] = bf16_hi(gate[e]);
+          for (int e = 0; e < 4; ++e) {
+            gf[2 * e] = bf16_lo(gate[e]);
+            gf[2 * e + 1] = bf16_hi(gate[e]);
+          }
+        }
       }
+      o_next = read_row(js, 0);  // wave-private LDS is in order: the group's writes are behind it
     }
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        float a8[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
-        const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[i] + 8 * half);
-        const int chunk = 4 * i + 2 * fg + half;
-        *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
+    for (int st = 0; st < 8; ++st) {
+      u32x4_t o = o_next;
+      if (js >= 0 && st + 1 < 8) o_next = read_row(js, st + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j < 4 && st < 2 * NI) convert_piece(j, st);
+      __builtin_amdgcn_sched_barrier(0);
+      if (js >= 0) {
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[js][st]);
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int row = 32 * j + it * 4 + o_rsub;
-      u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-      if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[j][it]);
-      __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * j + it) * c_step, 0, 0);
-    }
-    if (two_gates) {  // uniform, rare: rows behind the boundary are redone with their own gate row and stored again
+    if (js >= 0 && two_gates) {  // uniform, rare: rows behind the boundary are redone with their own gate row and stored again
 #pragma unroll 1
       for (int it = 0; it < 8; ++it) {
-        const int row = 32 * j + it * 4 + o_rsub, m = wrow0 + row;
+        const int row = 32 * js + it * 4 + o_rsub, m = wrow0 + row;
         if (o_live && m >= m_switch && m < M) {
           const u32x4_t y = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
           const u32x4_t r = __builtin_bit_cast(
-              u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, 0));
+              u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * js + it) * r_step, 0, 0));
           const u32x4_t g2 = *reinterpret_cast<const u32x4_t*>(
               ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
-          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * j + it) * c_step, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * js + it) * c_step, 0, 0);
         }
       }
     }
