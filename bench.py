@@ -109,7 +109,7 @@ def event_time_us(fn, iters: int, warmup: int, repeats: int = 3) -> float:
     return sorted(times)[len(times) // 2]
 
 
-def kernel_rooflines(dev, iters=50, warmup=10):
+def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
     """Each hand-written kernel alone at the cfg3 shape (B=1, N=16384)."""
     from sana_amd import ops
 
@@ -247,11 +247,15 @@ def kernel_rooflines(dev, iters=50, warmup=10):
     add("tconv_residual_cfg5", "mfma", 2 * Tf * Pf * 3 * C * C,
         event_time_us(lambda: ops.tconv_residual(buf, wt, Tf * Pf, Pf, out=ot), 10, 3),
         f"2*M*3C*C, M={Tf * Pf} (21 frames of 1560 tokens), C={C}")
-    xr = buf[Pf:].view(1, Tf, Pf, C).permute(0, 3, 1, 2)
-    w4 = wt.view(C, 3, C).permute(0, 2, 1).unsqueeze(-1).contiguous()
-    rows[-1]["library_conv_us"] = round(event_time_us(
-        lambda: xr + torch.nn.functional.conv2d(xr, w4, padding=(1, 0)), 3, 1), 2)
-    del buf, ot, xr
+    if stock_conv:
+        # off by default: on a fresh machine the convolution library first times its candidate kernels for this
+        # shape, a naive one among them that runs ~14 s per call -- about two minutes before the first result
+        xr = buf[Pf:].view(1, Tf, Pf, C).permute(0, 3, 1, 2)
+        w4 = wt.view(C, 3, C).permute(0, 2, 1).unsqueeze(-1).contiguous()
+        rows[-1]["library_conv_us"] = round(event_time_us(
+            lambda: xr + torch.nn.functional.conv2d(xr, w4, padding=(1, 0)), 3, 1), 2)
+        del xr
+    del buf, ot
     # plain device copy as a bandwidth yardstick of this box
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
@@ -340,6 +344,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--kernels-only", action="store_true", help="only the per-kernel section (profiling runs)")
+    ap.add_argument("--stock-conv", action="store_true",
+                    help="also time the stock convolution beside the temporal-conv GEMM (minutes of library tuning on a fresh machine)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -352,7 +358,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.kernels_only:
         with torch.no_grad():
-            kernels, copy_gbs = kernel_rooflines(dev)
+            kernels, copy_gbs = kernel_rooflines(dev, stock_conv=args.stock_conv)
         print(json.dumps({"kernels": kernels, "copy_GBps_this_box": copy_gbs}))
         return
     B, HW = 1, (128, 128)
@@ -383,7 +389,7 @@ def main():
         ms_per_step = wall * 1e3 / args.steps
         block_ms = ms_per_step / DEPTH
 
-        kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev)
+        kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev, stock_conv=args.stock_conv)
         ips_bf16 = images_per_s(dev, False, 20, 5)
         ips_w8 = images_per_s(dev, True, 20, 5)
         one_image_ms = 1e3 / images_per_s(dev, False, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
