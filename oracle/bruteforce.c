@@ -14,6 +14,16 @@
  * (diffusion/model/nets/sana_blocks.py:245-263).  The chunk-causal variant
  * restricts m to chunk(m) <= chunk(n) (sana_blocks.py:481-489, rotary = 1).
  *
+ * The rotary family (LiteLAReLURope / ChunkCausalAttention / CachedCausalAttention,
+ * sana_blocks.py:359-383, 481-489, 544-562) multiplies the channel pairs
+ * (2p, 2p+1) of relu(q_n), relu(k_n), read as complex numbers, by a per-token
+ * factor f[n][p] -- but only in the numerator; the denominator keeps the
+ * unrotated vectors (`z` from `k`, `q` at :378; `vk`, `out` from `k_rotated`,
+ * `q_rotated` at :380-381):
+ *
+ *   out[i, n] = sum_m v[i, m] * <rot_m(relu k_m), rot_n(relu q_n)>
+ *               / (sum_m <relu k_m, relu q_n> + eps)
+ *
  * The depthwise conv + gate follows GLUMBConv._apply_spatial
  * (diffusion/model/nets/basic_modules.py:161-167): 3x3, zero padding 1,
  * stride 1, one filter per channel, then a = first half, g = second half,
@@ -44,6 +54,49 @@ void brute_relu_attention(const double* q, const double* k, const double* v,
         for (int j = 0; j < d; ++j) s += relu(K[(size_t)m * d + j]) * relu(Q[(size_t)n * d + j]);
         den += s;
         for (int i = 0; i < d; ++i) O[(size_t)n * d + i] += V[(size_t)m * d + i] * s;
+      }
+      for (int i = 0; i < d; ++i) O[(size_t)n * d + i] /= (den + eps);
+    }
+  }
+}
+
+/* The rotary family in quadratic form.  q, k, v, out, chunk_of as above;
+ * f_re, f_im: [N][d/2] real and imaginary part of the per-token factors (any
+ * complex number, not only unit ones), shared by all BH.  <.,.> is the plain
+ * real dot product over the d channels of the rotated vectors. */
+static void rotate_token(const double* x, const double* f_re, const double* f_im, int d, double* y) {
+  for (int p = 0; p < d / 2; ++p) {
+    const double a = relu(x[2 * p]), b = relu(x[2 * p + 1]);
+    y[2 * p] = a * f_re[p] - b * f_im[p];
+    y[2 * p + 1] = a * f_im[p] + b * f_re[p];
+  }
+}
+
+void brute_relu_attention_rope(const double* q, const double* k, const double* v,
+                               const double* f_re, const double* f_im,
+                               const int32_t* chunk_of, double eps,
+                               int BH, int N, int d, double* out) {
+  double qr[512], kr[512];
+  if (d > 512 || (d & 1)) return;
+  for (int bh = 0; bh < BH; ++bh) {
+    const double* Q = q + (size_t)bh * N * d;
+    const double* K = k + (size_t)bh * N * d;
+    const double* V = v + (size_t)bh * N * d;
+    double* O = out + (size_t)bh * N * d;
+    for (int n = 0; n < N; ++n) {
+      double den = 0.0;
+      rotate_token(Q + (size_t)n * d, f_re + (size_t)n * (d / 2), f_im + (size_t)n * (d / 2), d, qr);
+      for (int i = 0; i < d; ++i) O[(size_t)n * d + i] = 0.0;
+      for (int m = 0; m < N; ++m) {
+        if (chunk_of && chunk_of[m] > chunk_of[n]) continue;
+        rotate_token(K + (size_t)m * d, f_re + (size_t)m * (d / 2), f_im + (size_t)m * (d / 2), d, kr);
+        double s_plain = 0.0, s_rot = 0.0;
+        for (int j = 0; j < d; ++j) {
+          s_plain += relu(K[(size_t)m * d + j]) * relu(Q[(size_t)n * d + j]);
+          s_rot += kr[j] * qr[j];
+        }
+        den += s_plain;
+        for (int i = 0; i < d; ++i) O[(size_t)n * d + i] += V[(size_t)m * d + i] * s_rot;
       }
       for (int i = 0; i < d; ++i) O[(size_t)n * d + i] /= (den + eps);
     }

@@ -46,6 +46,21 @@ def relu_attention(q, k, v, eps, chunk_of=None):
     return out
 
 
+def relu_attention_rope(q, k, v, freqs, eps, chunk_of=None):
+    """Rotary family: q, k, v float64 [BH, N, d]; freqs complex [N, d/2] (per-token factors
+    of the channel pairs, numerator only).  Returns [BH, N, d]."""
+    q, k, v = (np.ascontiguousarray(t, dtype=np.float64) for t in (q, k, v))
+    BH, N, d = q.shape
+    freqs = np.asarray(freqs).reshape(N, d // 2)
+    f_re = np.ascontiguousarray(freqs.real, dtype=np.float64)
+    f_im = np.ascontiguousarray(freqs.imag, dtype=np.float64)
+    out = np.full_like(q, np.nan)
+    co = None if chunk_of is None else np.ascontiguousarray(chunk_of, dtype=np.int32)
+    lib().brute_relu_attention_rope(_p(q), _p(k), _p(v), _p(f_re), _p(f_im), None if co is None else _p(co),
+                                    ctypes.c_double(eps), BH, N, d, _p(out))
+    return out
+
+
 def attention_state(k, v):
     """k, v: float64 [BH, N, d].  Returns [BH, d+1, d]."""
     k, v = (np.ascontiguousarray(t, dtype=np.float64) for t in (k, v))

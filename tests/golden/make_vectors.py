@@ -1,5 +1,5 @@
-"""Writes ``tests/golden/kat.npz``: known-answer vectors for the linear-attention and depthwise-gate
-kernels, computed in fp64 by the plain-C quadratic-form / 9-tap restatement (``oracle/bruteforce.c``).
+"""Writes ``tests/golden/kat.npz``: known-answer vectors for the linear-attention (plain, chunk-causal, rotary) and
+depthwise-gate kernels, computed in fp64 by the plain-C quadratic-form / 9-tap restatement (``oracle/bruteforce.c``).
 
 The reference holds no numeric fixtures for this path, so these vectors are the build's own: they
 freeze the brute-force answers on seeded inputs (all exactly representable in bf16), and both the
@@ -44,6 +44,19 @@ def main():
     w = bf16_values(g, 2 * C, 3, 3, scale=0.3)
     b = bf16_values(g, 2 * C, scale=0.1)
     vec.update(dw_u=u, dw_w=w, dw_b=b, dw_out=cbrute.dwconv_gate(u, w, b))
+    # rotary family: per-token complex factors on the channel pairs of relu(q), relu(k) in the NUMERATOR only
+    # (unit modulus, generic angles, stored as fp32-exact cos / sin so every consumer rotates by the same numbers),
+    # three chunks of 12 tokens for the chunk-causal form
+    for tag, BH, N, d in (("rope32", 2, 36, 32), ("rope112", 1, 36, 112)):
+        q, k, v = (bf16_values(g, BH, N, d) for _ in range(3))
+        theta = (torch.rand(N, d // 2, generator=g, dtype=torch.float64) - 0.5) * 6.0
+        cos, sin = torch.cos(theta).float().double().numpy(), torch.sin(theta).float().double().numpy()
+        freqs = cos + 1j * sin
+        chunk_of = np.repeat(np.arange(3, dtype=np.int32), 12)
+        vec.update({f"{tag}_q": q, f"{tag}_k": k, f"{tag}_v": v, f"{tag}_cos": cos, f"{tag}_sin": sin,
+                    f"{tag}_chunk_of": chunk_of,
+                    f"{tag}_out": cbrute.relu_attention_rope(q, k, v, freqs, 1e-8),
+                    f"{tag}_cc_out": cbrute.relu_attention_rope(q, k, v, freqs, 1e-8, chunk_of)})
     np.savez_compressed(OUT, **vec)
     print(f"wrote {OUT}: {os.path.getsize(OUT)} bytes, {len(vec)} arrays")
 

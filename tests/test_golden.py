@@ -62,6 +62,46 @@ def test_oracle_depthwise_gate_reproduces_fixture():
     assert rel_l2(out, T("dw_out")) < 1e-12
 
 
+def _module_fed_with(cls, q, k, v):
+    """An oracle attention module whose qkv projection reproduces the fixture's q, k, v exactly (N <= C, so a
+    weight with x @ W^T = [q | k | v] exists) and whose output projection is the identity."""
+    BH, N, d = q.shape
+    C = BH * d
+    tok = lambda t: t.transpose(0, 1).reshape(N, C)
+    target = torch.cat([tok(q), tok(k), tok(v)], dim=1)                 # [N, 3C]
+    x = torch.randn(N, C, generator=torch.Generator().manual_seed(1), dtype=torch.float64)
+    W = torch.linalg.lstsq(x, target).solution.T                        # [3C, C]
+    assert (x @ W.T - target).abs().max().item() < 1e-10
+    m = cls(C, C, dim=d, eps=1e-8).double()
+    with torch.no_grad():
+        m.qkv.weight.copy_(W)
+        m.proj.weight.copy_(torch.eye(C, dtype=torch.float64))
+        m.proj.bias.zero_()
+    return m, x[None], tok
+
+
+@pytest.mark.parametrize("tag", ["rope32", "rope112"])
+def test_oracle_rotary_family_reproduces_fixture(tag):
+    """LiteLAReLURope, ChunkCausalAttention and the streamed CachedCausalAttention against the frozen brute-force
+    answers (numerator rotated, denominator not: sana_blocks.py:378-381, 481-489, 544-562)."""
+    q, k, v = T(f"{tag}_q"), T(f"{tag}_k"), T(f"{tag}_v")
+    N = q.shape[1]
+    rot = torch.complex(T(f"{tag}_cos"), T(f"{tag}_sin"))[None, None]
+    m, x, tok = _module_fed_with(O.LiteLAReLURope, q, k, v)
+    assert rel_l2(m(x, rotary_emb=rot)[0], tok(T(f"{tag}_out"))) < 1e-9
+    cc, x, tok = _module_fed_with(O.ChunkCausalAttention, q, k, v)
+    ref_cc = tok(T(f"{tag}_cc_out"))
+    assert rel_l2(cc(x, HW=(3, 3, 4), rotary_emb=rot, chunk_index=[0, 1, 2])[0], ref_cc) < 1e-9
+    cm, x, tok = _module_fed_with(O.CachedCausalAttention, q, k, v)
+    acc, outs = [None, None], []
+    for c in range(3):
+        sl = slice(12 * c, 12 * c + 12)
+        o, cache = cm(x[:, sl], rotary_emb=rot[:, :, sl], save_kv_cache=True, kv_cache=[acc[0], acc[1]])
+        acc = [cache[i] if acc[i] is None else acc[i] + cache[i] for i in range(2)]
+        outs.append(o)
+    assert rel_l2(torch.cat(outs, 1)[0], ref_cc) < 1e-9
+
+
 # ----------------------------------------------------------------------------- GPU: kernels vs fixture
 
 @pytest.mark.gpu
@@ -100,3 +140,28 @@ def test_kernel_depthwise_gate_reproduces_fixture(cuda):
     assert rel_l2(y32.cpu(), ref) <= 1e-5
     y16 = ops.dwconv3x3_silu_gate(u.bfloat16().to(cuda), w.bfloat16().contiguous().to(cuda), b.bfloat16().to(cuda), True)
     assert (y16.cpu().double() - ref).abs().max().item() <= 2e-2 and rel_l2(y16.cpu(), ref) <= 1e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,d", [("rope32", 32), ("rope112", 112)])
+def test_kernels_rotary_family_reproduce_fixture(cuda, tag, d):
+    """sana_hip_linattn_state_pre / sana_hip_linattn_apply_pre with a rope table, whole sequence and three causal
+    chunks.  The kernels round the rotated operands to bf16 before the fp32-accumulating MFMA (the reference's
+    `.type_as(hidden_states)` after its fp64 rotation), the fixture does not: bf16 tolerance on the output."""
+    from sana_amd import ops
+    q, k, v = (T(f"{tag}_{n}") for n in "qkv")
+    BH, N, _ = q.shape
+    tm = lambda t: t.transpose(0, 1).reshape(1, N, BH * d).bfloat16().to(cuda)
+    table = torch.stack([T(f"{tag}_cos"), T(f"{tag}_sin")], dim=-1).float().contiguous().to(cuda)   # [N, d/2, 2]
+    pre = ops.QkPre(rope=table)
+    for key, chunks in ((f"{tag}_out", None), (f"{tag}_cc_out", [0, 12, 24])):
+        ref = T(key).transpose(0, 1).reshape(1, N, BH * d)
+        state = ops.linattn_state(tm(k), tm(v), chunks, causal=chunks is not None, pre=pre, head_dim=d)
+        for out_dtype in (torch.float32, torch.bfloat16):
+            out = ops.linattn_apply(tm(q), state, 1e-8, chunks, out_dtype=out_dtype, pre=pre).cpu()
+            mx, rl = (out.double() - ref).abs().max().item(), rel_l2(out, ref)
+            assert mx <= 2e-2 and rl <= 1e-2, f"{key} {out_dtype}: max-abs {mx:.3e} rel-L2 {rl:.3e}"
+        # the unrotated k-sum row of the state is exact in fp32: sum of relu(k) over the tokens seen so far
+        ksum = torch.relu(k).transpose(0, 1).reshape(N, BH, d)
+        want = ksum.sum(0) if chunks is None else ksum[:12].sum(0)
+        assert rel_l2(state[0, :, 0, d].cpu(), want) <= 1e-6

@@ -146,6 +146,87 @@ def test_cached_causal_stream_equals_chunk_causal():
     torch.testing.assert_close(torch.cat(outs, 1), full, rtol=1e-10, atol=1e-12)
 
 
+def _rope_case(cls, d, f, hh, ww, seed):
+    """Module, input, generic (non-unit) complex factors and the token-major q/k/v of every (batch, head)."""
+    heads = 2
+    C = heads * d
+    N = f * hh * ww
+    m, x = _attn_inputs(cls, C, d, N, seed=seed)
+    g = torch.Generator().manual_seed(100 + seed)
+    theta = (torch.rand(N, d // 2, generator=g, dtype=torch.float64) - 0.5) * 6.0
+    radius = 0.5 + torch.rand(N, d // 2, generator=g, dtype=torch.float64)      # not on the unit circle
+    rot = torch.polar(radius, theta)[None, None]
+    qkv = (x @ m.qkv.weight.T).view(2, N, 3, heads, d)
+    tm = lambda i: qkv[:, :, i].permute(0, 2, 1, 3).reshape(-1, N, d).detach().numpy()
+    return m, x, rot, (tm(0), tm(1), tm(2)), (C, N, heads)
+
+
+def _proj_of(att, m, C, N, heads, d):
+    att = torch.from_numpy(att).view(2, heads, N, d).permute(0, 2, 1, 3).reshape(2, N, C)
+    return att @ m.proj.weight.T + m.proj.bias
+
+
+@pytest.mark.parametrize("d", [32, 112])
+def test_relurope_matches_rotated_numerator_quadratic_form(d):
+    """Pins WHICH operands are rotated (sana_blocks.py:378-381): numerator rotated, denominator not.
+    Generic angles and radii, so a rotated denominator (or an unrotated numerator) gives other numbers."""
+    m, x, rot, (q, k, v), (C, N, heads) = _rope_case(O.LiteLAReLURope, d, 3, 2, 3, seed=5)
+    out = m(x, rotary_emb=rot)
+    ref = _proj_of(cbrute.relu_attention_rope(q, k, v, rot[0, 0].numpy(), 1e-8), m, C, N, heads, d)
+    torch.testing.assert_close(out, ref, rtol=1e-9, atol=1e-11)
+    # the two plausible mistakes are far away from the brute force: both sides rotated / none rotated
+    plain = _proj_of(cbrute.relu_attention(q, k, v, 1e-8), m, C, N, heads, d)
+    assert (plain - ref).abs().max() > 1e-3
+
+
+@pytest.mark.parametrize("d", [32, 112])
+@pytest.mark.parametrize("chunk_index", [[0, 1, 2, 3], [0, 3], [0, 1, 3]])
+def test_chunk_causal_rope_matches_masked_rotated_quadratic_form(d, chunk_index):
+    """sana_blocks.py:481-489 with a rotary embedding: cumulative rotated vk, cumulative UNROTATED k sum."""
+    f, hh, ww = 4, 2, 3
+    m, x, rot, (q, k, v), (C, N, heads) = _rope_case(O.ChunkCausalAttention, d, f, hh, ww, seed=6)
+    out = m(x, HW=(f, hh, ww), rotary_emb=rot, chunk_index=list(chunk_index))
+    bounds = list(chunk_index) + [f]
+    chunk_of = np.zeros(N, dtype=np.int32)
+    for ci, (a, b) in enumerate(zip(bounds[:-1], bounds[1:])):
+        chunk_of[a * hh * ww:b * hh * ww] = ci
+    ref = _proj_of(cbrute.relu_attention_rope(q, k, v, rot[0, 0].numpy(), 1e-8, chunk_of), m, C, N, heads, d)
+    torch.testing.assert_close(out, ref, rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("d", [32, 112])
+def test_cached_causal_rope_stream_matches_masked_rotated_quadratic_form(d):
+    """sana_blocks.py:544-562 streamed chunk by chunk (each call gets its own slice of the factors, the caller
+    accumulates the saved states) against the brute force on the whole sequence."""
+    f, hh, ww = 3, 2, 2
+    P = hh * ww
+    m, x, rot, (q, k, v), (C, N, heads) = _rope_case(O.CachedCausalAttention, d, f, hh, ww, seed=7)
+    acc = [None, None]
+    outs = []
+    for c in range(f):
+        cache = [acc[0], acc[1]]
+        o, cache = m(x[:, c * P:(c + 1) * P], rotary_emb=rot[:, :, c * P:(c + 1) * P], save_kv_cache=True,
+                     kv_cache=cache)
+        acc = [cache[0] if acc[0] is None else acc[0] + cache[0],
+               cache[1] if acc[1] is None else acc[1] + cache[1]]
+        outs.append(o)
+    chunk_of = np.repeat(np.arange(f, dtype=np.int32), P)
+    ref = _proj_of(cbrute.relu_attention_rope(q, k, v, rot[0, 0].numpy(), 1e-8, chunk_of), m, C, N, heads, d)
+    torch.testing.assert_close(torch.cat(outs, 1), ref, rtol=1e-9, atol=1e-11)
+
+
+def test_rotated_brute_force_reduces_to_the_plain_one_for_unit_factors():
+    rng = np.random.default_rng(0)
+    q, k, v = (rng.standard_normal((3, 10, 8)) for _ in range(3))
+    ones = np.ones((10, 4), dtype=np.complex128)
+    np.testing.assert_allclose(cbrute.relu_attention_rope(q, k, v, ones, 1e-8), cbrute.relu_attention(q, k, v, 1e-8),
+                               rtol=1e-13, atol=1e-14)
+    # a rotation common to all tokens leaves <rot k, rot q> unchanged (it is orthogonal): same answer
+    same = np.full((10, 4), np.exp(0.7j))
+    np.testing.assert_allclose(cbrute.relu_attention_rope(q, k, v, same, 1e-8), cbrute.relu_attention(q, k, v, 1e-8),
+                               rtol=1e-12, atol=1e-13)
+
+
 # ---------------------------------------------------------------- W8A16 quantiser
 
 
