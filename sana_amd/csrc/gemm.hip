@@ -846,17 +846,10 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(const float* __res
   *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
 }
 
-int compute_units() {
-  static int n = 0;  // same value from every thread that races here
-  if (n == 0) {
-    int dev = 0, cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
-      cu = 256;
-    n = cu;
-  }
-  return n;
-}
+// The library is built for one chip, MI355X: 256 compute units in 8 XCDs.  A constant (not a device query)
+// keeps the library free of global state and makes the plans -- and sana_hip_gemm_workspace_bytes -- the same on
+// every host, with or without a GPU.
+constexpr int compute_units() { return 256; }
 
 // Channel tile of the pipelined kernel (NI = 4: 256 channels, 3: 192).  One workgroup per compute unit at a
 // time, so the grid runs in rounds: the tile whose rounds x tile size is smaller wins; the narrower tile

@@ -521,17 +521,8 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   }
 }
 
-int compute_units112() {
-  static int n = 0;  // same value from every thread that races here
-  if (n == 0) {
-    int dev = 0, cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
-      cu = 256;
-    n = cu;
-  }
-  return n;
-}
+// MI355X: 256 compute units (a constant, so plans do not depend on the host the call is made on)
+constexpr int compute_units112() { return 256; }
 
 struct Plan112 {
   int nsplit, split_tokens;

@@ -15,6 +15,7 @@ Cross-attention, LayerNorm and the adaLN modulation use stock PyTorch-ROCm ops.
 """
 from __future__ import annotations
 
+import collections
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -138,6 +139,34 @@ def _rotary_real_tokens_(t: torch.Tensor, cos_sin) -> None:
     t.copy_((x.float() * cos + x_rot.float() * sin).to(t.dtype).reshape(B, N, C))
 
 
+# (cos, sin) tables derived from the callers' rotary_emb tensors, shared by all blocks of a model.  An entry keeps
+# its source tensor alive, so neither the tensor's id nor its storage address can be handed to another tensor while
+# the entry exists; the key names the memory the factors were read from and its version counter, so fresh views of
+# the same factors (a pipeline slicing one table per chunk, once per block) hit, and equal-shaped temporaries with
+# other contents miss.  Entries used while a HIP graph was being captured are never dropped: the graph holds the
+# table's address.
+_ROPE_TABLES: "collections.OrderedDict" = collections.OrderedDict()
+_ROPE_TABLE_LIMIT = 16
+
+
+def _rope_table_cached(rotary_emb: torch.Tensor, N: int, device, head_dim: int) -> torch.Tensor:
+    key = (rotary_emb.untyped_storage().data_ptr(), rotary_emb.storage_offset(), tuple(rotary_emb.shape),
+           tuple(rotary_emb.stride()), rotary_emb.dtype, rotary_emb.device, rotary_emb._version, N,
+           torch.device(device), head_dim)
+    capturing = rotary_emb.is_cuda and torch.cuda.is_current_stream_capturing()
+    entry = _ROPE_TABLES.get(key)
+    if entry is None:
+        entry = [rotary_emb, ops.rope_table(rotary_emb, N, device, head_dim=head_dim), capturing]
+        _ROPE_TABLES[key] = entry
+        if len(_ROPE_TABLES) > _ROPE_TABLE_LIMIT:
+            for old in [k for k, e in _ROPE_TABLES.items() if not e[2]][:len(_ROPE_TABLES) - _ROPE_TABLE_LIMIT]:
+                del _ROPE_TABLES[old]
+    else:
+        _ROPE_TABLES.move_to_end(key)
+        entry[2] = entry[2] or capturing
+    return entry[1]
+
+
 def _as_token_major(t: torch.Tensor, token_dim: int) -> torch.Tensor:
     """(B, h, d, N) [token_dim=3] or (B, h, N, d) [token_dim=2] -> [B, N, h*d] with
     unit channel stride, without a copy when the memory already is token-major."""
@@ -250,12 +279,7 @@ class LiteLA(nn.Module):
             raise NotImplementedError("qk-norm / rotary embedding inside the attention kernels is bf16 only")
         rope = None
         if rotary_emb is not None:
-            cache = self.__dict__.get("_rope_cache")
-            key = (id(rotary_emb), rotary_emb._version, N, qkv.device)
-            if cache is None or cache[0] != key:
-                cache = (key, ops.rope_table(rotary_emb, N, qkv.device, head_dim=self.dim))
-                self.__dict__["_rope_cache"] = cache
-            rope = cache[1]
+            rope = _rope_table_cached(rotary_emb, N, qkv.device, self.dim)
         if norm:
             if self.q_norm.eps != self.k_norm.eps:
                 raise NotImplementedError("q_norm and k_norm with different eps")

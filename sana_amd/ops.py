@@ -16,10 +16,12 @@ _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 HEAD_DIM = 32
 HEAD_DIMS = (32, 112)   # head dims with kernels: 32 (all dtypes), 112 (bf16; the video configurations)
 
-# One scratch buffer per device, grown on demand and shared by every call on that device (attention partial
-# states, split-k planes): calls are ordered by the stream they run on, so launching from two streams at once
-# on one device needs one process (or one copy of this module) per stream.
-_workspaces = {}     # (device index) -> uint8 tensor
+# Scratch buffers (attention partial states, split-k planes): one per (device, stream), so calls on different
+# streams never share scratch memory; calls on one stream are ordered by it.  A buffer that has become too small
+# is RETIRED, never freed: a captured HIP graph (or work still queued) may hold its address, and the allocator
+# would hand freed memory to the next tensor.  Sizes grow in powers of two, so everything retired on a stream is
+# smaller than its current buffer.
+_workspaces = {}     # (device index, raw stream handle) -> list of uint8 tensors, the last one current
 _chunk_tables = {}   # (device index, tuple) -> int32 tensor
 _CACHE_LIMIT = 256   # small derived device tensors (chunk tables, frame flags) kept per process
 
@@ -52,15 +54,19 @@ def _need_cuda(*ts: torch.Tensor) -> None:
             raise SanaHipError("the HIP kernels need device tensors (no CPU path exists)")
 
 
-def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     if nbytes == 0:
         return None
-    key = device.index
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    key = (device.index, _stream() if stream is None else stream)
+    bufs = _workspaces.get(key)
+    if bufs is None:
+        bufs = _workspaces[key] = []
+    if not bufs or bufs[-1].numel() < nbytes:
+        size = 1 << 20
+        while size < nbytes:
+            size <<= 1
+        bufs.append(torch.empty(size, dtype=torch.uint8, device=device))   # earlier ones stay alive in the list
+    return bufs[-1]
 
 
 def chunk_table(chunk_tokens: Optional[Sequence[int]], N: int, device) -> Tuple[Optional[torch.Tensor], int, int]:

@@ -126,3 +126,37 @@ def test_w8_state_keys():
         assert base + ".weight_q" in keys and base + ".weight_scale" in keys
     assert blk.state_dict()["attn.qkv.weight_q"].dtype == torch.int8
     assert "cross_attn.q_linear.weight" in keys and "mlp.depth_conv.conv.weight" in keys
+
+
+def test_rope_tables_of_equal_shaped_temporaries_are_never_confused():
+    """Streaming callers pass a fresh slice of the rotary factors per chunk: equal shape, other angles, and
+    CPython hands a freed temporary's id to the next one.  The (cos, sin) table a module derives must follow
+    the CONTENT: 20 blocks x 8 equal chunks, plus two whole videos of one length with different factors."""
+    from sana_amd import modules as M
+    from sana_amd import ops
+
+    d, n_chunk, n_chunks = 32, 12, 8
+    blocks = [S.LiteLAReLURope(64, 64, dim=d) for _ in range(20)]
+    qkv = torch.zeros(1, n_chunk, 3, 64, dtype=torch.bfloat16)
+
+    def factors(seed, n):
+        theta = torch.rand(n, d // 2, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * 6.0
+        return torch.polar(torch.ones_like(theta), theta)[None, None]
+
+    whole = factors(0, n_chunk * n_chunks)
+    for c in range(n_chunks):
+        for blk in blocks:
+            rot = whole[:, :, c * n_chunk:(c + 1) * n_chunk]          # a fresh view object per block and chunk
+            table = blk._pre(qkv, rot)[0].rope
+            assert torch.equal(table, ops.rope_table(rot, n_chunk, "cpu", head_dim=d)), (c,)
+    for seed in range(1, 40):                                          # temporaries that die between the calls
+        rot = factors(seed, n_chunk)
+        want = ops.rope_table(rot, n_chunk, "cpu", head_dim=d)
+        assert torch.equal(blocks[seed % 20]._pre(qkv, rot)[0].rope, want), seed
+        del rot
+    # an in-place update of a held tensor is seen (version counter), and the table store stays bounded
+    rot = factors(99, n_chunk)
+    first = blocks[0]._pre(qkv, rot)[0].rope.clone()
+    rot.mul_(-1)
+    assert torch.equal(blocks[0]._pre(qkv, rot)[0].rope, -first)
+    assert len(M._ROPE_TABLES) <= M._ROPE_TABLE_LIMIT
