@@ -4,7 +4,9 @@
  * Conventions
  *   - Every pointer is a DEVICE pointer unless the comment says "host".
  *   - The caller owns every buffer.  The library allocates nothing and keeps
- *     no global state; scratch space is passed in as `workspace`.
+ *     no global state; scratch space is passed in as `workspace`.  (The one
+ *     exception is sana_hip_linattn_state_noalloc, whose scratch is a fixed
+ *     array inside the library image.)
  *   - All work is enqueued on `stream` (a hipStream_t passed as void*; NULL is
  *     the default stream).  No entry point synchronises with the host.
  *   - Return value: SANA_OK (0) or a negative SANA_ERR_* code.  Nothing is
@@ -29,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 4
+#define SANA_HIP_ABI_VERSION 5
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -44,6 +46,8 @@ extern "C" {
 #define SANA_ERR_WORKSPACE (-4)  /* workspace missing or too small                 */
 #define SANA_ERR_LAUNCH (-5)     /* hipLaunchKernel reported an error              */
 #define SANA_ERR_DTYPE (-6)      /* dtype not supported by this entry point        */
+#define SANA_ERR_SCRATCH_LIMIT (-7) /* needs more than SANA_HIP_NOALLOC_SCRATCH_BYTES */
+#define SANA_ERR_RUNTIME (-8)    /* a HIP runtime call (device / symbol lookup) failed */
 
 /* GEMM epilogues */
 #define SANA_EPI_NONE 0       /* C = A W^T                       */
@@ -158,6 +162,32 @@ int sana_hip_linattn_apply_pre(const void* q, const float* state, void* out,
                                float eps, int io_dtype, int out_dtype,
                                const float* q_rinv, const void* q_weight, const float* rope,
                                void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Phase 1 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ *
+ * Same computation, arguments and result as sana_hip_linattn_state_pre (with k_rinv, k_weight and rope NULL: as
+ * sana_hip_linattn_state), but there is no workspace argument: the per-split partial states go to a fixed
+ * SANA_HIP_NOALLOC_SCRATCH_BYTES array of device memory that is part of the library image (every GPU the library
+ * runs on holds its own copy until the process ends).  The call allocates and frees nothing.
+ *   - A problem whose sana_hip_linattn_workspace_bytes(...) exceeds SANA_HIP_NOALLOC_SCRATCH_BYTES returns
+ *     SANA_ERR_SCRATCH_LIMIT and launches nothing (the block shapes of the benchmark configurations need
+ *     7.3 - 20.3 MiB).
+ *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+ *     threads) race.  Calls on one stream are ordered and safe.  Old contents never reach a result.
+ *   - The first call on each device resolves the array's address (hipGetSymbolAddress, once per device, the
+ *     device being current); make that call outside graph capture.  SANA_ERR_RUNTIME if the lookup fails.
+ */
+#define SANA_HIP_NOALLOC_SCRATCH_BYTES (24u << 20)
+
+int sana_hip_linattn_state_noalloc(const void* k, const void* v, float* state,
+                                   int B, int N, int h, int d,
+                                   int64_t stride_b, int64_t stride_n,
+                                   const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
+                                   int causal, int io_dtype,
+                                   const float* k_rinv, const void* k_weight, const float* rope,
+                                   void* stream);
 
 /* ---------------------------------------------------------------------------
  * Depthwise 3x3 conv (zero pad 1, stride 1) + bias + SiLU gate, channels-last

@@ -33,6 +33,10 @@ SIGNATURES = {
                                            c_int, c_int, c_int, c_int, c_int64, c_int64,
                                            c_void_p, c_int, c_int, c_int, c_int,
                                            c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sana_hip_linattn_state_noalloc": (c_int, [c_void_p, c_void_p, c_void_p,
+                                               c_int, c_int, c_int, c_int, c_int64, c_int64,
+                                               c_void_p, c_int, c_int, c_int, c_int,
+                                               c_void_p, c_void_p, c_void_p, c_void_p]),
     "sana_hip_linattn_apply_pre": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                            c_int64, c_int64, c_int64, c_int64,
                                            c_void_p, c_int, c_int, c_float, c_int, c_int,

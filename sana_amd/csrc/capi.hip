@@ -12,6 +12,8 @@ extern "C" __attribute__((visibility("default"))) const char* sana_hip_strerror(
     case SANA_ERR_WORKSPACE: return "workspace missing or too small";
     case SANA_ERR_LAUNCH: return "kernel launch failed";
     case SANA_ERR_DTYPE: return "dtype not supported by this entry point";
+    case SANA_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's fixed array holds (use the workspace entry point)";
+    case SANA_ERR_RUNTIME: return "HIP runtime call failed (no current device, or the scratch symbol could not be resolved)";
     default: return "unknown error code";
   }
 }

@@ -17,6 +17,8 @@
 //            applied with MFMA 16x16x32; rows 32..47 of the A operand all carry
 //            ksum so every lane gets its token's denominator in-lane.
 // fp32 io (and f16 phase 2) uses MFMA 32x32x2 f32 directly from global memory.
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -697,6 +699,54 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state_pre
   const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope};
   return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, chunk_starts, n_chunks,
                     max_chunk_tokens, causal, io_dtype, pre, stream);
+}
+
+// ---------------------------------------------------------------------------- phase 1 without a workspace argument
+// For callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid it): the
+// per-split partial states go to a fixed array in device memory instead of a caller-provided workspace.  Each GPU
+// the library runs on holds its own copy of the array, at its own address, until the process ends.  `scratch` is a
+// host-side stand-in for that symbol, not a device address: host code uses the address hipGetSymbolAddress returns
+// for the current device and never the array's name.
+static __device__ __align__(256) unsigned char scratch[SANA_HIP_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_addr[kMaxDevices];  // device address of `scratch` per GPU, looked up once per device
+std::mutex g_scratch_mutex;
+
+// The current device's copy of the array, or null when the runtime refuses the lookup.
+void* scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  p = g_scratch_addr[dev].load(std::memory_order_relaxed);
+  if (!p) {
+    void* addr = nullptr;
+    if (hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)) != hipSuccess || !addr) return nullptr;
+    g_scratch_addr[dev].store(addr, std::memory_order_release);
+    p = addr;
+  }
+  return p;
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state_noalloc(
+    const void* k, const void* v, float* state, int B, int N, int h, int d, int64_t stride_b, int64_t stride_n,
+    const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens, int causal, int io_dtype, const float* k_rinv,
+    const void* k_weight, const float* rope, void* stream) {
+  if (B <= 0 || N <= 0 || h <= 0 || n_chunks <= 0) return SANA_ERR_ARG;
+  const int longest = (n_chunks == 1 && !chunk_starts) ? N : max_chunk_tokens;
+  const size_t need = sana_hip_linattn_workspace_bytes(B, h, d, n_chunks, longest, io_dtype);
+  if (need > (size_t)SANA_HIP_NOALLOC_SCRATCH_BYTES) return SANA_ERR_SCRATCH_LIMIT;
+  void* ws = scratch_of_current_device();
+  if (!ws) return SANA_ERR_RUNTIME;
+  // every partial state the reduction reads is written by the launch before it (empty splits write zeros), so the
+  // array's old contents never reach a result and nothing has to be cleared
+  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope};
+  return state_impl(k, v, state, ws, (size_t)SANA_HIP_NOALLOC_SCRATCH_BYTES, B, N, h, d, stride_b, stride_n,
+                    chunk_starts, n_chunks, max_chunk_tokens, causal, io_dtype, pre, stream);
 }
 
 extern "C" __attribute__((visibility("default"))) int sana_hip_qk_rms(const void* q, const void* k, float* q_rinv,

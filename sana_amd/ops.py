@@ -156,12 +156,19 @@ def _head_dim(d: int) -> int:
     return d
 
 
+NOALLOC_SCRATCH_BYTES = 24 << 20   # SANA_HIP_NOALLOC_SCRATCH_BYTES of include/sana_hip.h
+
+
 def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False,
-                  pre: Optional[QkPre] = None, head_dim: int = HEAD_DIM) -> torch.Tensor:
+                  pre: Optional[QkPre] = None, head_dim: int = HEAD_DIM, out: Optional[torch.Tensor] = None,
+                  noalloc: bool = False) -> torch.Tensor:
     """Phase 1.  k, v: [B, N, C] token-major views (C = h*d).  Returns the fp32
-    state [B, h, n_chunks, d+1, d] (inclusive prefix over chunks when causal)."""
+    state [B, h, n_chunks, d+1, d] (inclusive prefix over chunks when causal).
+    ``out``: a state tensor to fill instead of a new one.  ``noalloc``: the partial states go to the library's
+    fixed per-GPU scratch array instead of a torch workspace (``sana_hip_linattn_state_noalloc``: with ``out``
+    given, nothing is allocated; problems beyond NOALLOC_SCRATCH_BYTES raise)."""
     d = _head_dim(head_dim)
-    _need_cuda(k, v)
+    _need_cuda(k, v, out)
     same = all(a == b or n == 1 for a, b, n in zip(k.stride(), v.stride(), k.shape))
     if k.shape != v.shape or k.dtype != v.dtype or not same:
         raise SanaHipError("k and v must share shape, dtype and strides")
@@ -172,20 +179,31 @@ def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: b
     sb, sn = _token_major_view(k, "k")
     tab, n_chunks, longest = chunk_table(chunk_tokens, N, k.device)
     lib = _lib.load()
-    state = torch.empty(B, h, n_chunks, d + 1, d, dtype=torch.float32, device=k.device)
+    if out is None:
+        state = torch.empty(B, h, n_chunks, d + 1, d, dtype=torch.float32, device=k.device)
+    else:
+        state = out
+        if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape) != (B, h, n_chunks, d + 1, d):
+            raise SanaHipError(f"out must be contiguous fp32 {(B, h, n_chunks, d + 1, d)}")
     if B * N == 0:
         if pre is not None:
             pre.check(k, d)
         return state.zero_()
+    shape = (B, N, h, d, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
+             1 if causal else 0, _dt(k))
+    pre_args = pre.check(k, d) if pre is not None else (None, None, None)
+    if noalloc:
+        code = lib.sana_hip_linattn_state_noalloc(k.data_ptr(), v.data_ptr(), state.data_ptr(), *shape, *pre_args,
+                                                  _stream())
+        _lib.check(code, "sana_hip_linattn_state_noalloc")
+        return state
     nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, d, n_chunks, longest, _dt(k))
     ws = _workspace(k.device, nbytes)
-    args = (k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes,
-            B, N, h, d, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
-            1 if causal else 0, _dt(k))
+    args = (k.data_ptr(), v.data_ptr(), state.data_ptr(), ws.data_ptr() if ws is not None else None, nbytes, *shape)
     if pre is None:
         code = lib.sana_hip_linattn_state(*args, _stream())
     else:
-        code = lib.sana_hip_linattn_state_pre(*args, *pre.check(k, d), _stream())
+        code = lib.sana_hip_linattn_state_pre(*args, *pre_args, _stream())
     _lib.check(code, "sana_hip_linattn_state")
     return state
 
