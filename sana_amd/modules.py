@@ -9,13 +9,20 @@ Same constructor arguments, forward signatures, attribute names and
   ``SanaMSBlock``          diffusion/model/nets/sana_multi_scale.py:54-157
 
 Forward only (inference).  The modules run on a GPU through ``libsana_hip.so``;
-there is no CPU path and no silent fallback: a configuration the kernels do
-not cover raises ``NotImplementedError`` at construction or call time.
-Cross-attention, LayerNorm and the adaLN modulation use stock PyTorch-ROCm ops.
+there is no CPU path: a configuration the kernels do not cover raises
+``NotImplementedError`` at construction or call time.  Cross-attention is stock
+PyTorch-ROCm ops by design.  A few options keep the HIP attention / depthwise
+kernels but take a stock op for one stage (fp16 / fp32 models: library GEMM for the
+linears; the real-valued pre-ReLU rotary embedding of ``LiteLA``; the temporal
+conv with a frame mask, C % 64 != 0 or a dtype other than bf16; the unfused
+LayerNorm / modulate / gate / residual seams outside bf16 inference).  Each of
+those logs one line per process and reason on the ``sana_amd`` logger
+(:func:`stock_path`), so nothing leaves the fast path silently.
 """
 from __future__ import annotations
 
 import collections
+import logging
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -26,6 +33,19 @@ from . import ops
 from ._lib import SanaHipError
 
 HEAD_DIM = ops.HEAD_DIM
+
+log = logging.getLogger("sana_amd")
+_stock_paths_seen = set()
+
+
+def stock_path(where: str, why: str) -> None:
+    """Record that ``where`` runs a stock PyTorch op instead of a kernel of this library because of ``why``:
+    one warning per (where, why) and process."""
+    key = (where, why)
+    if key not in _stock_paths_seen:
+        _stock_paths_seen.add(key)
+        log.warning("sana_amd: %s runs on stock PyTorch ops: %s", where, why)
+
 
 
 def _no_grad_only(*tensors):
@@ -69,9 +89,13 @@ def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None,
     lead = x.shape[:-1]
     K = x.shape[-1]
     if gate is not None:
-        if x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 3 and epilogue is None:
+        if x.dtype == torch.bfloat16 and gate.dtype == x.dtype and residual.dtype == x.dtype and x.is_cuda \
+                and x.dim() == 3 and epilogue is None:
             w = weight_q if weight_q is not None else weight
             return ops.gemm_gate_residual(x, w, bias, gate, residual, weight_scale if weight_q is not None else None)
+        stock_path("gated residual behind a linear", f"the fused epilogue needs bf16 [B, N, C] device input, gate and "
+                   f"residual and no activation; got x {x.dtype} {x.dim()}-d, gate {gate.dtype}, residual "
+                   f"{residual.dtype}, epilogue {epilogue!r}")
         return residual + gate * hip_linear(x, weight, bias, epilogue, weight_q, weight_scale)
     if x.dtype == torch.bfloat16 and x.is_cuda:
         x2 = x.reshape(-1, K)
@@ -91,6 +115,7 @@ def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None,
     if weight_q is not None:
         raise SanaHipError("W8A16 needs bf16 activations")
     # fp16 / fp32 models: plain library GEMM (hipBLASLt), activation as a stock op
+    stock_path("linear / 1x1 conv", f"the hand-written GEMM is bf16 only, input is {x.dtype} (library GEMM instead)")
     y = F.linear(x, weight.reshape(weight.shape[0], -1), bias)
     return F.silu(y) if epilogue == "silu" else y
 
@@ -234,9 +259,13 @@ class LiteLA(nn.Module):
         B, N, C = x.shape
         qkv = self.qkv(x).view(B, N, 3, C)
         if not isinstance(self.q_norm, nn.Identity):
+            stock_path("LiteLA q/k RMSNorm", "in-kernel norm is the bf16 path without image_rotary_emb; "
+                       f"got {x.dtype}, rotary_emb {'given' if rotary_emb is not None else 'absent'}")
             qkv[:, :, 0].copy_(self.q_norm(qkv[:, :, 0]))
             qkv[:, :, 1].copy_(self.k_norm(qkv[:, :, 1]))
         if rotary_emb is not None:
+            stock_path("LiteLA rotary embedding", "the real-valued pre-ReLU rotation of LiteLA.forward "
+                       "(sana_blocks.py:282-284) has no kernel; applied in place on the qkv buffer")
             _rotary_real_tokens_(qkv[:, :, 0], rotary_emb)
             _rotary_real_tokens_(qkv[:, :, 1], rotary_emb)
         return qkv
@@ -534,6 +563,15 @@ class GLUMBConvTemp(GLUMBConv):
                 and self.t_conv.kernel_size == (3, 1) and self.t_conv.in_channels == C and C % 64 == 0
                 and kwargs.get("frame_valid_mask") is None and not torch.is_grad_enabled())
 
+    def _tconv_stock_note(self, x: torch.Tensor, kwargs) -> None:
+        C = self.t_conv.out_channels
+        why = ("a frame_valid_mask is given" if kwargs.get("frame_valid_mask") is not None else
+               f"dtype {x.dtype} (the GEMM is bf16)" if x.dtype != torch.bfloat16 or self.t_conv.weight.dtype != torch.bfloat16 else
+               f"C = {C} is not a multiple of 64" if C % 64 else
+               f"kernel {tuple(self.t_conv.kernel_size)} is not (3, 1)" if self.t_conv.kernel_size != (3, 1) else
+               "autograd is enabled" if torch.is_grad_enabled() else "input is not on the GPU")
+        stock_path(f"{type(self).__name__} temporal conv", why + " (stock convolution instead of the tap GEMM)")
+
     def _tconv_weight(self) -> torch.Tensor:
         """t_conv.weight [C, C, t, 1] -> [C, t*C] with k = tap * C + input channel (derived data, rebuilt when
         the parameter changes; not part of the state_dict)."""
@@ -586,6 +624,7 @@ class GLUMBConvTemp(GLUMBConv):
         if self._tconv_gemm_ok(x, kwargs):
             buf = self._spatial_into_frames(x, HW)
             return self._tconv_residual(buf, HW, [0, HW[0]])
+        self._tconv_stock_note(x, kwargs)
         xr = self._spatial_bcthw(x, HW)
         frame_mask = kwargs.get("frame_valid_mask", None)
         if frame_mask is not None:
@@ -609,6 +648,7 @@ class ChunkGLUMBConvTemp(GLUMBConvTemp):
             buf = self._spatial_into_frames(x, HW)
             T = HW[0]
             return self._tconv_residual(buf, HW, sorted({0, *(int(i) for i in chunk_index if 0 < int(i) < T), T}))
+        self._tconv_stock_note(x, kwargs)
         xr = self._spatial_bcthw(x, HW)
         T = HW[0]
         frame_mask = kwargs.get("frame_valid_mask")
@@ -646,6 +686,7 @@ class CachedGLUMBConvTemp(GLUMBConvTemp):
                     kv_cache[-1] = buf[:, T * P:].transpose(1, 2).unsqueeze(2).detach().clone()
             out = self._tconv_residual(buf, HW, [0, T], left)
             return (out, kv_cache) if kv_cache is not None else out
+        self._tconv_stock_note(x, kwargs)
         xr = self._spatial_bcthw(x, HW)
         pad = self.t_conv.kernel_size[0] // 2
         x_in, padded = xr, 0
@@ -815,7 +856,10 @@ class SanaMSBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
             self.scale_shift_table[None] + t.reshape(B, 6, -1)
         ).chunk(6, dim=1)
-        if x.is_cuda and x.dtype == torch.bfloat16 and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
+        # (conditioning in another dtype than x -- an fp32 t with a bf16 x -- promotes in the stock op chain; the
+        # fused kernels read the modulation rows as x's dtype, so that case takes the stock composition below)
+        if x.is_cuda and x.dtype == torch.bfloat16 and shift_msa.dtype == x.dtype and C % 8 == 0 and C <= 8192 \
+                and not torch.is_grad_enabled():
             # fused seams: LayerNorm + modulate in one kernel, gate * out + residual in the GEMM epilogue
             h = ops.layernorm_modulate(x, scale_msa, shift_msa, self.norm1.eps)
             if "forward" in self.attn.__dict__:
@@ -826,6 +870,9 @@ class SanaMSBlock(nn.Module):
             # the cross-attention's residual add and norm2 + modulate in one pass
             x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask), scale_mlp, shift_mlp, self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)
+        stock_path("SanaMSBlock LayerNorm / modulate / gate / residual seams",
+                   f"the fused seams are bf16 inference only (C % 8 == 0, C <= 8192); got x {x.dtype}, t {t.dtype}, C = {C}, "
+                   f"grad {'on' if torch.is_grad_enabled() else 'off'}")
         x = x + self.drop_path(
             gate_msa * self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), HW=HW, rotary_emb=image_rotary_emb))
         x = x + self.cross_attn(x, y, mask)
@@ -898,10 +945,12 @@ class SanaVideoMSBlock(nn.Module):
     @staticmethod
     def _gate_residual(x, gate, y):
         """x + gate * y (gate [B, 1, C] or per frame [B, F, 1, C]); one fused pass on the bf16 device path."""
-        if x.is_cuda and x.dtype == torch.bfloat16 and y.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 \
-                and not torch.is_grad_enabled():
+        if x.is_cuda and x.dtype == torch.bfloat16 and y.dtype == torch.bfloat16 and gate.dtype == torch.bfloat16 \
+                and x.shape[-1] % 8 == 0 and not torch.is_grad_enabled():
             return ops.gate_residual(y, gate, x)
         B, N, C = x.shape
+        stock_path("SanaVideoMSBlock gate / residual", f"the fused pass is bf16 inference only; got {x.dtype} / {y.dtype}, "
+                   f"C = {C}, grad {'on' if torch.is_grad_enabled() else 'off'}")
         if gate.dim() == 4:
             return x + (gate * y.reshape(B, gate.shape[1], -1, C)).reshape(B, N, C)
         return x + gate * y
@@ -910,10 +959,13 @@ class SanaVideoMSBlock(nn.Module):
         """t2i_modulate(norm(x), shift, scale) with ``groups`` modulation rows per batch entry (1, or one per
         frame): shift / scale are [B, groups, 1, C] or [B, 1, C]."""
         B, N, C = x.shape
-        if x.is_cuda and x.dtype == torch.bfloat16 and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
+        if x.is_cuda and x.dtype == torch.bfloat16 and scale.dtype == x.dtype and shift.dtype == x.dtype \
+                and C % 8 == 0 and C <= 8192 and not torch.is_grad_enabled():
             h = ops.layernorm_modulate(x.reshape(B * groups, N // groups, C), scale.reshape(B * groups, 1, C),
                                        shift.reshape(B * groups, 1, C), norm.eps)
             return h.view(B, N, C)
+        stock_path("SanaVideoMSBlock LayerNorm / modulate", f"the fused kernel is bf16 inference only (C % 8 == 0, "
+                   f"C <= 8192); got {x.dtype}, C = {C}, grad {'on' if torch.is_grad_enabled() else 'off'}")
         if groups == 1:
             return t2i_modulate(norm(x), shift, scale)
         return t2i_modulate(norm(x).reshape(B, groups, -1, C), shift, scale).reshape(B, N, C)

@@ -381,6 +381,8 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
     epi = _EPI[epilogue]
     if bias is not None and epi == _lib.EPI_NONE:
         epi = _lib.EPI_BIAS
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
+        raise SanaHipError("bias must be contiguous bf16 [N]")
     if out is None:
         out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
     out, ldc = _rows(out, "out")
@@ -399,8 +401,10 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
 
 # --------------------------------------------------------------------------- fused seams of the block
 
-def _mod_rows(t: torch.Tensor, B: int, C: int, what: str) -> Tuple[torch.Tensor, int]:
+def _mod_rows(t: torch.Tensor, B: int, C: int, what: str, dtype=torch.bfloat16) -> Tuple[torch.Tensor, int]:
     """Per-batch row vectors [B, 1, C] / [B, C] with unit inner stride -> (tensor, batch stride)."""
+    if t.dtype != dtype:     # the kernels read these rows as 16-bit values: another dtype would be misread
+        raise SanaHipError(f"{what} must be {dtype} like the activations, got {t.dtype}")
     if t.dim() == 3 and t.shape[1] == 1:
         t = t[:, 0]
     if t.dim() != 2 or t.shape != (B, C) or t.stride(1) != 1:
@@ -420,6 +424,15 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     C = weight.shape[0]
     if a.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or gate.dtype != torch.bfloat16:
         raise SanaHipError("gemm_gate_residual is bf16 only")
+    if weight_scale is None and weight.dtype != torch.bfloat16:
+        raise SanaHipError(f"weight must be bf16 (or int8 together with weight_scale), got {weight.dtype}")
+    if weight_scale is not None and (weight.dtype != torch.int8 or weight_scale.dtype != torch.float32
+                                     or weight_scale.numel() != C or not weight_scale.is_contiguous()):
+        raise SanaHipError("W8A16 needs an int8 weight and contiguous fp32 scales, one per output channel")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != C or not bias.is_contiguous()):
+        raise SanaHipError("bias must be contiguous bf16 [C]")
+    if weight.reshape(C, -1).shape[1] != K:
+        raise SanaHipError(f"K mismatch: a {tuple(a.shape)} vs weight {tuple(weight.shape)}")
     a2, lda = _rows(a.reshape(B * Ntok, K), "a")
     w2, ldw = _rows(weight.reshape(C, -1), "weight")
     r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
@@ -497,8 +510,8 @@ def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor
     _need_cuda(x, scale, shift)
     B, Ntok, C = x.shape
     x2, ldx = _rows(x.reshape(B * Ntok, C), "x")
-    sc, s1 = _mod_rows(scale, B, C, "scale")
-    sh, s2 = _mod_rows(shift, B, C, "shift")
+    sc, s1 = _mod_rows(scale, B, C, "scale", x.dtype)
+    sh, s2 = _mod_rows(shift, B, C, "shift", x.dtype)
     if s1 != s2:
         raise SanaHipError("scale and shift must share their batch stride")
     out = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)
@@ -519,8 +532,8 @@ def add_layernorm_modulate(x: torch.Tensor, y: torch.Tensor, scale: torch.Tensor
     B, Ntok, C = x.shape
     x2, ldx = _rows(x.reshape(B * Ntok, C), "x")
     y2, ldy = _rows(y.reshape(B * Ntok, C), "y")
-    sc, s1 = _mod_rows(scale, B, C, "scale")
-    sh, s2 = _mod_rows(shift, B, C, "shift")
+    sc, s1 = _mod_rows(scale, B, C, "scale", x.dtype)
+    sh, s2 = _mod_rows(shift, B, C, "shift", x.dtype)
     if s1 != s2:
         raise SanaHipError("scale and shift must share their batch stride")
     total = torch.empty(B * Ntok, C, dtype=x.dtype, device=x.device)

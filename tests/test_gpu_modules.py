@@ -329,6 +329,79 @@ def test_block_replays_from_a_hip_graph(cuda):
         check(out, _ref64(ob, x.cpu(), y.cpu(), t.cpu(), HW=HW), "graph replay vs fp64 oracle", block=True)
 
 
+def test_graph_replay_survives_a_larger_eager_shape(cuda):
+    """A captured block holds the raw addresses of the scratch buffers it used (attention partial states, split-k
+    planes).  A later, larger eager call makes the library take bigger buffers; the captured ones must stay alive
+    and untouched by the allocator, so a replay still reproduces the eager result bit for bit."""
+    from sana_amd import ops
+    C, heads = 2240, 20
+    hb = S.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").bfloat16()
+    hb.load_state_dict(O.init_block_(O.SanaMSBlock(C, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv"),
+                                     8).bfloat16().state_dict())
+    hb = hb.to(cuda)
+    small, big = (32, 32), (64, 64)
+    x, y, t = (a.bfloat16().to(cuda) for a in O.block_inputs(1, small[0] * small[1], C, seed=8))
+    xb, yb, tb = (a.bfloat16().to(cuda) for a in O.block_inputs(2, big[0] * big[1], C, seed=9))
+    lib = ops._lib.load()
+    assert lib.sana_hip_linattn_workspace_bytes(1, C // 32, 32, 1, 1024, 1) > 0       # both kinds of scratch are in play
+    assert lib.sana_hip_gemm_workspace_bytes(1024, C, 5600) > 0
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                hb(x, y, t, HW=small)
+        torch.cuda.current_stream().wait_stream(side)
+        want = hb(x, y, t, HW=small).clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = hb(x, y, t, HW=small)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        held = sum(len(v) for v in ops._workspaces.values())
+        for r in range(3):
+            hb(xb, yb, tb, HW=big)                    # larger scratch on the eager stream
+            junk = [torch.full((1 << 22,), float(r), device=cuda) for _ in range(8)]   # takes whatever was freed
+            torch.cuda.synchronize()
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), f"replay {r} after a larger eager call"
+            del junk
+        assert sum(len(v) for v in ops._workspaces.values()) >= held   # nothing the graph may point at was dropped
+
+
+def test_conditioning_in_another_dtype_is_never_misread(cuda):
+    """t in fp32 with a bf16 x: the stock op chain promotes (scale_shift_table + t is fp32) and then fails in its
+    first linear, as the reference does; the fused kernels would misread the fp32 rows as bf16 and return garbage.
+    The block must end in an error, not a result, and the op wrappers themselves refuse such rows."""
+    from sana_amd import ops
+    from sana_amd._lib import SanaHipError
+    C, heads, B, HW = 96, 4, 2, (8, 12)
+    ob, hb = _pair(C, heads, seed=6)
+    hb = hb.to(cuda)
+    x, y, t = O.block_inputs(B, HW[0] * HW[1], C, n_text=16, seed=6)
+    x, y = x.bfloat16(), y.bfloat16()
+    with torch.no_grad():
+        with pytest.raises(RuntimeError):
+            hb(x.to(cuda), y.to(cuda), t.to(cuda), HW=HW)       # t stays fp32
+        with pytest.raises(RuntimeError):
+            ob(x, y, t, HW=HW)                                  # the stock composition fails the same way
+    xd = x.to(cuda)
+    rows32 = torch.zeros(B, 1, C, device=cuda)
+    with pytest.raises(SanaHipError):
+        ops.layernorm_modulate(xd, rows32, rows32)
+    w = torch.zeros(C, C, dtype=torch.bfloat16, device=cuda)
+    g16 = torch.zeros(B, 1, C, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(SanaHipError):
+        ops.gemm_gate_residual(xd, w, torch.zeros(C, device=cuda), g16, xd)                   # fp32 bias
+    with pytest.raises(SanaHipError):
+        ops.gemm_gate_residual(xd, w.to(torch.int8), None, g16, xd)                           # int8 weight, no scale
+    with pytest.raises(SanaHipError):
+        ops.gemm_gate_residual(xd, w, None, rows32, xd)                                       # fp32 gate
+
+
 def test_four_images_at_the_full_shape_equal_one_at_a_time(cuda):
     """B = 4 at the cfg3 shape (65536 tokens x 2240 channels, 4x the benchmark size: 1.5 GB hidden activation, row
     offsets past 2^31 bytes): images do not interact, so the batched block must reproduce the per-image calls --
