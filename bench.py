@@ -23,8 +23,11 @@ launch stream:
 ``--kernels-only`` runs just the per-kernel section (the command the rocprofv3
 summaries under profiles/ were taken with).  ``roofline.traffic`` is not
 measurable from inside the process: it is the HBM byte count of one launch of
-the dominant kernel from two ``rocprofv3 --pmc`` runs of that command
-(FETCH_SIZE, WRITE_SIZE), copied here from profiles/kernels_cfg3_hbm_traffic.txt.
+the dominant kernel from two ``rocprofv3 --pmc`` runs of ``--kernels-only --cfg3-only``
+(FETCH_SIZE, WRITE_SIZE), read at run time from profiles/kernels_cfg3_hbm_traffic.txt.
+``configs`` holds the two small configurations of the benchmark definition beside the
+headline: cfg1 (the LiteLA op alone, fp32, eps 1e-15) and cfg2 (one Sana-600M block,
+B=4), each with the oracle timed on the host cores.
 """
 from __future__ import annotations
 
@@ -40,9 +43,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of the dominant kernel (inverted-conv GEMM at cfg3), from the pmc summary
-# profiles/kernels_cfg3_hbm_traffic.txt: FETCH_SIZE x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE x 1.0.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 1640357273  # 1274.8 MB read + 367.0 MB written
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "kernels_cfg3_hbm_traffic.txt")
+DOMINANT_KERNEL_ROW = "gemm4_kernel<false, 2, 4>"   # the inverted-conv GEMM (bias + SiLU epilogue, 256-wide channel tile)
+
+
+def dominant_kernel_traffic_bytes():
+    """HBM-side bytes per launch of the dominant kernel, read from the committed rocprofv3 --pmc summary (columns
+    read_MB and write_MB of its row: FETCH_SIZE / WRITE_SIZE scaled by what a plain copy of known size reads
+    on the same counters).  None when the summary or the row is missing."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith(DOMINANT_KERNEL_ROW):
+                cols = line[len(DOMINANT_KERNEL_ROW):].split()
+                return int(round((float(cols[1]) + float(cols[4])) * 1e6))   # read_MB + write_MB
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
+
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -109,7 +126,7 @@ def event_time_us(fn, iters: int, warmup: int, repeats: int = 3) -> float:
     return sorted(times)[len(times) // 2]
 
 
-def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
+def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False, cfg3_only=False):
     """Each hand-written kernel alone at the cfg3 shape (B=1, N=16384)."""
     from sana_amd import ops
 
@@ -135,6 +152,27 @@ def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
     add("linattn_apply", "hbm", la_bytes,
         event_time_us(lambda: ops.linattn_apply(q, state, 1e-8, out=out), iters, warmup),
         "M*C*2 B (Q read) + M*C*2 B (out write) + state read")
+    if not cfg3_only:
+        _kernel_rooflines_other_shapes(dev, add, qkv, state, out, la_bytes, g, iters, warmup)
+    _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_only)
+    # plain device copy as a bandwidth yardstick of this box
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    t_us = event_time_us(lambda: dst.copy_(src), 20, 5)
+    copy_gbs = 2 * src.numel() / t_us / 1e3
+    for r in rows:   # the HBM-bound rows once more against what a plain copy reaches on this box
+        if r["bound"] == "hbm":
+            r["frac_of_copy_rate"] = round(r["achieved"] / copy_gbs, 3)
+    return rows, round(copy_gbs, 1)
+
+
+def _kernel_rooflines_other_shapes(dev, add, qkv, state, out, la_bytes, g, iters, warmup):
+    """The attention phases with q/k norm + rotary embedding on load, the chunk-causal video shape and the
+    112-wide heads (skipped by --cfg3-only, so a counter run sees every template instance at one shape only)."""
+    from sana_amd import ops
+
+    B, N, M = 1, 16384, 16384
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
     # the same two phases with q/k RMSNorm and the rotary embedding applied on load (LiteLAReLURope), plus
     # the statistics pass they need; and the chunk-causal video shape (21 frames x 30x52 tokens, one chunk per frame)
     wn = (1 + 0.1 * torch.randn(C, generator=g)).bfloat16().to(dev)
@@ -200,6 +238,12 @@ def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
         event_time_us(lambda: ops.linattn_apply(qkv5[:, :, 0], st112c, 1e-8, starts, out=out5, pre=pq5), iters, warmup),
         "cfg5 with 112-wide heads: Q read + out write + 21 states + rope table + 1/rms")
     del qkv5, out5, st112, st112c, rope5
+
+
+def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_only):
+    from sana_amd import ops
+
+    B, N, M = 1, 16384, 16384
     u = torch.randn(B, 128, 128, 2 * HID, generator=g).bfloat16().to(dev)
     dw = (torch.randn(2 * HID, 1, 3, 3, generator=g) * 0.3).bfloat16().to(dev)
     db = torch.zeros(2 * HID, dtype=torch.bfloat16, device=dev)
@@ -237,6 +281,8 @@ def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
         t_lib = event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 20, 5)
         rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt, plain GEMM(+bias) of the same shape, for scale only
         del a, w, o
+    if cfg3_only:
+        return
     # temporal (3, 1) conv of the video Mix-FFN (GLUMBConvTemp) + its residual at the cfg5 frame grid, as one GEMM over
     # the token-major frames; the stock convolution on the reference's (B, C, T, HW) view beside it
     Tf, Pf = 21, 30 * 52
@@ -256,15 +302,6 @@ def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False):
             lambda: xr + torch.nn.functional.conv2d(xr, w4, padding=(1, 0)), 3, 1), 2)
         del xr
     del buf, ot
-    # plain device copy as a bandwidth yardstick of this box
-    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-    dst = torch.empty_like(src)
-    t_us = event_time_us(lambda: dst.copy_(src), 20, 5)
-    copy_gbs = 2 * src.numel() / t_us / 1e3
-    for r in rows:   # the HBM-bound rows once more against what a plain copy reaches on this box
-        if r["bound"] == "hbm":
-            r["frac_of_copy_rate"] = round(r["achieved"] / copy_gbs, 3)
-    return rows, round(copy_gbs, 1)
 
 
 def images_per_s(dev, w8: bool, steps: int, warmup: int, B: int = 16) -> float:
@@ -336,6 +373,68 @@ def cpu_baseline(iters: int = 5):
                       f"iterations after 1 warm-up; os.cpu_count()={os.cpu_count()}, cpu='{model}'"}
 
 
+def small_configs(dev):
+    """The two small configurations of the benchmark definition, GPU and host side by side.
+    cfg1: the LiteLA attention op alone (state + apply), fp32, B=1, 36 heads x 32, N=1024, q, k, v ~ N(0, 1), eps 1e-15;
+    host: the oracle's two-matmul form of the same op (LiteLA.attn_matmul), fp32.
+    cfg2: one SanaMSBlock at Sana-600M width, bf16, B=4, N=32x32, C=1152, hidden 2880, 300 text tokens;
+    host: the oracle block in fp32 (bf16 GEMM / conv on the host is neither fair nor stable)."""
+    import sana_amd as S
+    from oracle import sana_oracle as O
+    from sana_amd import ops
+
+    threads = torch.get_num_threads()
+    res = {}
+    # ---- cfg1
+    B, h, d, N = 1, 36, 32, 1024
+    g = torch.Generator().manual_seed(0)
+    qkv = torch.randn(B, N, 3, h * d, generator=g)
+    qd = qkv.to(dev)
+    out = torch.empty(B, N, h * d, device=dev)
+
+    def gpu_op():
+        st = ops.linattn_state(qd[:, :, 1], qd[:, :, 2])
+        ops.linattn_apply(qd[:, :, 0], st, 1e-15, out=out)
+
+    t_gpu = event_time_us(gpu_op, 200, 20)
+    q4, k4, v4 = (qkv[:, :, i].reshape(B, N, h, d).permute(0, 2, 3, 1) for i in range(3))   # (B, h, d, N) views
+    with torch.no_grad():
+        O.relu_linear_attention(q4, k4.transpose(-1, -2), v4, 1e-15)
+        t0 = time.perf_counter()
+        for _ in range(50):
+            O.relu_linear_attention(q4, k4.transpose(-1, -2), v4, 1e-15)
+        t_cpu = (time.perf_counter() - t0) / 50 * 1e6
+    bytes1 = 4 * N * h * d * 4 + 2 * h * (d + 1) * d * 4
+    res["cfg1"] = {"workload": "LiteLA ReLU linear attention op alone, fp32, B=1, 36 heads x 32, N=1024, eps 1e-15",
+                   "gpu_us": round(t_gpu, 2), "gpu_launches": 3, "algorithmic_bytes": bytes1,
+                   "achieved_GBps": round(bytes1 / t_gpu / 1e3, 1),
+                   "cpu_baseline": {"value": round(t_cpu, 1), "unit": "us per op", "cores": threads, "kind": "port",
+                                    "sample": "the whole workload, 50 timed iterations after 1 warm-up"},
+                   "note": "three launches of a few microseconds each: bound by launch latency, not by HBM"}
+    # ---- cfg2
+    Cc, heads, Bb, HW = 1152, 16, 4, (32, 32)
+    ob = O.init_block_(O.SanaMSBlock(Cc, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv"), 0)
+    ob.attn.fp32_attention = True
+    hb = S.SanaMSBlock(Cc, heads, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv").bfloat16()
+    hb.load_state_dict({k_: v_.bfloat16() for k_, v_ in ob.state_dict().items()})
+    hb = hb.to(dev)
+    x, y, t = O.block_inputs(Bb, HW[0] * HW[1], Cc, seed=2)
+    xd, yd, td = (a.bfloat16().to(dev) for a in (x, y, t))
+    with torch.no_grad():
+        t_gpu = event_time_us(lambda: hb(xd, yd, td, HW=HW), 50, 10)
+        ob(x, y, t, HW=HW)
+        t0 = time.perf_counter()
+        for _ in range(5):
+            ob(x, y, t, HW=HW)
+        t_cpu = (time.perf_counter() - t0) / 5 * 1e3
+    res["cfg2"] = {"workload": "one SanaMSBlock at Sana-600M width, bf16, B=4, N=32x32=1024, C=1152, hidden 2880, "
+                               "300 text tokens, random init",
+                   "gpu_block_ms": round(t_gpu / 1e3, 4),
+                   "cpu_baseline": {"value": round(t_cpu, 2), "unit": "ms per block forward", "cores": threads,
+                                    "kind": "port", "sample": "the whole workload in fp32, 5 timed iterations after 1 warm-up"}}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -344,6 +443,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--kernels-only", action="store_true", help="only the per-kernel section (profiling runs)")
+    ap.add_argument("--cfg3-only", action="store_true",
+                    help="with --kernels-only: skip the video-shape and 112-wide-head launches (counter runs: every "
+                         "kernel instance then runs at the cfg3 shape only)")
     ap.add_argument("--stock-conv", action="store_true",
                     help="also time the stock convolution beside the temporal-conv GEMM (minutes of library tuning on a fresh machine)")
     args = ap.parse_args()
@@ -358,7 +460,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.kernels_only:
         with torch.no_grad():
-            kernels, copy_gbs = kernel_rooflines(dev, stock_conv=args.stock_conv)
+            kernels, copy_gbs = kernel_rooflines(dev, stock_conv=args.stock_conv, cfg3_only=args.cfg3_only)
         print(json.dumps({"kernels": kernels, "copy_GBps_this_box": copy_gbs}))
         return
     B, HW = 1, (128, 128)
@@ -393,6 +495,7 @@ def main():
         ips_bf16 = images_per_s(dev, False, 20, 5)
         ips_w8 = images_per_s(dev, True, 20, 5)
         one_image_ms = 1e3 / images_per_s(dev, False, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
+        one_image_ms_w8 = 1e3 / images_per_s(dev, True, 20, 5, B=1)
         video_ms = video_block_ms(dev)
     del blocks
     torch.cuda.empty_cache()
@@ -402,7 +505,7 @@ def main():
     if dom:
         roofline = {"kernel": "gemm4_kernel<bf16, bias+silu> (inverted 1x1 conv, M=16384 N=11200 K=2240)",
                     "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"], "unit": "TFLOP/s",
-                    "frac": dom["frac"], "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES}
+                    "frac": dom["frac"], "traffic": dominant_kernel_traffic_bytes()}
     line = {
         "metric": "Sana-1.6B SanaMSBlock forward latency @16384 tokens (4096px latent)",
         "value": round(block_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -412,6 +515,7 @@ def main():
                                "C=2240, 70x32 heads, Mix-FFN hidden 5600, 300 text tokens, random init"},
         "images_per_s_1024px": {"bf16": round(ips_bf16, 2), "w8a16": round(ips_w8, 2),
                                 "one_image_step_ms_bf16": round(one_image_ms, 3),
+                                "one_image_step_ms_w8a16": round(one_image_ms_w8, 3),
                                 "note": "B=16, N=1024: B / (20 x block latency); DiT blocks of one denoising step only "
                                         "(no text encoder, VAE, embedders, step count or CFG doubling); "
                                         "one_image_step_ms: the same 20 blocks at B=1"},
@@ -423,6 +527,7 @@ def main():
         "copy_GBps_this_box": copy_gbs,
         "peaks": {"hbm_GBps": HBM_PEAK_GBS, "mfma_bf16_TFLOPs": MFMA_BF16_PEAK_TFLOPS},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+        "configs": None if args.no_cpu_baseline else small_configs(dev),
     }
     print(json.dumps(line))
 

@@ -16,6 +16,14 @@
 // remapped so that each XCD (own L2) works on a compact group of tiles.
 #include "common.h"
 
+// Tuning knobs: non-temporal hint on the output stores / the residual loads of the pipelined kernel's epilogue.
+#ifndef SANA_GEMM_NT_STORE
+#define SANA_GEMM_NT_STORE 1
+#endif
+#ifndef SANA_GEMM_NT_RES
+#define SANA_GEMM_NT_RES 0
+#endif
+
 namespace sana {
 namespace {
 
@@ -724,7 +732,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
       for (int it = 0; it < 8; ++it)
         res[j][it] = __builtin_bit_cast(
-            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, 0));
+            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, SANA_GEMM_NT_RES ? kBufferNt : 0));
   }
   float bv[NI][16];
   if (HAS_BIAS) {
@@ -793,7 +801,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       __builtin_amdgcn_sched_barrier(0);
       if (js >= 0) {
         if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[js][st]);
-        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, SANA_GEMM_NT_STORE ? kBufferNt : 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }

@@ -28,6 +28,12 @@
 #ifndef SANA_LA_APPLY_TOKENS
 #define SANA_LA_APPLY_TOKENS 128
 #endif
+#ifndef SANA_LA_NT_LOAD
+#define SANA_LA_NT_LOAD 0
+#endif
+#ifndef SANA_LA_NT_STORE
+#define SANA_LA_NT_STORE 0
+#endif
 #ifndef SANA_LA_APPLY_U
 #define SANA_LA_APPLY_U 4
 #endif
@@ -99,8 +105,8 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
     for (int i = 0; i < 4; ++i) {
       const int tok = tile + ld_tok + 8 * i;
       if (ch_ok && tok < t1) {
-        kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n);
-        vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n);
+        kreg[i] = load_stream<SANA_LA_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(kbase + (int64_t)tok * stride_n));
+        vreg[i] = load_stream<SANA_LA_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(vbase + (int64_t)tok * stride_n));
         if (has_norm) rin[i] = pre.rinv[(int64_t)b * N + tok];
         if (has_rope) {
           const float* rp = pre.rope + ((int64_t)tok * 16 + (lane & 3) * 4) * 2;
@@ -397,7 +403,7 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int tok = t + 16 * u + 8 * j + ld_tok;
-        raw[u][j] = (tok < t1 && ld_ok) ? *reinterpret_cast<const u32x4_t*>(qrow + (int64_t)tok * q_stride_n) : zero4;
+        raw[u][j] = (tok < t1 && ld_ok) ? load_stream<SANA_LA_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(qrow + (int64_t)tok * q_stride_n)) : zero4;
       }
       const int tok = t + 16 * u + n;
       if (has_norm) rin[u] = tok < t1 ? pre.rinv[(int64_t)b * N + tok] : 0.f;
@@ -443,8 +449,8 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
               o1[s] = acc[1][s] / den;
             }
             float* op = reinterpret_cast<float*>(out) + o_off;
-            *reinterpret_cast<f32x4_t*>(op) = o0;
-            *reinterpret_cast<f32x4_t*>(op + 4) = o1;
+            store_stream<SANA_LA_NT_STORE != 0>(o0, reinterpret_cast<f32x4_t*>(op));
+            store_stream<SANA_LA_NT_STORE != 0>(o1, reinterpret_cast<f32x4_t*>(op + 4));
           }
         } else {
           const float inv = __builtin_amdgcn_rcpf(den);
@@ -463,8 +469,8 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
           const int tok_s = t + 16 * u + 8 * j + ld_tok;
           const u32x4_t o = *reinterpret_cast<const u32x4_t*>(ostage + slot_w[j]);
           if (tok_s < t1 && ld_ok)
-            *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + (int64_t)b * o_stride_b +
-                                        (int64_t)tok_s * o_stride_n + p * 64 + 8 * ld_chunk) = o;
+            store_stream<SANA_LA_NT_STORE != 0>(o, reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(out) + (int64_t)b * o_stride_b +
+                                                       (int64_t)tok_s * o_stride_n + p * 64 + 8 * ld_chunk));
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the next step overwrites
       }
@@ -552,7 +558,7 @@ __global__ __launch_bounds__(256) void qk_rms_kernel(const uint16_t* __restrict_
   const uint16_t* x = (blockIdx.y == 0 ? Q : K) + (row / N) * stride_b + (row % N) * stride_n;
   float acc = 0.f;
   for (int c0 = lane * 8; c0 < C; c0 += 512) {
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + c0);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + c0);  // cacheable: the attention kernels read q and k next
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float a = bf16_lo(v[e]), b2 = bf16_hi(v[e]);

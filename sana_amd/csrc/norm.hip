@@ -13,6 +13,13 @@
 // reproduced in registers.
 #include "common.h"
 
+#ifndef SANA_LN_NT_LOAD
+#define SANA_LN_NT_LOAD 0
+#endif
+#ifndef SANA_LN_NT_STORE
+#define SANA_LN_NT_STORE 0
+#endif
+
 namespace sana {
 namespace {
 
@@ -43,7 +50,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int ch = lane + 64 * i;
-    raw[i] = ch < nchunks ? *reinterpret_cast<const u32x4_t*>(xr + 8 * ch) : zero4;
+    raw[i] = ch < nchunks ? load_stream<SANA_LN_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(xr + 8 * ch)) : zero4;
   }
   if (ADD) {
     const uint16_t* yr = y + row * ldy;
@@ -52,11 +59,11 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
     for (int i = 0; i < NCH; ++i) {
       const int ch = lane + 64 * i;
       if (ch < nchunks) {
-        const u32x4_t b = *reinterpret_cast<const u32x4_t*>(yr + 8 * ch);
+        const u32x4_t b = load_stream<SANA_LN_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(yr + 8 * ch));
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           raw[i][e] = pack_bf16(bf16_lo(raw[i][e]) + bf16_lo(b[e]), bf16_hi(raw[i][e]) + bf16_hi(b[e]));
-        *reinterpret_cast<u32x4_t*>(sr + 8 * ch) = raw[i];
+        store_stream<SANA_LN_NT_STORE != 0>(raw[i], reinterpret_cast<u32x4_t*>(sr + 8 * ch));
       }
     }
   }
@@ -95,7 +102,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
         const uint32_t t = pack_bf16(bf16_lo(ln) * bf16_lo(s1), bf16_hi(ln) * bf16_hi(s1));
         o[e] = pack_bf16(bf16_lo(t) + bf16_lo(sh[e]), bf16_hi(t) + bf16_hi(sh[e]));
       }
-      *reinterpret_cast<u32x4_t*>(orow + 8 * ch) = o;
+      store_stream<SANA_LN_NT_STORE != 0>(o, reinterpret_cast<u32x4_t*>(orow + 8 * ch));
     }
   }
 }
@@ -114,8 +121,8 @@ __global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __re
   if (id >= M * chunks) return;
   const int64_t m = id / chunks;
   const int n = (int)(id - m * chunks) * 8;
-  const u32x4_t yv = *reinterpret_cast<const u32x4_t*>(y + m * ldy + n);
-  const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(res + m * ldr + n);
+  const u32x4_t yv = load_stream<SANA_LN_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(y + m * ldy + n));
+  const u32x4_t rv = load_stream<SANA_LN_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(res + m * ldr + n));
   const u32x4_t gv = *reinterpret_cast<const u32x4_t*>(gate + (m / rows_per_gate) * gate_stride + n);
   u32x4_t o;
 #pragma unroll
@@ -123,7 +130,7 @@ __global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __re
     const uint32_t t = pack_bf16(bf16_lo(gv[e]) * bf16_lo(yv[e]), bf16_hi(gv[e]) * bf16_hi(yv[e]));
     o[e] = pack_bf16(bf16_lo(rv[e]) + bf16_lo(t), bf16_hi(rv[e]) + bf16_hi(t));
   }
-  *reinterpret_cast<u32x4_t*>(out + m * ldo + n) = o;
+  store_stream<SANA_LN_NT_STORE != 0>(o, reinterpret_cast<u32x4_t*>(out + m * ldo + n));
 }
 
 }  // namespace
