@@ -14,6 +14,8 @@
 // double buffered (2 x 64 KB); 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
 // that ds_read_b128 / ds_write_b128 are bank-conflict free.  Workgroup ids are
 // remapped so that each XCD (own L2) works on a compact group of tiles.
+#include <algorithm>
+
 #include "common.h"
 
 // Tuning knobs: non-temporal hint on the output stores / the residual loads of the pipelined kernel's epilogue.
@@ -869,6 +871,25 @@ int pick_ni(int M, int N) {
   return cost192 < cost256 ? 3 : 4;
 }
 
+// Channels to cover with 256-wide tiles when the rest goes to 192-wide ones in a second launch, or 0 when one width
+// for all of N is at least as good.  Costs in rounds of 256 workgroups: a 192-wide round counts 0.78 (3/4 of the
+// math, 4 % more operand traffic per MFMA), the second launch 0.05; the mix must win by 2 %.
+int mixed_split(int M, int N) {
+  const int64_t cu = compute_units(), tiles_t = (M + BT - 1) / BT;
+  auto rounds = [&](int64_t col_tiles) { return (double)((tiles_t * col_tiles + cu - 1) / cu); };
+  const double pure = std::min(rounds((N + 255) / 256), 0.78 * rounds((N + 191) / 192));
+  double best = pure * 0.98;
+  int best_wide = 0;
+  for (int a = 1; a * 256 < N; ++a) {
+    const double cost = rounds(a) + 0.78 * rounds((N - a * 256 + 191) / 192) + 0.05;
+    if (cost < best) {
+      best = cost;
+      best_wide = a * 256;
+    }
+  }
+  return best_wide;
+}
+
 // Which kernel, and whether K is split.  A workgroup's K loop is a latency chain whatever the grid: about
 // 1.1 us per k-tile for the 256-wide pipelined kernel, 0.8 us for the 128 x 128 one (a quarter of the math, but
 // the same load / LDS / barrier round trip).  A grid that covers the chip keeps the 256-wide kernel (throughput
@@ -1003,6 +1024,24 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
     return launch_small<W8>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
   if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
     float* ws = aligned16(workspace) ? static_cast<float*>(workspace) : nullptr;
+    // Mixed channel tiling: the first n_wide channels in 256-wide tiles, the rest in 192-wide ones, as two launches
+    // over disjoint column ranges of C, when that needs fewer rounds of the chip than either width alone (qkv at
+    // 16384 tokens, N = 6720: 27 x 256 is 7 rounds of 256 tiles, 24 x 256 + 3 x 192 is 6 rounds + one of 192-wide
+    // tiles, 6.8 round-equivalents).  Same k order per output: bit-identical to the single launch.
+    if (!taps && plan_gemm(M, N, K, W8).S == 1) {
+      const int n_wide = mixed_split(M, N);
+      if (n_wide > 0) {
+        const int rc = launch4<W8, 4>(a, W, scale, ep, c, M, n_wide, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
+        if (rc != SANA_OK) return rc;
+        EpiArgs ep2 = ep;
+        if (ep2.bias) ep2.bias += n_wide;
+        if (ep2.gate) ep2.gate += n_wide;
+        if (ep2.res) ep2.res += n_wide;
+        return launch4<W8, 3>(a, static_cast<const char*>(W) + (int64_t)n_wide * ldw * (W8 ? 1 : 2),
+                              scale ? scale + n_wide : nullptr, ep2, c + n_wide, M, N - n_wide, K, lda, ldw, ldc, epilogue,
+                              s, nullptr, nullptr, 0);
+      }
+    }
     return pick_ni(M, N) == 3
                ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes)
                : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes);

@@ -138,6 +138,38 @@ def test_gemm_strided_views(cuda):
     assert out[:, :8].abs().max() == 0 and out[:, 144:].abs().max() == 0
 
 
+@pytest.mark.parametrize("w8", [False, True])
+def test_gemm_mixed_channel_tiling_is_bit_identical(cuda, w8):
+    """qkv at 16384 tokens (N = 6720) runs as two launches: 24 tiles of 256 channels and 3 of 192.  Every output sums
+    its k products in the same order whatever the tiling, so the first 256 rows -- which alone are one launch of one
+    width -- must come out bit for bit the same; bias, SiLU, the gated residual and int8 weights ride along."""
+    from sana_amd.modules import quantize_w8
+    M, N, K = 16384, 6720, 192
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(M, K, generator=g).bfloat16().to(cuda)
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(cuda)
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16().to(cuda)
+    if w8:
+        wq, sc = quantize_w8(w)
+        run = lambda x, epi: ops.gemm_w8a16(x, wq, sc, bias, epi, expand=False)
+    else:
+        run = lambda x, epi: ops.gemm_bf16(x, w, bias, epi)
+    for epi in ("bias", "bias_silu"):
+        whole, head = run(a, epi), run(a[:256], epi)
+        assert torch.equal(whole[:256], head)
+        # a tile row in the middle and the last one, against the same rows alone
+        assert torch.equal(whole[8192:8448], run(a[8192:8448], epi))
+        assert torch.equal(whole[-256:], run(a[-256:], epi))
+    if not w8:
+        ref = a[:512].double() @ w.double().T + bias.double()
+        assert rel_l2(run(a, "bias")[:512].cpu(), ref.cpu()) <= 4e-3
+        gate = (torch.randn(1, 1, N, generator=g) * 0.5).bfloat16().to(cuda)
+        res = torch.randn(1, M, N, generator=g).bfloat16().to(cuda)
+        whole = ops.gemm_gate_residual(a.view(1, M, K), w, bias, gate, res)
+        head = ops.gemm_gate_residual(a[:256].view(1, 256, K), w, bias, gate, res[:, :256])
+        assert torch.equal(whole[0, :256], head[0])
+
+
 def test_gemm_exact_on_integer_inputs(cuda):
     """Small integers: every product and partial sum is exact in fp32, the result is exact in bf16."""
     g = torch.Generator().manual_seed(3)
