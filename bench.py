@@ -422,6 +422,8 @@ def small_configs(dev):
     xd, yd, td = (a.bfloat16().to(dev) for a in (x, y, t))
     with torch.no_grad():
         t_gpu = event_time_us(lambda: hb(xd, yd, td, HW=HW), 50, 10)
+        graphed = S.GraphedCall(lambda a, b, c: hb(a, b, c, HW=HW), (xd, yd, td))
+        t_graph = event_time_us(lambda: graphed(xd, yd, td), 50, 10)
         ob(x, y, t, HW=HW)
         t0 = time.perf_counter()
         for _ in range(5):
@@ -429,7 +431,9 @@ def small_configs(dev):
         t_cpu = (time.perf_counter() - t0) / 5 * 1e3
     res["cfg2"] = {"workload": "one SanaMSBlock at Sana-600M width, bf16, B=4, N=32x32=1024, C=1152, hidden 2880, "
                                "300 text tokens, random init",
-                   "gpu_block_ms": round(t_gpu / 1e3, 4),
+                   "gpu_block_ms": round(t_gpu / 1e3, 4), "gpu_block_ms_hip_graph": round(t_graph / 1e3, 4),
+                   "note": "eager issue of the block's ~25 launches from Python is host-bound at this size; "
+                           "gpu_block_ms_hip_graph replays the same launches from one captured HIP graph (sana_amd.GraphedCall)",
                    "cpu_baseline": {"value": round(t_cpu, 2), "unit": "ms per block forward", "cores": threads,
                                     "kind": "port", "sample": "the whole workload in fp32, 5 timed iterations after 1 warm-up"}}
     return res

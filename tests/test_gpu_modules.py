@@ -329,6 +329,29 @@ def test_block_replays_from_a_hip_graph(cuda):
         check(out, _ref64(ob, x.cpu(), y.cpu(), t.cpu(), HW=HW), "graph replay vs fp64 oracle", block=True)
 
 
+def test_graphed_call_replays_a_chain_of_blocks(cuda):
+    """sana_amd.GraphedCall: two chained blocks captured once; replays with new inputs equal the eager chain bit for
+    bit, with eager work and synchronisations between the replays."""
+    C, heads, B, HW = 256, 8, 2, (16, 16)
+    blocks = []
+    for seed in (11, 12):
+        _, hb = _pair(C, heads, seed=seed)
+        blocks.append(hb.to(cuda))
+    chain = lambda x, y, t: blocks[1](blocks[0](x, y, t, HW=HW), y, t, HW=HW)
+    x, y, t = (a.bfloat16().to(cuda) for a in O.block_inputs(B, HW[0] * HW[1], C, seed=13))
+    graphed = S.GraphedCall(chain, (x, y, t))
+    with torch.no_grad():
+        for r in range(3):
+            xr = torch.randn(x.shape, generator=torch.Generator().manual_seed(20 + r)).bfloat16().to(cuda)
+            out = graphed(xr, y, t)
+            torch.cuda.synchronize()
+            eager = chain(xr, y, t)
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {r}"
+    with pytest.raises(ValueError):
+        graphed(x[:1], y, t)
+
+
 def test_graph_replay_survives_a_larger_eager_shape(cuda):
     """A captured block holds the raw addresses of the scratch buffers it used (attention partial states, split-k
     planes).  A later, larger eager call makes the library take bigger buffers; the captured ones must stay alive
