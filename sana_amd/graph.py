@@ -17,14 +17,15 @@ class GraphedCall:
     """``fn(*tensors)`` captured into a HIP graph on the tensors' device.
 
     ``fn`` must be a fixed sequence of device work on its tensor arguments (shapes, dtypes and every non-tensor
-    argument baked in), e.g. ``lambda x, y, t: block(x, y, t, HW=(32, 32))``.  Calling the object copies the new
-    arguments into the captured input buffers, replays, and returns the captured output tensor (the same tensor
-    every time: clone it to keep a result across calls)."""
+    argument baked in), e.g. ``lambda x, y, t: block(x, y, t, HW=(32, 32))``.  The example tensors become the
+    captured input buffers: calling the object copies any argument that is another tensor into them (passing the
+    example tensors themselves, updated in place, costs no copy), replays, and returns the captured output tensor
+    (the same tensor every time: clone it to keep a result across calls)."""
 
     def __init__(self, fn: Callable[..., torch.Tensor], example: Sequence[torch.Tensor], warmup: int = 2):
         if not example or not all(torch.is_tensor(t) and t.is_cuda for t in example):
             raise ValueError("GraphedCall needs device tensors as example arguments")
-        self._inputs = [t.clone() for t in example]
+        self._inputs = list(example)   # the example tensors ARE the captured input buffers
         with torch.no_grad():
             side = torch.cuda.Stream(device=example[0].device)
             side.wait_stream(torch.cuda.current_stream())
