@@ -462,8 +462,8 @@ class GLUMBConv(nn.Module):
         super().__init__()
         out_feature = out_feature or in_features
         use_bias, norm, act = _tuple3(use_bias), _tuple3(norm), _tuple3(act)
-        if kernel_size != 3 or stride != 1 or dilation != 1 or padding not in (None, 1):
-            raise NotImplementedError("GLUMBConv HIP path: kernel_size=3, stride=1, dilation=1 only")
+        if kernel_size != 3 or stride != 1 or dilation < 1 or padding not in (None, dilation):
+            raise NotImplementedError("GLUMBConv HIP path: kernel_size=3, stride=1, 'same' padding only")
         if any(n is not None for n in norm):
             raise NotImplementedError("GLUMBConv HIP path: norm must be (None, None, None)")
         if tuple(act) != ("silu", "silu", None):
@@ -474,6 +474,11 @@ class GLUMBConv(nn.Module):
         self.inverted_conv = self._pointwise_layer(in_features, hidden_features * 2, use_bias[0], "silu")
         self.depth_conv = ConvLayer(hidden_features * 2, hidden_features * 2, 3, groups=hidden_features * 2,
                                     use_bias=use_bias[1], act=None)
+        # dilation > 1 (`glumbconv_dilate`, diffusion/model/nets/sana.py:126-134) has no kernel: the depthwise stage
+        # then runs as the stock convolution (logged), the two 1x1 convolutions stay on the MFMA GEMM
+        self.dilation = dilation
+        self.depth_conv.conv.dilation = (dilation, dilation)
+        self.depth_conv.conv.padding = (dilation, dilation)
         self.point_conv = self._pointwise_layer(hidden_features, out_feature, use_bias[2], None)
         self.round_like_reference = True
 
@@ -507,8 +512,15 @@ class GLUMBConv(nn.Module):
         ic, pc = self._pointwise_params(self.inverted_conv), self._pointwise_params(self.point_conv)
         dc = self.depth_conv.conv
         u = hip_linear(x, ic.weight, ic.bias, "silu", getattr(ic, "weight_q", None), getattr(ic, "weight_scale", None))
-        y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
-                                    round_like_reference=self.round_like_reference)
+        if self.dilation == 1:
+            y = ops.dwconv3x3_silu_gate(u.view(frames, H, W, u.shape[-1]), dc.weight, dc.bias,
+                                        round_like_reference=self.round_like_reference)
+        else:
+            stock_path("GLUMBConv depthwise conv", f"dilation {self.dilation} has no kernel (stock convolution, "
+                       "chunk, SiLU and product on a channels-last view)")
+            w4 = dc(u.view(frames, H, W, u.shape[-1]).permute(0, 3, 1, 2))          # NCHW view of NHWC memory
+            a, g = torch.chunk(w4, 2, dim=1)
+            y = (a * self.glu_act(g)).permute(0, 2, 3, 1).contiguous()
         return hip_linear(y.view(B, N, y.shape[-1]), pc.weight, pc.bias, None,
                           getattr(pc, "weight_q", None), getattr(pc, "weight_scale", None), gate, residual, out)
 

@@ -329,6 +329,32 @@ def test_block_replays_from_a_hip_graph(cuda):
         check(out, _ref64(ob, x.cpu(), y.cpu(), t.cpu(), HW=HW), "graph replay vs fp64 oracle", block=True)
 
 
+def test_glumbconv_with_dilation_takes_the_logged_stock_depthwise(cuda, caplog):
+    """dilation = 2 (`glumbconv_dilate`): no depthwise kernel, so that one stage is the stock convolution -- said
+    once on the logger -- between the two MFMA GEMMs; same keys, same result as the oracle."""
+    import logging
+    from sana_amd import modules as M
+    C, Hd, B, HW = 64, 160, 2, (9, 7)
+    om = O.GLUMBConv(C, Hd, use_bias=(True, True, False), norm=(None, None, None), act=("silu", "silu", None), dilation=2)
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        for p in om.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.2)
+    om = om.bfloat16()
+    hm = S.GLUMBConv(C, Hd, use_bias=(True, True, False), norm=(None, None, None), act=("silu", "silu", None),
+                     dilation=2).bfloat16()
+    hm.load_state_dict(om.state_dict(), strict=True)
+    hm = hm.to(cuda)
+    x = torch.randn(B, HW[0] * HW[1], C, generator=g).bfloat16()
+    M._stock_paths_seen.clear()
+    with torch.no_grad(), caplog.at_level(logging.WARNING, logger="sana_amd"):
+        out = hm(x.to(cuda), HW=HW)
+        hm(x.to(cuda), HW=HW)
+        ref = _ref64(om, x, HW=HW)
+    check(out, ref, "GLUMBConv dilation 2")
+    assert sum("dilation 2" in r.getMessage() for r in caplog.records) == 1
+
+
 def test_graphed_call_replays_a_chain_of_blocks(cuda):
     """sana_amd.GraphedCall: two chained blocks captured once; replays with new inputs equal the eager chain bit for
     bit, with eager work and synchronisations between the replays."""

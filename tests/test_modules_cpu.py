@@ -93,8 +93,12 @@ def test_unsupported_options_fail_loudly():
     with pytest.raises(NotImplementedError):
         S.LiteLA(128, 128, dim=64)          # head dims with kernels: 32 and 112
     assert S.LiteLA(224, 224, dim=112).heads == 2
+    # dilation 2 (glumbconv_dilate) is accepted: its depthwise stage is a logged stock convolution; same keys
+    dil = S.GLUMBConv(64, 160, dilation=2)
+    assert dil.depth_conv.conv.dilation == (2, 2) and dil.depth_conv.conv.padding == (2, 2)
+    assert list(dil.state_dict()) == list(O.GLUMBConv(64, 160, dilation=2).state_dict())
     with pytest.raises(NotImplementedError):
-        S.GLUMBConv(64, 160, dilation=2)
+        S.GLUMBConv(64, 160, stride=2)
     with pytest.raises(NotImplementedError):
         S.GLUMBConv(64, 160, norm=("bn2d", None, None))
     with pytest.raises(NotImplementedError):
