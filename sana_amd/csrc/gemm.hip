@@ -4,14 +4,17 @@
 // Both operands are K-contiguous, which is exactly the MFMA operand layout (a
 // lane holds 8 consecutive k of one row), so nothing is transposed.  The MFMA
 // "row" operand is the WEIGHT tile and the "column" operand the ACTIVATION
-// tile: in the 32x32 accumulator layout a lane then owns one token (column)
-// and 16 output channels.  Weight rows are stored to LDS in a permuted order
-// (row 16*g + 4*q + s of a 32-row block goes to LDS row 8*q + 4*g + s) so that
-// those 16 channels are contiguous and a lane stores 32 contiguous bytes of C.
+// tile: a lane of the accumulator then owns one token (column) and a few output
+// channels (rows).  Weight rows are permuted on their way into LDS so that the
+// channels a lane owns are contiguous in C (the pipelined kernel: 8*NI channels
+// from 2*NI MFMA tiles of 16; the compiler-scheduled one: 16 channels per 32x32 tile).
 //
 // Workgroup tile 256 (tokens) x 256 (channels) x 64 (k), four waves in 2x2,
-// each 128x128 = 4x4 MFMA 32x32x16 tiles (256 fp32 accumulators).  LDS is
-// double buffered (2 x 64 KB); 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
+// each 128x128 (256 fp32 accumulators).  The pipelined kernel multiplies with
+// v_mfma_f32_16x16x32_bf16: on this chip the matrix pipes are power-limited, and
+// with random bf16 operands a loop of nothing but 32x32x16 MFMAs settles at 1.64 GHz
+// (0.69 of the 2.5 PFLOP/s peak) where the same flops as 16x16x32 run at 1.9-2.0 GHz.
+// LDS is double buffered (2 x 64 KB); 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
 // that ds_read_b128 / ds_write_b128 are bank-conflict free.  Workgroup ids are
 // remapped so that each XCD (own L2) works on a compact group of tiles.
 #include <algorithm>
@@ -45,6 +48,14 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * ROW_BYTES 
 __device__ __forceinline__ int wrow_to_lds(int n) {
   const int blk = n & ~31, r = n & 31;
   return blk + 8 * ((r >> 2) & 3) + 4 * (r >> 4) + (r & 3);
+}
+
+// acc += W fragment (16 channels x 32 k) . A fragment (32 k x 16 tokens), as an asm statement so that the
+// accumulator is one AGPR quad in and out: given the builtin, whose destination may differ from its addend, the
+// register allocator rotates accumulators through other registers across the loop edge (dozens of copies and
+// their wait states per k-tile in some instances).
+__device__ __forceinline__ void mfma_acc(f32x4_t& c, u32x4_t a, u32x4_t b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
 __device__ __forceinline__ uint32_t dequant2(uint32_t q4, int which, float s, float off) {
@@ -382,24 +393,27 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
 
 
 // ============================================================================
-// Pipelined kernel (K % 16 == 0, K >= 64; bf16 and int8 weights): 256 threads, one
+// Pipelined kernel (K % 32 == 0, K >= 64; bf16 and int8 weights): 256 threads, one
 // wave per SIMD with the whole register file (256 accumulators + 256 VGPRs), each
-// wave a sub-tile of 128 tokens x 32*NI channels = NI x 4 MFMA tiles (NI = 4: 128x128,
-// every fragment read from LDS feeds four MFMAs; NI = 3 or 2 narrows the workgroup's
-// channel tile to 192 or 128 where that fills the last round of workgroups better).  With a single wave per SIMD nothing
+// wave a sub-tile of 128 tokens x 32*NI channels = 2*NI x 8 MFMA tiles of 16x16
+// (NI = 4: 128x128; NI = 3 narrows the workgroup's channel tile to 192 where that fills
+// the last round of workgroups better).  With a single wave per SIMD nothing
 // else hides a stalled memory instruction, so the main loop is one hand-ordered
-// stream (pinned with sched_barrier): a k-tile is 16*NI MFMA slots and a slot carries
-// one or two LDS / global instructions (NI = 4, bf16):
-//   * even slots of k-steps 0-2 read the fragments of the next k-step;
-//   * slot 3q+1 stores staging quad q (k-tile kt+1) into the other LDS stage and
-//     slot 3q+2 reloads the same registers with k-tile kt+2, so every global load
-//     has a whole k-tile (about 1 us) to land and one 64-register set is enough
+// stream (pinned with sched_barrier): a k-tile is two k-steps of 32 = 2 * 16*NI MFMA
+// slots of 16 cycles, and a lone wave issues about one other instruction per 5 cycles,
+// so a slot carries at most a fragment read, a store or a load (bf16):
+//   * k-step 0: the fragments of k-step 1, and all staging -- quad q (k-tile kt+1) is
+//     stored into the other LDS stage and the same registers are re-loaded with
+//     k-tile kt+2 one slot later, so every global load has a whole k-tile (about
+//     1 us) to land and one 64-register set is enough;
+//   * the only barrier sits right behind it, and the next tile's k-step-0 fragments
+//     are read over the rest of k-step 1, which runs from the other fragment buffer
 //     (int8 weights: 16 values per quad, converted two at a time in the MFMA slots
-//     before they are stored, the quad reloaded after its last piece);
-//   * the only barrier sits in k-step 3 after the last store; the slots behind it
-//     read k-step 0 of the next tile.
+//     before they are stored, the quad reloaded after its last piece; their barrier
+//     stays at the end of the k-tile).
+// The MFMAs are asm statements with the accumulator tied in and out (see mfma_acc).
 // Rows past M / N read as zero (buffer range check) and only feed outputs that are
-// never stored; the last k-tile runs just the k-steps that exist.  Needs K % 16 == 0 and K >= 64.
+// never stored; the last k-tile runs just the k-steps that exist.
 // ============================================================================
 // SPLIT (split-k, for shapes with too few tiles to fill the chip): grid row z multiplies its own range of
 // k-tiles and stores the raw fp32 accumulators to C taken as float [gridDim.y][M][N]; splitk_epilogue_kernel
@@ -448,36 +462,46 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   const int g_chunk = tid & 7, g_row = tid >> 3;
   const int a_last = min(BT, M - m0) - 1, w_last = min(BCN, N - n0) - 1;  // last valid row of each tile
   const uint32_t ulda = (uint32_t)lda, uldw = (uint32_t)ldw;
-  const int a_dst0 = swz(g_row, g_chunk);                            // rows +32*q keep the key: +4096 bytes each
-  const int w_dst0 = TILE_BYTES + swz(wrow_to_lds(g_row), g_chunk);  // the row permutation stays inside 32-row blocks
+  const int a_dst0 = swz(g_row, g_chunk);               // rows +32*q keep the key: +4096 bytes each
+  const int w_dst0 = TILE_BYTES + swz(g_row, g_chunk);  // LDS rows g_row + 32*q; the weight-row permutation is on the global side
+  // LDS row L of a wave's block of 32*NI weight rows belongs to MFMA tile L / 16 as its row L % 16 = 4*g + r, and
+  // holds channel 8*NI*g + 4*(L / 16) + r of the block: a lane's accumulators (tile i, registers r) are then the
+  // 8*NI contiguous channels 8*NI*g + 4*i + r.  The thread's quad q (LDS rows g_row + 32*q) is channel
+  // w_chan0 + 8*(q % NI) + 32*NI*(q / NI) of the tile.
+  const int w_chan0 = 8 * NI * ((g_row >> 2) & 3) + 4 * (g_row >> 4) + (g_row & 3);
   constexpr int NWQ = W8 ? NI : 2 * NI;  // W quads per thread
   constexpr int NQ = 8 + NWQ;
   u32x4_t rs[NQ];  // the k-tile in flight: A quads 0..7, then the W quads
   const int q_chunk = tid & 3, q_row = tid >> 2;
-  const int q_dst_lo = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk);  // rows +64*q: +8192 bytes, same key
-  const int q_dst_hi = TILE_BYTES + swz(wrow_to_lds(q_row), 2 * q_chunk + 1);
+  const int q_dst_lo = TILE_BYTES + swz(q_row, 2 * q_chunk);  // LDS rows q_row + 64*q: +8192 bytes, same key
+  const int q_dst_hi = TILE_BYTES + swz(q_row, 2 * q_chunk + 1);
   float wscale[NI], woff[NI];
+  int q_voff[NI];  // int8 quads: byte offset of the channel that LDS row q_row + 64*q holds
   if (W8) {
 #pragma unroll
     for (int q = 0; q < NI; ++q) {
-      wscale[q] = scale[n0 + min(q_row + 64 * q, w_last)];
+      const int L = q_row + 64 * q, blk = L / (32 * NI), l = L % (32 * NI);
+      const int chan = blk * 32 * NI + 8 * NI * ((l >> 2) & 3) + 4 * (l >> 4) + (l & 3);
+      q_voff[q] = chan * (int)ldw + 16 * q_chunk;
+      wscale[q] = scale[n0 + min(chan, w_last)];
       woff[q] = -128.f * wscale[q];
     }
   }
   u32x4_t dq[2];  // dequantised halves of the int8 quad being converted
 
   const int wc = wave & 1, wt = wave >> 1;
-  const int fr = lane & 31, fg = lane >> 5;
+  const int fr = lane & 15, fg = lane >> 4;
   const int x7 = swz_key(fr);
   const int w_off = TILE_BYTES + (wc * 32 * NI + fr) * ROW_BYTES, a_off = (wt * 128 + fr) * ROW_BYTES;
-  f32x16_t acc[NI][4];
+  constexpr int NWT = 2 * NI;  // MFMA tiles of 16 channels per wave (and 8 tiles of 16 tokens)
+  f32x4_t acc[NWT][8];
 #pragma unroll
-  for (int i = 0; i < NI; ++i)
+  for (int i = 0; i < NWT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  u32x4_t fw[2][NI], fa[2][4];
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  u32x4_t fw[2][NWT], fa[2][8];
 
 #define SANA_G4_PIN() __builtin_amdgcn_sched_barrier(0)
   // Operand tiles are read with buffer loads: the tile's rows are one resource each for A and W (scalar
@@ -522,15 +546,17 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       const_cast<char*>(static_cast<const char*>(Wv) + (int64_t)n0 * ldw * (W8 ? 1 : 2)), 0,
       (int)(((int64_t)w_last * ldw + K) * (W8 ? 1 : 2)), 0x00020000);
   const int voff_a = (g_row * (int)ulda + 8 * g_chunk) * 2;
-  const int voff_w = W8 ? q_row * (int)uldw + 16 * q_chunk : (g_row * (int)uldw + 8 * g_chunk) * 2;
-  const int step_a = 32 * (int)ulda * 2, step_w = W8 ? 64 * (int)uldw : 32 * (int)uldw * 2;
+  const int voff_w = (w_chan0 * (int)uldw + 8 * g_chunk) * 2;  // bf16 weights
+  const int step_a = 32 * (int)ulda * 2, step_w1 = (int)uldw * 2;
   auto gload = [&](int q, int k0) {
     if (q < 8) {
       const int off = (TAPS == 2 ? voffq[q] : voff_a) + (q * step_a + (TAPS ? a_kb : k0 * 2));
       const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0);
       rs[q] = __builtin_bit_cast(u32x4_t, v);
     } else {
-      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w + ((q - 8) * step_w + k0 * (W8 ? 1 : 2)), 0, 0);
+      const int wq = q - 8;
+      const int off = W8 ? q_voff[wq] + k0 : voff_w + ((8 * (wq % NI) + 32 * NI * (wq / NI)) * step_w1 + k0 * 2);
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, off, 0, 0);
       rs[q] = __builtin_bit_cast(u32x4_t, v);
     }
   };
@@ -548,16 +574,20 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       *reinterpret_cast<u32x4_t*>(base + (piece < 4 ? q_dst_lo : q_dst_hi)) = dq[piece >> 2];
     }
   };
-  constexpr int NFR = NI + 4;  // fragment reads per k-step
-  auto fread = [&](const unsigned char* st, int buf, int ks, int q) {  // q < NI: W fragment, else A fragment
-    const int col = ((2 * ks + fg) ^ x7) << 4;
-    if (q < NI) fw[buf][q] = *reinterpret_cast<const u32x4_t*>(st + w_off + q * 32 * ROW_BYTES + col);
-    else fa[buf][q - NI] = *reinterpret_cast<const u32x4_t*>(st + a_off + (q - NI) * 32 * ROW_BYTES + col);
+  constexpr int NFR = NWT + 8;  // fragment reads per k-step (of 32)
+  // read r of a k-step, in the order the MFMAs need them: W tile 0, the eight A tiles, then W tiles 1 ..
+  auto fread = [&](const unsigned char* st, int buf, int ks, int r) {
+    const int col = ((4 * ks + fg) ^ x7) << 4;
+    if (r == 0 || r > 8) {
+      const int i = r == 0 ? 0 : r - 8;
+      fw[buf][i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 16 * ROW_BYTES + col);
+    } else {
+      fa[buf][r - 1] = *reinterpret_cast<const u32x4_t*>(st + a_off + (r - 1) * 16 * ROW_BYTES + col);
+    }
   };
-  auto mfma = [&](int buf, int t) {  // t < 4 * NI
-    const int i = t >> 2, j = t & 3;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[buf][i]),
-                                                       __builtin_bit_cast(bf16x8_t, fa[buf][j]), acc[i][j], 0, 0, 0);
+  auto mfma = [&](int buf, int t) {  // t < 8 * NWT
+    const int i = t >> 3, j = t & 7;
+    mfma_acc(acc[i][j], fw[buf][i], fa[buf][j]);
   };
 
   const int KT = (K + BK - 1) / BK;
@@ -586,45 +616,57 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
   for (int q = 0; q < NFR; ++q) fread(smem, 0, 0, q);
 
-  // slots per k-step, the barrier slot (the NFR slots behind it read the next tile's k-step 0), and
-  // the spacing of the staging quads in front of it
-  constexpr int SL = 4 * NI, BAR = 4 * SL - NFR - 1;
-  constexpr int QSTRIDE = (BAR - 2) / NQ;  // bf16: store quad q at slot 1 + q*QSTRIDE, reload it one slot later
-  static_assert(QSTRIDE >= 2 && 4 * 7 + 1 < BAR && 8 * NI + 2 < BAR, "staging does not fit in front of the barrier");
+  // Slots: a k-tile is two k-steps of 32 = 2 * SL MFMAs of 16 cycles each, and a lone wave issues about one
+  // other instruction per 5 cycles, so no slot carries more than a fragment read or a store or a load.
+  //  * k-step 0: the fragments of k-step 1 (read r at slot r*SL/NFR), and all staging -- quad q stored to the other
+  //    LDS stage at slot 1 + q*QSTRIDE and re-loaded (k-tile kt+2) one slot later;
+  //  * the barrier right behind it (slot SL + 2), and the next tile's k-step-0 fragments spread over the rest
+  //    of k-step 1, which runs from the other fragment buffer.
+  // int8 weights convert 8*NI pieces in the MFMA slots as well, so their barrier stays at the end of the k-tile.
+  constexpr int SL = 8 * NWT, TS = 2 * SL;
+  constexpr int BAR = W8 ? TS - NFR - 1 : SL + 2;
+  constexpr int RSTR = W8 ? 1 : (TS - BAR - 1 - 8) / NFR;  // spacing of the reads behind the barrier
+  constexpr int QSTRIDE = SL / NQ;                           // bf16: spacing of the staging quads
+  constexpr int PSTR = (BAR - 4) / (8 * NI);                 // int8: piece n (two values) at slot 2 + n*PSTR
+  static_assert(W8 || (QSTRIDE >= 2 && 1 + (NQ - 1) * QSTRIDE < BAR - 2 && RSTR >= 1 && BAR + 1 + (NFR - 1) * RSTR < TS),
+                "staging does not fit in front of the barrier");
+  static_assert(!W8 || (4 * 7 + 1 < BAR && PSTR >= 1), "staging does not fit in front of the barrier");
   for (int kt = 0; kt < KT - 1; ++kt) {
     const int cur = kt & 1;
     const unsigned char* st = smem + cur * 2 * TILE_BYTES;
     const unsigned char* stn = smem + (cur ^ 1) * 2 * TILE_BYTES;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
       for (int t = 0; t < SL; ++t) {
         const int slot = ks * SL + t;
-        mfma(ks & 1, t);
+        mfma(ks, t);
         SANA_G4_PIN();
-        if (ks < 3) {
-          // read r of the next k-step goes to slot (r * SL) / NFR of this one
+        if (ks == 0) {
+          // read r of k-step 1 goes to slot (r * SL) / NFR of k-step 0
           if (((t * NFR + SL - 1) / SL) * SL / NFR == t && (t * NFR + SL - 1) / SL < NFR)
-            fread(st, (ks + 1) & 1, ks + 1, (t * NFR + SL - 1) / SL);
+            fread(st, 1, 1, (t * NFR + SL - 1) / SL);
         }
         if (slot == BAR) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own LDS stores done; no fence: loads stay in flight
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
-        } else if (slot > BAR) {
-          fread(stn, 0, 0, slot - BAR - 1);
+        } else if (slot > BAR && (slot - BAR - 1) % RSTR == 0 && (slot - BAR - 1) / RSTR < NFR) {
+          fread(stn, 0, 0, (slot - BAR - 1) / RSTR);
         }
         if (!W8) {
           if (slot >= 1 && (slot - 1) % QSTRIDE == 0 && (slot - 1) / QSTRIDE < NQ) lstore((slot - 1) / QSTRIDE, cur ^ 1);
           if (slot >= 2 && (slot - 2) % QSTRIDE == 0 && (slot - 2) / QSTRIDE < NQ)
             gload((slot - 2) / QSTRIDE, (kt + 2) * BK);
         } else {
-          // A quad q: store at slot 4q, reload at 4q+1.  int8 piece n at slot n+2 (its half is stored
-          // with pieces 3 and 7), the quad is reloaded right after its last piece.
+          // A quad q: store at slot 4q, reload at 4q+1.  int8 piece n at slot 2 + n*PSTR (its half is stored
+          // with pieces 3 and 7), the quad is reloaded one slot after its last piece.
           if (slot % 4 == 0 && slot / 4 < 8) lstore(slot / 4, cur ^ 1);
           if (slot % 4 == 1 && slot / 4 < 8) gload(slot / 4, (kt + 2) * BK);
-          if (slot >= 2 && slot < 2 + 8 * NI) dequant_piece((slot - 2) >> 3, (slot - 2) & 7, cur ^ 1);
-          if (slot >= 10 && slot <= 2 + 8 * NI && (slot - 10) % 8 == 0) gload(8 + (slot - 10) / 8, (kt + 2) * BK);
+          if (slot >= 2 && (slot - 2) % PSTR == 0 && (slot - 2) / PSTR < 8 * NI)
+            dequant_piece(((slot - 2) / PSTR) >> 3, ((slot - 2) / PSTR) & 7, cur ^ 1);
+          if (slot >= 3 && (slot - 3) % PSTR == 0 && (slot - 3) / PSTR < 8 * NI && (((slot - 3) / PSTR) & 7) == 7)
+            gload(8 + (((slot - 3) / PSTR) >> 3), (kt + 2) * BK);
         }
         SANA_G4_PIN();
       }
@@ -644,40 +686,39 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // The lane's bias values (16 consecutive channels per MFMA tile, packed) are requested here, ahead of
   // the last k-tile, so that their latency hides behind its MFMAs.
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
-  u32x4_t bpk[NI][2];
+  u32x4_t bpk[NI];  // the lane's 8*NI contiguous channels, in chunks of 8
   if (HAS_BIAS) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg + 8 * half;  // N % 8 == 0: a chunk is in or out
-        bpk[i][half] = (ep.bias && n < N) ? *reinterpret_cast<const u32x4_t*>(ep.bias + n) : u32x4_t{0u, 0u, 0u, 0u};
-      }
+    for (int c = 0; c < NI; ++c) {
+      const int n = n0 + wc * 32 * NI + 8 * NI * fg + 8 * c;  // N % 8 == 0: a chunk is in or out
+      bpk[c] = (ep.bias && n < N) ? *reinterpret_cast<const u32x4_t*>(ep.bias + n) : u32x4_t{0u, 0u, 0u, 0u};
+    }
   }
   const int o_chunk = lane & 15, o_rsub = lane >> 4;
   const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
   const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
-  {  // last k-tile: no successor, and K % 64 may leave fewer than four k-steps
+  {  // last k-tile: no successor, and K % 64 may leave one k-step of 32 instead of two
     const unsigned char* st = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
-    const int steps = (K - (KT - 1) * BK) / 16;
+    const int steps = (K - (KT - 1) * BK) / 32;
     for (int ks = 0; ks < steps; ++ks) {
-      const int col = ((2 * ks + fg) ^ x7) << 4;
-      u32x4_t w4[NI], a4[4];
+      const int col = ((4 * ks + fg) ^ x7) << 4;
+      u32x4_t w8[NWT], a8[8];
 #pragma unroll
-      for (int i = 0; i < NI; ++i) w4[i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 32 * ROW_BYTES + col);
+      for (int i = 0; i < NWT; ++i) w8[i] = *reinterpret_cast<const u32x4_t*>(st + w_off + i * 16 * ROW_BYTES + col);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) a4[j] = *reinterpret_cast<const u32x4_t*>(st + a_off + j * 32 * ROW_BYTES + col);
+      for (int j = 0; j < 8; ++j) a8[j] = *reinterpret_cast<const u32x4_t*>(st + a_off + j * 16 * ROW_BYTES + col);
 #pragma unroll
-      for (int i = 0; i < NI; ++i)
+      for (int i = 0; i < NWT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, w4[i]),
-                                                             __builtin_bit_cast(bf16x8_t, a4[j]), acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) mfma_acc(acc[i][j], w8[i], a8[j]);
     }
+    // the MFMAs are asm statements, so the compiler does not know that their results are in flight: wait out the
+    // last ones before anything reads an accumulator
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
   }
 
-  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 32*j + lane%32,
-  // channel n0 + wc*128 + 32*i + 16*(lane/32) + r.  The wave's sub-tile goes through its own 32 KB of
+  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 16*j + lane%16,
+  // channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  The wave's sub-tile goes through its own 32 KB of
   // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
   // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
   // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
@@ -691,18 +732,14 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     const __amdgpu_buffer_rsrc_t rsrc_p =
         __builtin_amdgcn_make_buffer_rsrc(plane, 0, (int)((int64_t)prows * N * 4), 0x00020000);
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = n0 + wc * 32 * NI + 32 * i + 16 * fg;
+    for (int i = 0; i < NWT; ++i) {
+      const int n = n0 + wc * 32 * NI + 8 * NI * fg + 4 * i;  // the lane's four channels of tile i
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int row_off = ((32 * j + fr) * N + n) * 4;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2],
-                      v3 = acc[i][j][4 * q + 3];
-          const u32x4_t o = {__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)};
-          __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n + 4 * q < N ? row_off + 16 * q : (int)0x80000000u, 0, 0);
-        }
+      for (int j = 0; j < 8; ++j) {
+        const int row_off = ((16 * j + fr) * N + n) * 4;
+        const u32x4_t o = {__float_as_uint(acc[i][j][0]), __float_as_uint(acc[i][j][1]), __float_as_uint(acc[i][j][2]),
+                           __float_as_uint(acc[i][j][3])};
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n < N ? row_off : (int)0x80000000u, 0, 0);
       }
     }
     return;
@@ -736,31 +773,29 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
         res[j][it] = __builtin_bit_cast(
             u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, SANA_GEMM_NT_RES ? kBufferNt : 0));
   }
-  float bv[NI][16];
+  float bv[NI][8];
   if (HAS_BIAS) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+    for (int c = 0; c < NI; ++c)
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          bv[i][8 * half + 2 * e] = bf16_lo(bpk[i][half][e]);
-          bv[i][8 * half + 2 * e + 1] = bf16_hi(bpk[i][half][e]);
-        }
+      for (int e = 0; e < 4; ++e) {
+        bv[c][2 * e] = bf16_lo(bpk[c][e]);
+        bv[c][2 * e + 1] = bf16_hi(bpk[c][e]);
+      }
   }
   // Software-pipelined over the four groups of 32 tokens: step s of phase j converts piece s of group j
   // (accumulators -> activation -> LDS) and stores row chunk s of group j - 1 (LDS -> gate / residual -> global).
   // Handing a 16-byte-per-lane store to the memory pipeline keeps it busy for ~130 clocks, during which the
   // wave can issue VALU work but not another store: one store between two pieces of arithmetic costs a
   // fraction of what eight stores in a row cost.
-  auto convert_piece = [&](int j, int p) {  // p = 2 * i + half
-    const int i = p >> 1, half = p & 1;
-    const int tok = 32 * j + fr;
+  auto convert_piece = [&](int jg, int p) {  // group jg of 32 tokens = token tiles 2*jg, 2*jg + 1; p = NI * (tile & 1) + c
+    const int j = 2 * jg + p / NI, c = p % NI;  // c: the lane's c-th chunk of 8 channels = W tiles 2c, 2c + 1
+    const int tok = 16 * j + fr;
     float a8[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
-    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[i] + 8 * half);
-    const int chunk = 4 * i + 2 * fg + half;
+    for (int r = 0; r < 4; ++r) a8[r] = acc[2 * c][j][r], a8[4 + r] = acc[2 * c + 1][j][r];
+    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
+    const int chunk = NI * fg + c;
     *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
   };
   auto read_row = [&](int j, int it) {
@@ -908,7 +943,7 @@ struct GemmPlan {
 GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   GemmPlan pl = {false, 1, 0, 0};
   const int KT = (K + BK - 1) / BK, cu = compute_units();
-  const bool pipelined = K % 16 == 0 && K >= 64;
+  const bool pipelined = K % 32 == 0 && K >= 64;
   const double us_tile = pipelined ? 1.1 : 1.4, us_tile_small = 0.8, us_launch = 5.0, bytes_per_us = 3.0e6;
   double best = KT * us_tile;
   if (pipelined) {
@@ -1022,7 +1057,7 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
   uint16_t* c = static_cast<uint16_t*>(C);
   if (!taps && plan_gemm(M, N, K, W8).small)
     return launch_small<W8>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
-  if (K % 16 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
+  if (K % 32 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
     float* ws = aligned16(workspace) ? static_cast<float*>(workspace) : nullptr;
     // Mixed channel tiling: the first n_wide channels in 256-wide tiles, the rest in 192-wide ones, as two launches
     // over disjoint column ranges of C, when that needs fewer rounds of the chip than either width alone (qkv at
