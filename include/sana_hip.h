@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 5
+#define SANA_HIP_ABI_VERSION 6
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -297,6 +297,20 @@ int sana_hip_add_layernorm_modulate(const void* x, const void* y, const void* sc
  */
 int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, int N, int K,
                         int64_t ldw, int64_t ldo, void* stream);
+
+/* Softmax attention of many queries over a short key set, bf16: the core of the block's cross-attention to the
+ * text tokens (diffusion/model/nets/sana_blocks.py:69-98: F.scaled_dot_product_attention(q, k, v, attn_mask) at
+ * :92, scale = head_dim ** -0.5, and the additive mask (1 - mask) * -10000 of :89-90).
+ *   q:   bf16 [B][N][H*d] with row stride ldq (the q_linear output as it is: no head transpose);
+ *   kv:  bf16 [B][Nk][2][H*d] with row stride ldkv >= 2*H*d (the kv_linear output: keys, then values);
+ *   key_bias: fp32 [B] rows of Nk values bias_stride apart, added to the scaled scores of every head and query
+ *        (0 / -10000 for the reference's padding mask), or NULL;
+ *   out: bf16 [B][N][H*d] with row stride ldo (what proj reads).
+ * Probabilities are rounded to bf16 before they multiply v, as fused attention kernels do; sums in fp32.
+ * Nk <= 320, 64 < d <= 112, d % 8 == 0 (Sana: 2240 / 20 = 112, 1152 / 16 = 72); SANA_ERR_SHAPE otherwise. */
+int sana_hip_cross_attention(const void* q, const void* kv, const float* key_bias, void* out, int B, int N,
+                             int Nk, int H, int d, int64_t ldq, int64_t ldkv, int64_t ldo,
+                             int64_t bias_stride, float scale, void* stream);
 
 /* Gated residual update as one elementwise pass:
  *   out[m][:] = residual[m][:] + gate[m / rows_per_gate][:] * y[m][:]

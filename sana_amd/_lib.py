@@ -59,6 +59,8 @@ SIGNATURES = {
                                                 c_int, c_void_p]),
     "sana_hip_gate_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64,
                                        c_int64, c_int, c_int64, c_int, c_void_p]),
+    "sana_hip_cross_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                         c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
     "sana_hip_layernorm_modulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                             c_int64, c_int64, c_int, c_int64, c_float, c_int, c_void_p]),
 }

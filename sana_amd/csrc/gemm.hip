@@ -392,6 +392,163 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
 }
 
 
+// Epilogue of the pipelined kernels.  acc[i][j][r] (MFMA 16x16 tiles: i = channel tile of the wave, j = token tile):
+// token m0 + wt*128 + 16*j + lane%16, channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  bpk: the lane's 8*NI bias
+// values, packed (the caller requests them ahead of its last k-tile so that their latency hides behind its MFMAs).
+template <int EPI, int NI, bool SPLIT>
+__device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u32x4_t (&bpk)[NI], unsigned char* smem,
+                                              const EpiArgs& ep, uint16_t* __restrict__ C, int M, int N, int64_t ldc,
+                                              int m0, int n0) {
+  constexpr int NWT = 2 * NI;
+  constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wc = wave & 1, wt = wave >> 1;
+  const int fr = lane & 15, fg = lane >> 4;
+  const int o_chunk = lane & 15, o_rsub = lane >> 4;
+  const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
+  const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
+  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 16*j + lane%16,
+  // channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  The wave's sub-tile goes through its own 32 KB of
+  // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
+  // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
+  // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
+  if (SPLIT) {
+    // raw accumulators -> partial[z][M][N] (fp32, dense): a lane owns 16 consecutive channels of one token per
+    // MFMA tile, stored as four 16-byte pieces through a buffer resource over the wave's rows of this range's
+    // plane (rows past M fall outside it and are dropped; channel pieces past N get the idle offset)
+    const int prow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;
+    const int prows = max(0, min(128, M - prow0));
+    float* plane = reinterpret_cast<float*>(C) + ((int64_t)blockIdx.y * M + prow0) * N;
+    const __amdgpu_buffer_rsrc_t rsrc_p =
+        __builtin_amdgcn_make_buffer_rsrc(plane, 0, (int)((int64_t)prows * N * 4), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < NWT; ++i) {
+      const int n = n0 + wc * 32 * NI + 8 * NI * fg + 4 * i;  // the lane's four channels of tile i
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row_off = ((16 * j + fr) * N + n) * 4;
+        const u32x4_t o = {__float_as_uint(acc[i][j][0]), __float_as_uint(acc[i][j][1]), __float_as_uint(acc[i][j][2]),
+                           __float_as_uint(acc[i][j][3])};
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n < N ? row_off : (int)0x80000000u, 0, 0);
+      }
+    }
+    return;
+  }
+  __syncthreads();  // every wave is done with the operand tiles
+  unsigned char* stg = smem + wave * 32768;
+  // Global accesses of the epilogue are buffer loads / stores on the wave's 128 rows of C (and of the
+  // residual): a row costs one vector add for its offset, rows past M and channel pieces past N fall
+  // outside the resource (loads return zero, stores are dropped) -- no 64-bit address arithmetic, no
+  // per-row predication.
+  const int wrow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;  // first row of this wave (a scalar: it goes into resources)
+  const int wrows = max(0, min(128, M - wrow0));          // its rows that exist
+  const int idle_off = (int)0x80000000u;
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+      C + (int64_t)wrow0 * ldc, 0, wrows ? (int)((((int64_t)wrows - 1) * ldc + N) * 2) : 0, 0x00020000);
+  const int c_off0 = o_live ? (o_rsub * (int)ldc + o_n) * 2 : idle_off, c_step = 4 * (int)ldc * 2;
+  // Gated residual: the residual rows this lane will add are requested now, a whole epilogue ahead
+  // of their use (128 registers that the main loop no longer needs; asking for them before the last
+  // k-tile makes the compiler spill).
+  u32x4_t res[4][8];
+  const bool gated = EPI == SANA_EPI_GATE_RES;
+  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(gated ? ep.res + (int64_t)wrow0 * ep.ldr : nullptr), 0,
+      gated && wrows ? (int)((((int64_t)wrows - 1) * ep.ldr + N) * 2) : 0, 0x00020000);
+  const int r_off0 = o_live ? (o_rsub * (int)ep.ldr + o_n) * 2 : idle_off, r_step = 4 * (int)ep.ldr * 2;
+  if (EPI == SANA_EPI_GATE_RES) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int it = 0; it < 8; ++it)
+        res[j][it] = __builtin_bit_cast(
+            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, SANA_GEMM_NT_RES ? kBufferNt : 0));
+  }
+  float bv[NI][8];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int c = 0; c < NI; ++c)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bv[c][2 * e] = bf16_lo(bpk[c][e]);
+        bv[c][2 * e + 1] = bf16_hi(bpk[c][e]);
+      }
+  }
+  // Software-pipelined over the four groups of 32 tokens: step s of phase j converts piece s of group j
+  // (accumulators -> activation -> LDS) and stores row chunk s of group j - 1 (LDS -> gate / residual -> global).
+  // Handing a 16-byte-per-lane store to the memory pipeline keeps it busy for ~130 clocks, during which the
+  // wave can issue VALU work but not another store: one store between two pieces of arithmetic costs a
+  // fraction of what eight stores in a row cost.
+  auto convert_piece = [&](int jg, int p) {  // group jg of 32 tokens = token tiles 2*jg, 2*jg + 1; p = NI * (tile & 1) + c
+    const int j = 2 * jg + p / NI, c = p % NI;  // c: the lane's c-th chunk of 8 channels = W tiles 2c, 2c + 1
+    const int tok = 16 * j + fr;
+    float a8[8];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) a8[r] = acc[2 * c][j][r], a8[4 + r] = acc[2 * c + 1][j][r];
+    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
+    const int chunk = NI * fg + c;
+    *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
+  };
+  auto read_row = [&](int j, int it) {
+    const int row = 32 * j + it * 4 + o_rsub;
+    return *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
+  };
+#pragma unroll
+  for (int j = 0; j <= 4; ++j) {
+    const int js = j - 1;  // the group whose rows are stored in this phase
+    // The lane's eight gate values, as floats.  One gate row serves the whole group of 32 tokens unless a
+    // batch boundary runs through it: then the rows from m_switch on take the next gate row (gates are per
+    // batch entry; entries shorter than 32 tokens take the slow way, a division per row).
+    const int m_first = wrow0 + 32 * js;
+    int m_switch = 0;
+    bool two_gates = false;
+    float gf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // no gate: 1.0, a plain residual add
+    u32x4_t o_next = {0u, 0u, 0u, 0u};
+    if (js >= 0) {
+      if (EPI == SANA_EPI_GATE_RES) {
+        const int g_first = m_first / ep.rows_per_gate;
+        m_switch = (g_first + 1) * ep.rows_per_gate;
+        two_gates = ep.gate && m_switch < min(m_first + 32, M);
+        if (ep.gate && o_live && m_first < M) {
+          const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            gf[2 * e] = bf16_lo(gate[e]);
+            gf[2 * e + 1] = bf16_hi(gate[e]);
+          }
+        }
+      }
+      o_next = read_row(js, 0);  // wave-private LDS is in order: the group's writes are behind it
+    }
+#pragma unroll
+    for (int st = 0; st < 8; ++st) {
+      u32x4_t o = o_next;
+      if (js >= 0 && st + 1 < 8) o_next = read_row(js, st + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j < 4 && st < 2 * NI) convert_piece(j, st);
+      __builtin_amdgcn_sched_barrier(0);
+      if (js >= 0) {
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[js][st]);
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, SANA_GEMM_NT_STORE ? kBufferNt : 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (js >= 0 && two_gates) {  // uniform, rare: rows behind the boundary are redone with their own gate row and stored again
+#pragma unroll 1
+      for (int it = 0; it < 8; ++it) {
+        const int row = 32 * js + it * 4 + o_rsub, m = wrow0 + row;
+        if (o_live && m >= m_switch && m < M) {
+          const u32x4_t y = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
+          const u32x4_t r = __builtin_bit_cast(
+              u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * js + it) * r_step, 0, 0));
+          const u32x4_t g2 = *reinterpret_cast<const u32x4_t*>(
+              ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
+          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * js + it) * c_step, 0, 0);
+        }
+      }
+    }
+  }
+}
+
 // ============================================================================
 // Pipelined kernel (K % 32 == 0, K >= 64; bf16 and int8 weights): 256 threads, one
 // wave per SIMD with the whole register file (256 accumulators + 256 VGPRs), each
@@ -694,9 +851,6 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       bpk[c] = (ep.bias && n < N) ? *reinterpret_cast<const u32x4_t*>(ep.bias + n) : u32x4_t{0u, 0u, 0u, 0u};
     }
   }
-  const int o_chunk = lane & 15, o_rsub = lane >> 4;
-  const int o_n = n0 + wc * 32 * NI + o_chunk * 8;
-  const bool o_live = o_chunk < 4 * NI && o_n < N;  // a staged row holds 4*NI chunks (the row pitch stays 256 bytes)
   {  // last k-tile: no successor, and K % 64 may leave one k-step of 32 instead of two
     const unsigned char* st = smem + ((KT - 1) & 1) * 2 * TILE_BYTES;
     const int steps = (K - (KT - 1) * BK) / 32;
@@ -717,146 +871,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
   }
 
-  // ---- epilogue.  acc[i][j][r]: token m0 + wt*128 + 16*j + lane%16,
-  // channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  The wave's sub-tile goes through its own 32 KB of
-  // LDS ([128 tokens][256 bytes], 16-byte chunks XOR-swizzled by token % 16) and comes back
-  // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
-  // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
-  if (SPLIT) {
-    // raw accumulators -> partial[z][M][N] (fp32, dense): a lane owns 16 consecutive channels of one token per
-    // MFMA tile, stored as four 16-byte pieces through a buffer resource over the wave's rows of this range's
-    // plane (rows past M fall outside it and are dropped; channel pieces past N get the idle offset)
-    const int prow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;
-    const int prows = max(0, min(128, M - prow0));
-    float* plane = reinterpret_cast<float*>(C) + ((int64_t)blockIdx.y * M + prow0) * N;
-    const __amdgpu_buffer_rsrc_t rsrc_p =
-        __builtin_amdgcn_make_buffer_rsrc(plane, 0, (int)((int64_t)prows * N * 4), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < NWT; ++i) {
-      const int n = n0 + wc * 32 * NI + 8 * NI * fg + 4 * i;  // the lane's four channels of tile i
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int row_off = ((16 * j + fr) * N + n) * 4;
-        const u32x4_t o = {__float_as_uint(acc[i][j][0]), __float_as_uint(acc[i][j][1]), __float_as_uint(acc[i][j][2]),
-                           __float_as_uint(acc[i][j][3])};
-        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n < N ? row_off : (int)0x80000000u, 0, 0);
-      }
-    }
-    return;
-  }
-  __syncthreads();  // every wave is done with the operand tiles
-  unsigned char* stg = smem + wave * 32768;
-  // Global accesses of the epilogue are buffer loads / stores on the wave's 128 rows of C (and of the
-  // residual): a row costs one vector add for its offset, rows past M and channel pieces past N fall
-  // outside the resource (loads return zero, stores are dropped) -- no 64-bit address arithmetic, no
-  // per-row predication.
-  const int wrow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;  // first row of this wave (a scalar: it goes into resources)
-  const int wrows = max(0, min(128, M - wrow0));          // its rows that exist
-  const int idle_off = (int)0x80000000u;
-  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
-      C + (int64_t)wrow0 * ldc, 0, wrows ? (int)((((int64_t)wrows - 1) * ldc + N) * 2) : 0, 0x00020000);
-  const int c_off0 = o_live ? (o_rsub * (int)ldc + o_n) * 2 : idle_off, c_step = 4 * (int)ldc * 2;
-  // Gated residual: the residual rows this lane will add are requested now, a whole epilogue ahead
-  // of their use (128 registers that the main loop no longer needs; asking for them before the last
-  // k-tile makes the compiler spill).
-  u32x4_t res[4][8];
-  const bool gated = EPI == SANA_EPI_GATE_RES;
-  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(gated ? ep.res + (int64_t)wrow0 * ep.ldr : nullptr), 0,
-      gated && wrows ? (int)((((int64_t)wrows - 1) * ep.ldr + N) * 2) : 0, 0x00020000);
-  const int r_off0 = o_live ? (o_rsub * (int)ep.ldr + o_n) * 2 : idle_off, r_step = 4 * (int)ep.ldr * 2;
-  if (EPI == SANA_EPI_GATE_RES) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int it = 0; it < 8; ++it)
-        res[j][it] = __builtin_bit_cast(
-            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * j + it) * r_step, 0, SANA_GEMM_NT_RES ? kBufferNt : 0));
-  }
-  float bv[NI][8];
-  if (HAS_BIAS) {
-#pragma unroll
-    for (int c = 0; c < NI; ++c)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        bv[c][2 * e] = bf16_lo(bpk[c][e]);
-        bv[c][2 * e + 1] = bf16_hi(bpk[c][e]);
-      }
-  }
-  // Software-pipelined over the four groups of 32 tokens: step s of phase j converts piece s of group j
-  // (accumulators -> activation -> LDS) and stores row chunk s of group j - 1 (LDS -> gate / residual -> global).
-  // Handing a 16-byte-per-lane store to the memory pipeline keeps it busy for ~130 clocks, during which the
-  // wave can issue VALU work but not another store: one store between two pieces of arithmetic costs a
-  // fraction of what eight stores in a row cost.
-  auto convert_piece = [&](int jg, int p) {  // group jg of 32 tokens = token tiles 2*jg, 2*jg + 1; p = NI * (tile & 1) + c
-    const int j = 2 * jg + p / NI, c = p % NI;  // c: the lane's c-th chunk of 8 channels = W tiles 2c, 2c + 1
-    const int tok = 16 * j + fr;
-    float a8[8];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) a8[r] = acc[2 * c][j][r], a8[4 + r] = acc[2 * c + 1][j][r];
-    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
-    const int chunk = NI * fg + c;
-    *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
-  };
-  auto read_row = [&](int j, int it) {
-    const int row = 32 * j + it * 4 + o_rsub;
-    return *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-  };
-#pragma unroll
-  for (int j = 0; j <= 4; ++j) {
-    const int js = j - 1;  // the group whose rows are stored in this phase
-    // The lane's eight gate values, as floats.  One gate row serves the whole group of 32 tokens unless a
-    // batch boundary runs through it: then the rows from m_switch on take the next gate row (gates are per
-    // batch entry; entries shorter than 32 tokens take the slow way, a division per row).
-    const int m_first = wrow0 + 32 * js;
-    int m_switch = 0;
-    bool two_gates = false;
-    float gf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // no gate: 1.0, a plain residual add
-    u32x4_t o_next = {0u, 0u, 0u, 0u};
-    if (js >= 0) {
-      if (EPI == SANA_EPI_GATE_RES) {
-        const int g_first = m_first / ep.rows_per_gate;
-        m_switch = (g_first + 1) * ep.rows_per_gate;
-        two_gates = ep.gate && m_switch < min(m_first + 32, M);
-        if (ep.gate && o_live && m_first < M) {
-          const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            gf[2 * e] = bf16_lo(gate[e]);
-            gf[2 * e + 1] = bf16_hi(gate[e]);
-          }
-        }
-      }
-      o_next = read_row(js, 0);  // wave-private LDS is in order: the group's writes are behind it
-    }
-#pragma unroll
-    for (int st = 0; st < 8; ++st) {
-      u32x4_t o = o_next;
-      if (js >= 0 && st + 1 < 8) o_next = read_row(js, st + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      if (j < 4 && st < 2 * NI) convert_piece(j, st);
-      __builtin_amdgcn_sched_barrier(0);
-      if (js >= 0) {
-        if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[js][st]);
-        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, SANA_GEMM_NT_STORE ? kBufferNt : 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (js >= 0 && two_gates) {  // uniform, rare: rows behind the boundary are redone with their own gate row and stored again
-#pragma unroll 1
-      for (int it = 0; it < 8; ++it) {
-        const int row = 32 * js + it * 4 + o_rsub, m = wrow0 + row;
-        if (o_live && m >= m_switch && m < M) {
-          const u32x4_t y = *reinterpret_cast<const u32x4_t*>(stg + row * 256 + ((o_chunk ^ (row & 15)) << 4));
-          const u32x4_t r = __builtin_bit_cast(
-              u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * js + it) * r_step, 0, 0));
-          const u32x4_t g2 = *reinterpret_cast<const u32x4_t*>(
-              ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
-          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * js + it) * c_step, 0, 0);
-        }
-      }
-    }
-  }
+  finish_tile16<EPI, NI, SPLIT>(acc, bpk, smem, ep, C, M, N, ldc, m0, n0);
 }
 
 // Second half of a split-k GEMM: partial[S][M][N] (fp32) -> C = epilogue(sum over the S k-ranges, added in

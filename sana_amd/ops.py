@@ -546,6 +546,47 @@ def add_layernorm_modulate(x: torch.Tensor, y: torch.Tensor, scale: torch.Tensor
     _lib.check(code, "sana_hip_add_layernorm_modulate")
     return total.view(B, Ntok, C), out.view(B, Ntok, C)
 
+CROSS_ATTN_MAX_KEYS = 320     # keys of one (batch, head) that fit LDS together with their values
+
+
+def cross_attention_supported(head_dim: int, n_keys: int) -> bool:
+    """Shapes sana_hip_cross_attention takes: one head's keys and values held in LDS."""
+    return 64 < head_dim <= 112 and head_dim % 8 == 0 and 0 < n_keys <= CROSS_ATTN_MAX_KEYS
+
+
+def cross_attention(q: torch.Tensor, kv: torch.Tensor, num_heads: int, key_bias: Optional[torch.Tensor] = None,
+                    scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(q k^T * scale + key_bias) v per head, bf16.  q: [B, N, C] (q_linear's output), kv: [B, Nk, 2C]
+    (kv_linear's output: keys then values), key_bias: fp32 [B, Nk] added to every head's and query's scores
+    (0 / -10000 for a padding mask) or None.  Returns [B, N, C], token-major like q."""
+    _need_cuda(q, kv, key_bias)
+    if q.dim() != 3 or kv.dim() != 3 or q.dtype != torch.bfloat16 or kv.dtype != torch.bfloat16:
+        raise SanaHipError("cross_attention needs bf16 q [B, N, C] and kv [B, Nk, 2C]")
+    B, N, C = q.shape
+    Nk = kv.shape[1]
+    if kv.shape[0] != B or kv.shape[2] != 2 * C or C % num_heads:
+        raise SanaHipError(f"kv {tuple(kv.shape)} does not match q {tuple(q.shape)} with {num_heads} heads")
+    d = C // num_heads
+    if not cross_attention_supported(d, Nk):
+        raise SanaHipError(f"cross_attention holds one head's keys in LDS: head_dim {d} (72 .. 112), {Nk} keys (<= 320)")
+    if q.stride(2) != 1 or kv.stride(2) != 1 or q.stride(0) != N * q.stride(1) or kv.stride(0) != Nk * kv.stride(1):
+        raise SanaHipError("cross_attention needs q and kv rows with unit inner stride, batch entries back to back")
+    if key_bias is not None:
+        if key_bias.dtype != torch.float32 or key_bias.shape != (B, Nk) or key_bias.stride(1) != 1:
+            raise SanaHipError("key_bias must be fp32 [B, Nk] with unit inner stride")
+    if out is None:
+        out = torch.empty(B, N, C, dtype=torch.bfloat16, device=q.device)
+    elif out.shape != (B, N, C) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise SanaHipError("out must be a contiguous bf16 [B, N, C] tensor")
+    if B * N == 0:
+        return out
+    code = _lib.load().sana_hip_cross_attention(
+        q.data_ptr(), kv.data_ptr(), None if key_bias is None else key_bias.data_ptr(), out.data_ptr(), B, N, Nk,
+        num_heads, d, q.stride(1), kv.stride(1), C, 0 if key_bias is None else key_bias.stride(0),
+        float(d ** -0.5 if scale is None else scale), _stream())
+    _lib.check(code, "sana_hip_cross_attention")
+    return out
+
 
 def gate_residual(y: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
     """residual + gate * y in one pass with the stock op pair's two roundings; y, residual: [B, N, C] bf16;
