@@ -251,6 +251,14 @@ def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_onl
         event_time_us(lambda: ops.dwconv3x3_silu_gate(u, dw, db, True), iters, warmup),
         "M*2H*2 B read + M*H*2 B write + weights")
     del u
+    # cross-attention to 300 text tokens, 20 heads of 112 (the block's num_heads): two products of 2*M*300*C flops
+    xq = torch.randn(B, N, C, generator=g).bfloat16().to(dev)
+    xkv = torch.randn(B, 300, 2 * C, generator=g).bfloat16().to(dev)
+    xo = torch.empty_like(xq)
+    add("cross_attention_300_keys", "mfma", 4 * M * 300 * C,
+        event_time_us(lambda: ops.cross_attention(xq, xkv, HEADS_X, out=xo), iters, warmup),
+        "4*M*Nk*C flops (q k^T and p v), Nk=300, 20 heads of 112; also moves 2*M*C*2 B (147 MB)")
+    del xq, xo
     x_ln = torch.randn(B, N, C, generator=g).bfloat16().to(dev)
     mod = (torch.randn(B, 6, C, generator=g) * 0.5).bfloat16().to(dev)
     add("layernorm_modulate", "hbm", 2 * M * C * 2,

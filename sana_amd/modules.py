@@ -763,8 +763,8 @@ def t2i_modulate(x, shift, scale):
 
 class MultiHeadCrossAttention(nn.Module):
     """Cross-attention to the text tokens (reference: sana_blocks.py:48-98, the scaled_dot_product_attention
-    branch): bf16 inference runs q_linear / proj on this library's GEMM and the attention itself as the short-key
-    softmax kernel; everything else (other dtypes, training, more than 320 text tokens, 4-d masks) is stock ops."""
+    branch): bf16 inference runs the attention itself as the short-key softmax kernel between stock linears;
+    everything else (other dtypes, training, more than 320 text tokens, 4-d masks) is stock ops."""
 
     def __init__(self, d_model, num_heads, attn_drop=0.0, proj_drop=0.0, qk_norm=False, **block_kwargs):
         super().__init__()
@@ -808,22 +808,23 @@ class MultiHeadCrossAttention(nn.Module):
     def forward(self, x, cond, mask=None):
         B, N, C = x.shape
         H, d = self.num_heads, self.head_dim
-        # HIP path: q_linear and proj as GEMMs of this library at their native width, softmax(q k^T) v over the
-        # short text sequence as one kernel that reads q and writes its output token-major (no head transposes)
+        # HIP path: softmax(q k^T) v over the short text sequence as one kernel that reads q_linear's output and
+        # writes proj's input token-major (no head transposes, no padded head_dim)
         if (x.is_cuda and x.dtype == torch.bfloat16 and cond.dtype == torch.bfloat16 and not torch.is_grad_enabled()
                 and cond.dim() == 3 and cond.shape[0] == B and ops.cross_attention_supported(d, cond.shape[1])
                 and (mask is None or (mask.ndim == 2 and tuple(mask.shape) == (B, cond.shape[1])))
                 and self.q_linear.weight.dtype == torch.bfloat16):
-            q = ops.gemm_bf16(x.reshape(B * N, C), self.q_linear.weight, self.q_linear.bias, "bias").view(B, N, C)
-            kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)           # [B, Nk, 2C]: a few hundred rows
+            # (the three linears stay library GEMM calls at their native width: at 16384 rows they take what this
+            # library's GEMM takes, at a few hundred rows they are faster, and they cost less host time per call)
+            q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
+            kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)           # [B, Nk, 2C]
             if not isinstance(self.q_norm, nn.Identity):
                 q = self.q_norm(q)
             if not isinstance(self.k_norm, nn.Identity):
                 kv = torch.cat([self.k_norm(kv[:, :, :C]), kv[:, :, C:]], dim=-1)
             bias = None if mask is None else (1.0 - mask.to(torch.float32)) * -10000.0   # sana_blocks.py:89-90
             o = ops.cross_attention(q, kv, H, bias)
-            o = ops.gemm_bf16(o.view(B * N, C), self.proj.weight, self.proj.bias, "bias").view(B, N, C)
-            return self.proj_drop(o)
+            return self.proj_drop(F.linear(o, self.proj.weight, self.proj.bias))
         if x.is_cuda:
             stock_path("cross-attention",
                        f"the HIP path is bf16 inference with head_dim 72 .. 112, at most {ops.CROSS_ATTN_MAX_KEYS} text tokens "
