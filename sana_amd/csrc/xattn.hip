@@ -37,7 +37,10 @@ template <int DK>
 __device__ __forceinline__ int xa_kkey(int row) {  // K rows of DK*64 bytes
   return DK == 4 ? (row & 15) : DK == 3 ? ((row >> 2) & 3) : DK == 2 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
-__device__ __forceinline__ int xa_vkey(int row) { return (row >> 1) & 7; }  // V^T rows of 640 bytes
+// V^T rows of 640 bytes: rows alternate between the two halves of the bank space, (row / 2) % 8 spreads a 16-row
+// fragment read over the 8 slots of a half; the (row / 16) % 4 term does the same for the transposing writes of
+// the staging pass, whose lanes hold one key at rows 8 apart
+__device__ __forceinline__ int xa_vkey(int row) { return ((row >> 1) ^ ((row >> 4) & 3)) & 7; }
 
 // position of key m inside its group of 32 in V^T (and in the probability operand)
 __device__ __forceinline__ int xa_vpos(int m) {
@@ -69,23 +72,44 @@ __global__ __launch_bounds__(64 * NW) void cross_attn_kernel(const uint16_t* __r
       __syncthreads();   // everyone is done with the previous head's K / V
       const uint16_t* kbase = kv + (int64_t)b * Nk * ldkv + (int64_t)h * d;
       const uint16_t* vbase = kbase + (int64_t)H * d;
-      for (int idx = tid; idx < XA_NKP * KCH; idx += 64 * NW) {
-        const int row = idx / KCH, c = idx - row * KCH;
-        u32x4_t val = {0u, 0u, 0u, 0u};
-        if (row < Nk && 8 * c < d) val = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)row * ldkv + 8 * c);
-        *reinterpret_cast<u32x4_t*>(sk + row * KPITCH + ((c ^ xa_kkey<DK>(row)) << 4)) = val;
+      // a thread's loads go out in batches of SB before the LDS writes of the batch (the rows come out of the L2: one
+      // load per round trip would make staging a chain of ~20 latencies)
+      constexpr int NT = 64 * NW, SB = 5;
+      for (int base = tid; base < XA_NKP * KCH; base += SB * NT) {
+        u32x4_t val[SB];
+#pragma unroll
+        for (int i = 0; i < SB; ++i) {
+          const int idx = base + i * NT, row = idx / KCH, c = idx - row * KCH;
+          val[i] = u32x4_t{0u, 0u, 0u, 0u};
+          if (row < Nk && 8 * c < d) val[i] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)row * ldkv + 8 * c);
+        }
+#pragma unroll
+        for (int i = 0; i < SB; ++i) {
+          const int idx = base + i * NT, row = idx / KCH, c = idx - row * KCH;
+          if (row < XA_NKP) *reinterpret_cast<u32x4_t*>(sk + row * KPITCH + ((c ^ xa_kkey<DK>(row)) << 4)) = val[i];
+        }
       }
       // V^T: a thread takes 8 channels of one key and scatters them over 8 rows
-      for (int idx = tid; idx < XA_NKP * DT * 2; idx += 64 * NW) {
-        const int row = idx / (DT * 2), c = idx - row * (DT * 2);
-        u32x4_t val = {0u, 0u, 0u, 0u};
-        if (row < Nk && 8 * c < d) val = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)row * ldkv + 8 * c);
-        const int p = xa_vpos(row);
+      for (int base = tid; base < XA_NKP * DT * 2; base += SB * NT) {
+        u32x4_t val[SB];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int dr = 8 * c + e;
-          const uint16_t x = (uint16_t)(e & 1 ? val[e >> 1] >> 16 : val[e >> 1] & 0xffffu);
-          *reinterpret_cast<uint16_t*>(sv + dr * XA_VPITCH + (((p >> 3) ^ xa_vkey(dr)) << 4) + (p & 7) * 2) = x;
+        for (int i = 0; i < SB; ++i) {
+          const int idx = base + i * NT, row = idx / (DT * 2), c = idx - row * (DT * 2);
+          val[i] = u32x4_t{0u, 0u, 0u, 0u};
+          if (row < Nk && 8 * c < d) val[i] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)row * ldkv + 8 * c);
+        }
+#pragma unroll
+        for (int i = 0; i < SB; ++i) {
+          const int idx = base + i * NT, row = idx / (DT * 2), c = idx - row * (DT * 2);
+          if (row < XA_NKP) {
+            const int p = xa_vpos(row);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int dr = 8 * c + e;
+              const uint16_t x = (uint16_t)(e & 1 ? val[i][e >> 1] >> 16 : val[i][e >> 1] & 0xffffu);
+              *reinterpret_cast<uint16_t*>(sv + dr * XA_VPITCH + (((p >> 3) ^ xa_vkey(dr)) << 4) + (p & 7) * 2) = x;
+            }
+          }
         }
       }
       for (int m = tid; m < XA_NKP; m += 64 * NW)
