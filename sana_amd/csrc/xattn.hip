@@ -29,7 +29,6 @@ namespace sana {
 namespace {
 
 constexpr int XA_NKP = 320;       // keys an LDS image holds (padded)
-constexpr int XA_KT = XA_NKP / 16;  // 16-key tiles
 constexpr int XA_VPITCH = XA_NKP * 2;  // bytes per row of V^T
 
 // 16-byte-slot swizzles that make 16 consecutive rows of one chunk hit 16 different bank groups
