@@ -265,7 +265,9 @@ def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_onl
         event_time_us(lambda: ops.layernorm_modulate(x_ln, mod[:, 1:2], mod[:, 0:1], 1e-6), iters, warmup),
         "M*C*2 B read + M*C*2 B write")
     for name, Nn, Kk, epi in (("gemm_qkv", 3 * C, C, None), ("gemm_proj_gate_residual", C, C, "gate_res"),
-                              ("gemm_inverted", 2 * HID, C, "bias_silu"), ("gemm_point_gate_residual", C, HID, "gate_res"),
+                              ("gemm_inverted", 2 * HID, C, "bias_silu"),
+                              ("gemm_inverted_bias_only", 2 * HID, C, "bias"),   # what the library figure beside it computes
+                              ("gemm_point_gate_residual", C, HID, "gate_res"),
                               ("gemm_inverted_w8a16", 2 * HID, C, "w8_bias_silu"),
                               ("gemm_inverted_w8a16_in_loop", 2 * HID, C, "w8_bias_silu_fused")):
         a = torch.randn(M, Kk, generator=g).bfloat16().to(dev)
