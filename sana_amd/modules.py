@@ -805,25 +805,51 @@ class MultiHeadCrossAttention(nn.Module):
             self.__dict__["_pad_cache"] = cache
         return cache[1]
 
-    def forward(self, x, cond, mask=None):
+    def _attend(self, x, cond, mask):
+        """The HIP path up to proj's input -- softmax(q k^T) v over the short text sequence as one kernel that reads
+        q_linear's output and writes proj's input token-major (no head transposes, no padded head_dim) -- or None
+        when the call is outside it."""
         B, N, C = x.shape
         H, d = self.num_heads, self.head_dim
-        # HIP path: softmax(q k^T) v over the short text sequence as one kernel that reads q_linear's output and
-        # writes proj's input token-major (no head transposes, no padded head_dim)
-        if (x.is_cuda and x.dtype == torch.bfloat16 and cond.dtype == torch.bfloat16 and not torch.is_grad_enabled()
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and cond.dtype == torch.bfloat16 and not torch.is_grad_enabled()
                 and cond.dim() == 3 and cond.shape[0] == B and ops.cross_attention_supported(d, cond.shape[1])
                 and (mask is None or (mask.ndim == 2 and tuple(mask.shape) == (B, cond.shape[1])))
                 and self.q_linear.weight.dtype == torch.bfloat16):
-            # (the three linears stay library GEMM calls at their native width: at 16384 rows they take what this
-            # library's GEMM takes, at a few hundred rows they are faster, and they cost less host time per call)
-            q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
-            kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)           # [B, Nk, 2C]
-            if not isinstance(self.q_norm, nn.Identity):
-                q = self.q_norm(q)
-            if not isinstance(self.k_norm, nn.Identity):
-                kv = torch.cat([self.k_norm(kv[:, :, :C]), kv[:, :, C:]], dim=-1)
-            bias = None if mask is None else (1.0 - mask.to(torch.float32)) * -10000.0   # sana_blocks.py:89-90
-            o = ops.cross_attention(q, kv, H, bias)
+            return None
+        # (q_linear and kv_linear stay library GEMM calls at their native width: at 16384 rows they take what this
+        # library's GEMM takes, at a few hundred rows they are faster, and they cost less host time per call)
+        q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
+        kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)           # [B, Nk, 2C]
+        if not isinstance(self.q_norm, nn.Identity):
+            q = self.q_norm(q)
+        if not isinstance(self.k_norm, nn.Identity):
+            kv = torch.cat([self.k_norm(kv[:, :, :C]), kv[:, :, C:]], dim=-1)
+        bias = None if mask is None else (1.0 - mask.to(torch.float32)) * -10000.0   # sana_blocks.py:89-90
+        return ops.cross_attention(q, kv, H, bias)
+
+    # rows from which proj + the block's residual add run as ONE GEMM of this library (its gated-residual epilogue
+    # with a gate of ones: x + (o W^T + b), the same two roundings as the stock linear and add) instead of a
+    # library GEMM and an elementwise pass; below it the library GEMM's shorter latency chain wins
+    RESIDUAL_GEMM_MIN_ROWS = 4096
+
+    def forward_residual(self, x, cond, mask=None):
+        """x + self(x, cond, mask) -- what the blocks compute (sana_multi_scale.py:154) -- with the add inside the
+        projection GEMM's epilogue when the call is on the HIP path and large enough."""
+        B, N, C = x.shape
+        if B * N >= self.RESIDUAL_GEMM_MIN_ROWS and isinstance(self.proj_drop, nn.Dropout) and self.proj_drop.p == 0.0:
+            o = self._attend(x, cond, mask)
+            if o is not None:
+                ones = self.__dict__.get("_ones_gate")
+                if ones is None or ones.device != x.device or ones.shape[-1] != C:
+                    ones = self.__dict__["_ones_gate"] = torch.ones(1, 1, C, dtype=torch.bfloat16, device=x.device)
+                return ops.gemm_gate_residual(o, self.proj.weight, self.proj.bias, ones.expand(B, 1, C), x)
+        return x + self(x, cond, mask)
+
+    def forward(self, x, cond, mask=None):
+        B, N, C = x.shape
+        H, d = self.num_heads, self.head_dim
+        o = self._attend(x, cond, mask)
+        if o is not None:
             return self.proj_drop(F.linear(o, self.proj.weight, self.proj.bias))
         if x.is_cuda:
             stock_path("cross-attention",
@@ -902,8 +928,13 @@ class SanaMSBlock(nn.Module):
                 x = ops.gate_residual(self.attn(h, HW=HW, rotary_emb=image_rotary_emb), gate_msa, x)
             else:
                 x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
-            # the cross-attention's residual add and norm2 + modulate in one pass
-            x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask), scale_mlp, shift_mlp, self.norm2.eps)
+            if B * N >= self.cross_attn.RESIDUAL_GEMM_MIN_ROWS:
+                # the cross-attention's residual add inside its projection GEMM, then norm2 + modulate
+                x = self.cross_attn.forward_residual(x, y, mask)
+                h = ops.layernorm_modulate(x, scale_mlp, shift_mlp, self.norm2.eps)
+            else:
+                # the cross-attention's residual add and norm2 + modulate in one pass
+                x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask), scale_mlp, shift_mlp, self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)
         stock_path("SanaMSBlock LayerNorm / modulate / gate / residual seams",
                    f"the fused seams are bf16 inference only (C % 8 == 0, C <= 8192); got x {x.dtype}, t {t.dtype}, C = {C}, "
@@ -1019,7 +1050,7 @@ class SanaVideoMSBlock(nn.Module):
             x = self.attn.forward_gated(h, gate_msa, x, **attn_kw)
         else:
             x = self._gate_residual(x, gate_msa, self.attn(h, **attn_kw))
-        x = x + self.cross_attn(x, y, mask=mask)
+        x = self.cross_attn.forward_residual(x, y, mask=mask)
         mlp_kw = {"HW": THW}
         if chunk_index is not None:
             mlp_kw["chunk_index"] = chunk_index[:]
@@ -1055,7 +1086,7 @@ class SanaVideoMSBlock(nn.Module):
                 x_sa, kv_cache = x_sa
             feats["x_self_attn"] = x_sa
             x = self._gate_residual(x, gate_msa, x_sa)
-        x = x + self.cross_attn(x, y, mask=mask)
+        x = self.cross_attn.forward_residual(x, y, mask=mask)
         feats["x_cross_attn"] = x
         mlp_kw = {"HW": THW}
         if chunk_index is not None:

@@ -106,3 +106,31 @@ def test_cross_attention_module_matches_oracle(cuda, C, H, B, N, Nk, masked):
         ref = om.float()(x.float(), y.float(), mask)
     mx = (out.cpu().double() - ref.double()).abs().max().item()
     assert mx <= 2e-2 and rel_l2(out.cpu(), ref) <= 1e-2, (mx, rel_l2(out.cpu(), ref))
+
+
+def test_residual_add_inside_the_projection_gemm(cuda):
+    """x + cross_attn(x, y): from 4096 rows on the add is the projection GEMM's epilogue (two roundings, as the stock
+    linear + add); against the oracle module's output plus x, and against the unfused composition of this module (same
+    products, another fp32 summation order inside the two GEMMs: at most one bf16 ulp of the sum apart)."""
+    C, H, B, N, Nk = 2240, 20, 2, 2048, 300
+    g = torch.Generator().manual_seed(3)
+    om = O.MultiHeadCrossAttention(C, H)
+    with torch.no_grad():
+        for p in om.parameters():
+            p.copy_(torch.nn.init.trunc_normal_(torch.empty(p.shape), std=0.02, generator=g))
+    om = om.bfloat16()
+    hm = S.modules.MultiHeadCrossAttention(C, H).bfloat16()
+    hm.load_state_dict(om.state_dict())
+    hm = hm.to(cuda)
+    assert B * N >= hm.RESIDUAL_GEMM_MIN_ROWS
+    x = torch.randn(B, N, C, generator=g).bfloat16()
+    y = torch.randn(B, Nk, C, generator=g).bfloat16()
+    with torch.no_grad():
+        fused = hm.forward_residual(x.to(cuda), y.to(cuda))
+        plain = x.to(cuda) + hm(x.to(cuda), y.to(cuda))
+        ref = x.float() + om.float()(x.float(), y.float())
+    assert (fused.float() - plain.float()).abs().max().item() <= 2 ** -7 * plain.float().abs().max().item()
+    mx = (fused.cpu().double() - ref.double()).abs()
+    assert (mx > 2e-2 + 2.0 ** -7 * ref.double().abs()).sum().item() == 0 and rel_l2(fused.cpu(), ref) <= 1e-2
+    small = hm.forward_residual(x[:, :64].to(cuda), y.to(cuda))       # below the threshold: the composition itself
+    assert torch.equal(small, x[:, :64].to(cuda) + hm(x[:, :64].to(cuda), y.to(cuda)))
