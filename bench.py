@@ -314,20 +314,43 @@ def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_onl
     del buf, ot
 
 
-def images_per_s(dev, w8: bool, steps: int, warmup: int, B: int = 16) -> float:
-    """1024px shape of Sana-1.6B: B images of N=1024 tokens; DiT blocks of one denoising step only."""
+_STATES = {}
+
+
+def make_blocks(dev, w8: bool = False):
+    """The DEPTH blocks of Sana-1.6B (random init, one seed per block), bf16 or W8A16."""
+    import sana_amd as S
+
+    blocks = []
+    for i in range(DEPTH):
+        blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
+        if i not in _STATES:
+            _STATES[i] = make_state(i)
+        blk.load_state_dict(_STATES[i])
+        blk = blk.to(dev)
+        blocks.append(blk.quantize_w8_() if w8 else blk)
+    return blocks
+
+
+def chain_step(blocks, cond, x, y, t, HW):
+    """One denoising step's block loop (sana_multi_scale.py:368-383); ``cond``: the blocks' StepConditioning,
+    evaluated inside the step (text keys / values and modulation rows of all blocks in two launches)."""
+    h = x
+    for blk, c in zip(blocks, cond(y, t)):
+        h = blk(h, y, t, None, HW, None, **c)
+    return h
+
+
+def images_per_s(dev, blocks, steps: int, warmup: int, B: int = 16) -> float:
+    """1024px shape of Sana-1.6B: B images of N=1024 tokens; the DEPTH DiT blocks of one denoising step only."""
     import sana_amd as S
 
     HW = (32, 32)
-    blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
-    blk.load_state_dict(make_state(0))
-    blk = blk.to(dev)
-    if w8:
-        blk.quantize_w8_()
+    cond = S.StepConditioning(blocks)
     x, y, t = (a.bfloat16().to(dev) for a in make_inputs(B, HW[0] * HW[1]))
     with torch.no_grad():
-        t_us = event_time_us(lambda: blk(x, y, t, HW=HW), steps, warmup)
-    return B / (DEPTH * t_us * 1e-6)
+        t_us = event_time_us(lambda: chain_step(blocks, cond, x, y, t, HW), steps, warmup)
+    return B / (t_us * 1e-6)
 
 
 def video_block_ms(dev, steps: int = 10, warmup: int = 3) -> float:
@@ -479,18 +502,12 @@ def main():
         return
     B, HW = 1, (128, 128)
     N = HW[0] * HW[1]
-    blocks = []
-    for i in range(DEPTH):
-        blk = S.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv").bfloat16()
-        blk.load_state_dict(make_state(i))
-        blocks.append(blk.to(dev))
+    blocks = make_blocks(dev)
+    cond = S.StepConditioning(blocks)
     x, y, t = (a.bfloat16().to(dev) for a in make_inputs(B, N))
 
     def step():
-        h = x
-        for blk in blocks:
-            h = blk(h, y, t, None, HW, None)
-        return h
+        return chain_step(blocks, cond, x, y, t, HW)
 
     with torch.no_grad():
         for _ in range(args.warmup):
@@ -506,10 +523,12 @@ def main():
         block_ms = ms_per_step / DEPTH
 
         kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev, stock_conv=args.stock_conv)
-        ips_bf16 = images_per_s(dev, False, 20, 5)
-        ips_w8 = images_per_s(dev, True, 20, 5)
-        one_image_ms = 1e3 / images_per_s(dev, False, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
-        one_image_ms_w8 = 1e3 / images_per_s(dev, True, 20, 5, B=1)
+        ips_bf16 = images_per_s(dev, blocks, 5, 2)
+        one_image_ms = 1e3 / images_per_s(dev, blocks, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
+        del cond, blocks
+        blocks = make_blocks(dev, w8=True)
+        ips_w8 = images_per_s(dev, blocks, 5, 2)
+        one_image_ms_w8 = 1e3 / images_per_s(dev, blocks, 20, 5, B=1)
         video_ms = video_block_ms(dev)
     del blocks
     torch.cuda.empty_cache()
@@ -530,7 +549,7 @@ def main():
         "images_per_s_1024px": {"bf16": round(ips_bf16, 2), "w8a16": round(ips_w8, 2),
                                 "one_image_step_ms_bf16": round(one_image_ms, 3),
                                 "one_image_step_ms_w8a16": round(one_image_ms_w8, 3),
-                                "note": "B=16, N=1024: B / (20 x block latency); DiT blocks of one denoising step only "
+                                "note": "B=16, N=1024: B / time of the 20 chained blocks; DiT blocks of one denoising step only "
                                         "(no text encoder, VAE, embedders, step count or CFG doubling); "
                                         "one_image_step_ms: the same 20 blocks at B=1"},
         "video_block_ms": {"value": round(video_ms, 3),

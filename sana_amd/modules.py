@@ -805,10 +805,11 @@ class MultiHeadCrossAttention(nn.Module):
             self.__dict__["_pad_cache"] = cache
         return cache[1]
 
-    def _attend(self, x, cond, mask):
+    def _attend(self, x, cond, mask, kv=None):
         """The HIP path up to proj's input -- softmax(q k^T) v over the short text sequence as one kernel that reads
         q_linear's output and writes proj's input token-major (no head transposes, no padded head_dim) -- or None
-        when the call is outside it."""
+        when the call is outside it.  ``kv``: kv_linear(cond) computed by the caller ([B, Nk, 2C] rows, see
+        ``StepConditioning``)."""
         B, N, C = x.shape
         H, d = self.num_heads, self.head_dim
         if not (x.is_cuda and x.dtype == torch.bfloat16 and cond.dtype == torch.bfloat16 and not torch.is_grad_enabled()
@@ -819,7 +820,8 @@ class MultiHeadCrossAttention(nn.Module):
         # (q_linear and kv_linear stay library GEMM calls at their native width: at 16384 rows they take what this
         # library's GEMM takes, at a few hundred rows they are faster, and they cost less host time per call)
         q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
-        kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)           # [B, Nk, 2C]
+        if kv is None:
+            kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)       # [B, Nk, 2C]
         if not isinstance(self.q_norm, nn.Identity):
             q = self.q_norm(q)
         if not isinstance(self.k_norm, nn.Identity):
@@ -832,23 +834,23 @@ class MultiHeadCrossAttention(nn.Module):
     # library GEMM and an elementwise pass; below it the library GEMM's shorter latency chain wins
     RESIDUAL_GEMM_MIN_ROWS = 4096
 
-    def forward_residual(self, x, cond, mask=None):
+    def forward_residual(self, x, cond, mask=None, kv=None):
         """x + self(x, cond, mask) -- what the blocks compute (sana_multi_scale.py:154) -- with the add inside the
         projection GEMM's epilogue when the call is on the HIP path and large enough."""
         B, N, C = x.shape
         if B * N >= self.RESIDUAL_GEMM_MIN_ROWS and isinstance(self.proj_drop, nn.Dropout) and self.proj_drop.p == 0.0:
-            o = self._attend(x, cond, mask)
+            o = self._attend(x, cond, mask, kv)
             if o is not None:
                 ones = self.__dict__.get("_ones_gate")
                 if ones is None or ones.device != x.device or ones.shape[-1] != C:
                     ones = self.__dict__["_ones_gate"] = torch.ones(1, 1, C, dtype=torch.bfloat16, device=x.device)
                 return ops.gemm_gate_residual(o, self.proj.weight, self.proj.bias, ones.expand(B, 1, C), x)
-        return x + self(x, cond, mask)
+        return x + self(x, cond, mask, kv)
 
-    def forward(self, x, cond, mask=None):
+    def forward(self, x, cond, mask=None, kv=None):
         B, N, C = x.shape
         H, d = self.num_heads, self.head_dim
-        o = self._attend(x, cond, mask)
+        o = self._attend(x, cond, mask, kv)
         if o is not None:
             return self.proj_drop(F.linear(o, self.proj.weight, self.proj.bias))
         if x.is_cuda:
@@ -913,10 +915,14 @@ class SanaMSBlock(nn.Module):
         self.scale_shift_table = nn.Parameter(torch.randn(6, hidden_size) / hidden_size ** 0.5)
 
     def forward(self, x, y, t, mask=None, HW=None, image_rotary_emb=None, **kwargs):
+        """The reference's signature (sana_multi_scale.py:141).  Two optional keywords ride in ``kwargs``:
+        ``text_kv`` / ``modulation``, this block's share of a ``StepConditioning`` call (kv_linear(y) and
+        scale_shift_table + t computed for all blocks of the step at once); absent, the block computes them."""
         B, N, C = x.shape
-        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
-            self.scale_shift_table[None] + t.reshape(B, 6, -1)
-        ).chunk(6, dim=1)
+        text_kv, modulation = kwargs.get("text_kv"), kwargs.get("modulation")
+        if modulation is None:
+            modulation = self.scale_shift_table[None] + t.reshape(B, 6, -1)
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = modulation.chunk(6, dim=1)
         # (conditioning in another dtype than x -- an fp32 t with a bf16 x -- promotes in the stock op chain; the
         # fused kernels read the modulation rows as x's dtype, so that case takes the stock composition below)
         if x.is_cuda and x.dtype == torch.bfloat16 and shift_msa.dtype == x.dtype and C % 8 == 0 and C <= 8192 \
@@ -930,11 +936,12 @@ class SanaMSBlock(nn.Module):
                 x = self.attn.forward_gated(h, gate_msa, x, rotary_emb=image_rotary_emb)
             if B * N >= self.cross_attn.RESIDUAL_GEMM_MIN_ROWS:
                 # the cross-attention's residual add inside its projection GEMM, then norm2 + modulate
-                x = self.cross_attn.forward_residual(x, y, mask)
+                x = self.cross_attn.forward_residual(x, y, mask, text_kv)
                 h = ops.layernorm_modulate(x, scale_mlp, shift_mlp, self.norm2.eps)
             else:
                 # the cross-attention's residual add and norm2 + modulate in one pass
-                x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask), scale_mlp, shift_mlp, self.norm2.eps)
+                x, h = ops.add_layernorm_modulate(x, self.cross_attn(x, y, mask, text_kv), scale_mlp, shift_mlp,
+                                                   self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)
         stock_path("SanaMSBlock LayerNorm / modulate / gate / residual seams",
                    f"the fused seams are bf16 inference only (C % 8 == 0, C <= 8192); got x {x.dtype}, t {t.dtype}, C = {C}, "
@@ -951,6 +958,51 @@ class SanaMSBlock(nn.Module):
         self.attn.quantize_w8_()
         self.mlp.quantize_w8_()
         return self
+
+
+class StepConditioning:
+    """What every block of one denoising step derives from the step's conditioning alone, for all the blocks of a
+    model in two launches: the text tokens' keys and values (``cross_attn.kv_linear(y)``, sana_blocks.py:77 -- a few
+    hundred rows, i.e. one latency-bound GEMM per block when the blocks run it themselves, and ONE well-filled GEMM
+    over the blocks' stacked weights here) and the six modulation rows (``scale_shift_table + t``,
+    sana_multi_scale.py:146-148).  The block loop of the model (sana_multi_scale.py:368-383) becomes
+
+        cond = StepConditioning(blocks)             # once per model
+        for blk, c in zip(blocks, cond(y, t)):      # every step: nothing is kept from one call to the next
+            x = blk(x, y, t, mask, HW, **c)
+
+    The stacked weights are a derived copy (2 * C * C * 2 bytes per block), rebuilt when a block's parameters
+    change, and not part of any state_dict.  Outside bf16 inference on the GPU the call returns empty dicts and
+    the blocks compute their own."""
+
+    def __init__(self, blocks):
+        self.blocks = list(blocks)
+        self._key = None
+
+    def _stacked(self):
+        ps = [(b.cross_attn.kv_linear.weight, b.cross_attn.kv_linear.bias, b.scale_shift_table) for b in self.blocks]
+        key = tuple((p.data_ptr(), p._version) for trio in ps for p in trio)
+        if key != self._key:
+            with torch.no_grad():
+                self._w = torch.cat([w for w, _, _ in ps])                     # [L * 2C, C]
+                self._b = torch.cat([b for _, b, _ in ps])                     # [L * 2C]
+                self._tab = torch.stack([s for _, _, s in ps])[:, None]        # [L, 1, 6, C]
+            self._key = key
+        return self._w, self._b, self._tab
+
+    def __call__(self, y, t):
+        L = len(self.blocks)
+        ca = self.blocks[0].cross_attn if L else None
+        if not (L and y.is_cuda and y.dtype == torch.bfloat16 and t.dtype == torch.bfloat16 and y.dim() == 3
+                and not torch.is_grad_enabled() and ca.kv_linear.weight.dtype == torch.bfloat16
+                and self.blocks[0].scale_shift_table.dtype == torch.bfloat16
+                and all(b.cross_attn.d_model == ca.d_model for b in self.blocks)):
+            return [{} for _ in self.blocks]
+        w, b, tab = self._stacked()
+        B, Nk, C = y.shape
+        kv = ops.gemm_bf16(y.reshape(B * Nk, C), w, b, "bias").view(B, Nk, L, 2 * C)
+        mod = tab + t.reshape(1, B, 6, -1)                                     # [L, B, 6, C]
+        return [dict(text_kv=kv[:, :, i], modulation=mod[i]) for i in range(L)]
 
 
 class ChunkedLiteLAReLURope(LiteLAReLURope):

@@ -85,6 +85,45 @@ def test_cfg3_all_twenty_blocks_and_chain_drift(cuda):
             del ob, hb
 
 
+def test_step_conditioning_shared_by_the_blocks(cuda):
+    """Three blocks of the step with their text keys / values and modulation rows computed at once
+    (``StepConditioning``: one GEMM over the stacked kv_linear weights, one add), each against the oracle block on
+    the oracle chain's running activation and against the same block computing its own: the modulation rows are the same add (bit-identical), the keys /
+    values one bf16 ulp apart at most (same products, another fp32 summation order), and a changed parameter is
+    picked up by the next call.  B=2 with a text mask; 4096 rows and 1024 rows (both cross-attention routes)."""
+    states = [bench.make_state(i) for i in range(3)]
+    obs = [oracle_block(st) for st in states]
+    hbs = [hip_block(st, cuda) for st in states]
+    cond = S.StepConditioning(hbs)
+    for B, HW in ((2, (64, 32)), (1, (32, 32))):
+        x, y, t = (a.bfloat16() for a in bench.make_inputs(B, HW[0] * HW[1]))
+        mask = torch.ones(B, y.shape[1], dtype=torch.int64)
+        mask[-1, 200:] = 0
+        xd, yd, td, md = x.to(cuda), y.to(cuda), t.to(cuda), mask.to(cuda)
+        with torch.no_grad():
+            cs = cond(yd, td)
+            assert len(cs) == 3
+            ref = x.float()
+            for i, (ob, hb, c) in enumerate(zip(obs, hbs, cs)):
+                assert torch.equal(c["modulation"], hb.scale_shift_table[None] + td.reshape(B, 6, -1))
+                kv = torch.nn.functional.linear(yd, hb.cross_attn.kv_linear.weight, hb.cross_attn.kv_linear.bias)
+                assert c["text_kv"].shape == kv.shape
+                assert ((c["text_kv"].float() - kv.float()).abs() <= 2.0 ** -7 * kv.float().abs() + 1e-5).all()
+                xin = ref.bfloat16()                      # every block on the oracle chain's running activation
+                ref = ob(xin.float(), y.float(), t.float(), mask=mask, HW=HW)
+                h_shared = hb(xin.to(cuda), yd, td, md, HW, **c)
+                check_block(h_shared, ref, f"block {i} with shared conditioning, B={B}")
+                assert rel_l2(h_shared.cpu(), hb(xin.to(cuda), yd, td, md, HW).cpu()) <= 2e-3
+    with torch.no_grad():
+        hbs[1].cross_attn.kv_linear.bias.add_(1.0)
+        hbs[2].scale_shift_table.mul_(2.0)
+        cs = cond(yd, td)
+        kv = torch.nn.functional.linear(yd, hbs[1].cross_attn.kv_linear.weight, hbs[1].cross_attn.kv_linear.bias)
+        assert ((cs[1]["text_kv"].float() - kv.float()).abs() <= 2.0 ** -7 * kv.float().abs() + 1e-5).all()
+        assert torch.equal(cs[2]["modulation"], hbs[2].scale_shift_table[None] + td.reshape(1, 6, -1))
+        assert cond(yd.float(), td.float()) == [{}, {}, {}]          # outside bf16: the blocks compute their own
+
+
 def test_cfg4_w8a16_block_at_batch_16(cuda):
     """Every qkv / proj / 1x1-conv weight int8 per output channel, B=16 images of 1024 tokens: 16384 rows, so the
     GEMMs take the route that expands the int8 weight to bf16 once per call.  Bit-identical to the bf16 block on
