@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 6
+#define SANA_HIP_ABI_VERSION 7
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -267,6 +267,27 @@ int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_sc
                                 int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc,
                                 int rows_per_gate, int64_t gate_stride,
                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * qkv projection + phase 1 of the linear attention in one GEMM (bf16, head_dim 32, no q/k transform):
+ *   Q = A Wq^T (+ bias)            stored, bf16 [B*N][C] with row stride ldq
+ *   state[b][h] = [V_h | 1]^T relu(K_h)  over the N tokens of batch entry b, fp32 [B*heads][33][32]
+ * replaces `qkv = self.qkv(x)` together with the `vk = v @ k^T` half of LiteLA.forward
+ * (diffusion/model/nets/sana_blocks.py:270-296, :245-263): k and v are never written -- the column tiles that
+ * produce them are contracted over their tokens in the GEMM's epilogue (k and v rounded to bf16 first, products in
+ * fp32, exactly the values sana_hip_linattn_state reads back from memory; the sums differ from its sums by fp32
+ * summation order only).  sana_hip_linattn_apply then takes Q and the state.
+ *   The weight comes in the layout sana_hip_qkv_state_rows describes: rows[i] is the row of the reference's
+ *   [3C][C] qkv weight (and entry of its bias) that row i of W_tiled holds, or -1 for a zero row.  With rows ==
+ *   NULL the function returns the number of rows; with a buffer of that capacity it fills it (host code, no GPU).
+ *   A: bf16 [B*N][C] (row stride lda); W_tiled: bf16 [rows][C] (row stride ldw); bias_tiled: bf16 [rows] or NULL.
+ *   N % 256 == 0, C == 32 * heads.  workspace: sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads) bytes (one
+ *   partial state per 256 tokens, added in token order by a second launch: deterministic, no atomics). */
+int sana_hip_qkv_state_rows(int C, int heads, int32_t* rows, int capacity);
+size_t sana_hip_gemm_qkv_state_workspace_bytes(int B, int N, int heads);
+int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const void* bias_tiled, void* Q, float* state,
+                            void* workspace, size_t workspace_bytes, int B, int N, int C, int heads,
+                            int64_t lda, int64_t ldw, int64_t ldq, void* stream);
 
 /* LayerNorm without affine (eps inside the rsqrt) + adaLN modulation:
  *   out[m][:] = LN(x[m][:]) * (1 + scale[m / rows_per_mod][:]) + shift[m / rows_per_mod][:]

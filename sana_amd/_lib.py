@@ -54,6 +54,10 @@ SIGNATURES = {
     "sana_hip_gemm_gate_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64,
                                             c_int, c_int64, c_void_p, c_size_t, c_void_p]),
+    "sana_hip_qkv_state_rows": (c_int, [c_int, c_int, c_void_p, c_int]),
+    "sana_hip_gemm_qkv_state_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "sana_hip_gemm_qkv_state": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                        c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_void_p]),
     "sana_hip_add_layernorm_modulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                 c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int64, c_float,
                                                 c_int, c_void_p]),

@@ -101,8 +101,14 @@ struct EpiArgs {
   const uint16_t* res;   // [M, N] with row stride ldr
   int64_t ldr, gate_stride;
   int rows_per_gate;
+  // SANA_EPI_QKV_STATE only: per-token-tile partial states, [B * heads][tiles_per_batch][33 * 32] fp32
+  float* part;
+  int q_cols, q_pad, heads, tiles_per_batch;  // q_cols = C (columns of the q region), q_pad = C rounded up to the tile
 };
 #define SANA_EPI_GATE_RES 3
+// (not part of the C ABI's epilogue codes) qkv projection of the linear attention with the k / v column tiles
+// contracted over their tokens in the epilogue instead of stored: see state_tile16
+#define SANA_EPI_QKV_STATE 4
 
 // Virtual concatenation of the A operand along k: columns [t*kc, (t+1)*kc) of the GEMM's A are columns
 // [0, kc) of the matrix whose row m is row m + t*stride of the buffer (a convolution over rows as one GEMM,
@@ -395,6 +401,114 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
 }
 
 
+// Epilogue of a k / v column tile of the fused qkv projection (SANA_EPI_QKV_STATE, 256-wide tiles only).  The tile's
+// 256 weight rows are, per wave column wc, [K of head 4T+2wc | V of it | K of head 4T+2wc+1 | V of it] (32 rows
+// each; the caller lays the weight out that way, see sana_hip_qkv_state_rows), so lane group g = lane / 16 of a wave
+// holds, for its tokens lane % 16 + 16 j, all 32 channels of one of those four blocks.  Instead of storing k and v,
+// the wave contracts them over its 128 tokens: S[dv][dk] += v[n][dv] * relu(k[n][dk]) and ksum[dk] += relu(k[n][dk])
+// with v and k rounded to bf16 first (what the unfused path stores and reads back), products in fp32 on the MFMA.
+// The contraction index of v_mfma_f32_16x16x32_bf16 is the token, and which token sits in which k slot is free as
+// long as both operands agree: the 8 tokens a lane holds for one channel (j = 0 .. 7) ARE one operand fragment, it
+// only sits in the wrong lane (the lane is the token group, the MFMA wants the channel there), so it takes one trip
+// through the wave's LDS: written at [channel][token group ^ channel % 16] (16 bytes each, conflict-free both ways),
+// read back as [channel = lane % 16][token group 4 m + lane / 16] for the m-th MFMA of a chain of four.  The two
+// token halves of the workgroup are added through LDS and the sum goes to this token tile's slot of the partial
+// states, which a second kernel adds up in tile order (deterministic, no atomics).
+__device__ __forceinline__ void state_tile16(f32x4_t (&acc)[8][8], const u32x4_t (&bpk)[4], unsigned char* smem,
+                                             const EpiArgs& ep, int m0, int n0) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wc = wave & 1, wt = wave >> 1;
+  const int fr = lane & 15, fg = lane >> 4;
+  __syncthreads();  // every wave is done with the operand tiles
+  unsigned char* stg = smem + wave * 32768;
+  // relu for the k blocks (fg even) as a packed signed-integer max on the bf16 pairs; int16 minimum = no-op for v
+  const uint32_t floor2 = (fg & 1) ? 0x80008000u : 0u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t bw0 = bpk[i >> 1][2 * (i & 1)], bw1 = bpk[i >> 1][2 * (i & 1) + 1];
+    const float b4[4] = {bf16_lo(bw0), bf16_hi(bw0), bf16_lo(bw1), bf16_hi(bw1)};  // channels 4 i + r of the lane's 32
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      u32x4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t pk = pack_bf16(acc[i][2 * e][r] + b4[r], acc[i][2 * e + 1][r] + b4[r]);
+        o[e] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2_t, pk),
+                                                                    __builtin_bit_cast(s16x2_t, floor2)));
+      }
+      const int row = 32 * fg + 4 * i + r;
+      *reinterpret_cast<u32x4_t*>(stg + row * 256 + ((fr ^ (row & 15)) << 4)) = o;
+    }
+  }
+  // wave-private LDS is in order: the reads below see the writes above.  hh: the wave's two heads.
+  f32x4_t S[2][2][2], Ks[2][2];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Ks[hh][b][r] = 0.f, S[hh][0][b][r] = 0.f, S[hh][1][b][r] = 0.f;
+    }
+  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int slot = ((4 * m + fg) ^ fr) << 4;
+      u32x4_t kf[2], vf[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        kf[b] = *reinterpret_cast<const u32x4_t*>(stg + (64 * hh + 16 * b + fr) * 256 + slot);
+        vf[b] = *reinterpret_cast<const u32x4_t*>(stg + (64 * hh + 32 + 16 * b + fr) * 256 + slot);
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        // (the builtin, not the main loop's asm statement: the compiler then places the wait states itself)
+        S[hh][0][b] = mfma_16x16x32_bf16(vf[0], kf[b], S[hh][0][b]);
+        S[hh][1][b] = mfma_16x16x32_bf16(vf[1], kf[b], S[hh][1][b]);
+        Ks[hh][b] = mfma_16x16x32_bf16(ones, kf[b], Ks[hh][b]);
+      }
+    }
+  }
+  // add the two token halves: wave wt = 1 hands its 48 values per lane to wave wt = 0 of the same channel half
+  float* xch = reinterpret_cast<float*>(stg) + lane;
+  if (wt == 1) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          xch[(((hh * 2 + b) * 3 + 0) * 4 + r) * 64] = S[hh][0][b][r];
+          xch[(((hh * 2 + b) * 3 + 1) * 4 + r) * 64] = S[hh][1][b][r];
+          xch[(((hh * 2 + b) * 3 + 2) * 4 + r) * 64] = Ks[hh][b][r];
+        }
+  }
+  __syncthreads();
+  if (wt == 0) {
+    const float* oth = reinterpret_cast<const float*>(smem + (wave + 2) * 32768) + lane;
+    const int tile_kv = (n0 - ep.q_pad) >> 8;
+    const int tile_m = m0 >> 8;
+    const int bi = tile_m / ep.tiles_per_batch, split = tile_m - bi * ep.tiles_per_batch;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int head = 4 * tile_kv + 2 * wc + hh;
+      if (head < ep.heads) {
+        float* o = ep.part + (((int64_t)bi * ep.heads + head) * ep.tiles_per_batch + split) * (33 * 32);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            o[(4 * fg + r) * 32 + 16 * b + fr] = S[hh][0][b][r] + oth[(((hh * 2 + b) * 3 + 0) * 4 + r) * 64];
+            o[(16 + 4 * fg + r) * 32 + 16 * b + fr] = S[hh][1][b][r] + oth[(((hh * 2 + b) * 3 + 1) * 4 + r) * 64];
+          }
+          if (fg == 0) o[32 * 32 + 16 * b + fr] = Ks[hh][b][0] + oth[(((hh * 2 + b) * 3 + 2) * 4 + 0) * 64];
+        }
+      }
+    }
+  }
+}
+
 // Epilogue of the pipelined kernels.  acc[i][j][r] (MFMA 16x16 tiles: i = channel tile of the wave, j = token tile):
 // token m0 + wt*128 + 16*j + lane%16, channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  bpk: the lane's 8*NI bias
 // values, packed (the caller requests them ahead of its last k-tile so that their latency hides behind its MFMAs).
@@ -404,6 +518,14 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
                                               int m0, int n0) {
   constexpr int NWT = 2 * NI;
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
+  if constexpr (EPI == SANA_EPI_QKV_STATE) {
+    static_assert(NI == 4 && !SPLIT, "the fused qkv projection runs 256-wide tiles, unsplit");
+    if (n0 >= ep.q_pad) {  // uniform per workgroup: a k / v tile
+      state_tile16(acc, bpk, smem, ep, m0, n0);
+      return;
+    }
+    N = ep.q_cols;  // a q tile: stored like any biased output, columns past C dropped
+  }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wc = wave & 1, wt = wave >> 1;
   const int fr = lane & 15, fg = lane >> 4;
@@ -487,7 +609,7 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
     float a8[8];
 #pragma unroll
     for (int r = 0; r < 4; ++r) a8[r] = acc[2 * c][j][r], a8[4 + r] = acc[2 * c + 1][j][r];
-    const u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
+    const u32x4_t o = epi_pack8<(EPI == SANA_EPI_GATE_RES || EPI == SANA_EPI_QKV_STATE) ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
     const int chunk = NI * fg + c;
     *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
   };
@@ -1136,8 +1258,38 @@ int check_gate_res(const void* gate, const void* residual, int M, int N, int64_t
   return SANA_OK;
 }
 
+// Sum of the per-token-tile partial states of the fused qkv projection: part[bh][nsplit][33 * 32] -> state[bh][33 * 32].
+// A workgroup takes 64 elements of one (batch, head): four threads per element add every fourth tile in tile order
+// (independent loads, all in flight together), and the four sums are added in a fixed order -- deterministic.
+__global__ __launch_bounds__(256) void qkv_state_reduce_kernel(const float* __restrict__ part, float* __restrict__ state,
+                                                                int nsplit) {
+  constexpr int ELEMS = 33 * 32, SLICES = (ELEMS + 63) / 64;
+  __shared__ float red[4][64];
+  const int bh = blockIdx.x / SLICES, e = (blockIdx.x % SLICES) * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
+  float s = 0.f;
+  if (e < ELEMS) {
+    const float* p = part + ((int64_t)bh * nsplit) * ELEMS + e;
+    for (int sp0 = grp; sp0 < nsplit; sp0 += 32) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = (sp0 + 4 * u < nsplit) ? p[(int64_t)(sp0 + 4 * u) * ELEMS] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+  }
+  red[grp][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (grp == 0 && e < ELEMS)
+    state[(int64_t)bh * ELEMS + e] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+}
+
+// Rows of the fused qkv projection's weight layout for C = 32 * heads channels: the q rows padded to whole 256-wide
+// tiles, then one tile per four heads, [K h | V h | K h+1 | V h+1] for the tile's first and second pair of heads.
+int qkv_state_q_pad(int C) { return (C + 255) / 256 * 256; }
+int qkv_state_rows_total(int C, int heads) { return qkv_state_q_pad(C) + (heads + 3) / 4 * 256; }
+
 EpiArgs plain_epi(const void* bias) {
-  EpiArgs e = {static_cast<const uint16_t*>(bias), nullptr, nullptr, 0, 0, 1};
+  EpiArgs e = {static_cast<const uint16_t*>(bias), nullptr, nullptr, 0, 0, 1, nullptr, 0, 0, 0, 0};
   return e;
 }
 
@@ -1184,7 +1336,7 @@ SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const flo
   rc = check_gate_res(gate, residual, M, N, ldr, rows_per_gate, gate_stride);
   if (rc != SANA_OK) return rc;
   const EpiArgs e = {static_cast<const uint16_t*>(bias), static_cast<const uint16_t*>(gate),
-                     static_cast<const uint16_t*>(residual), ldr, gate_stride, rows_per_gate};
+                     static_cast<const uint16_t*>(residual), ldr, gate_stride, rows_per_gate, nullptr, 0, 0, 0, 0};
   hipStream_t s = static_cast<hipStream_t>(stream);
   return w8 ? launch<true>(A, W, w8_scale, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s, nullptr, workspace,
                            workspace_bytes)
@@ -1203,7 +1355,7 @@ SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, in
   if (ldx % 8 || ldw % 8 || ldo % 8 || !aligned16(X) || !aligned16(W) || !aligned16(out)) return SANA_ERR_ALIGN;
   if (x_rows * ldx * 2 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;  // 32-bit byte offsets inside the buffer
   const uint16_t* x = static_cast<const uint16_t*>(X);
-  const EpiArgs e = {nullptr, nullptr, x + (taps / 2) * tap_rows * ldx, ldx, 0, M};
+  const EpiArgs e = {nullptr, nullptr, x + (taps / 2) * tap_rows * ldx, ldx, 0, M, nullptr, 0, 0, 0, 0};
   const Taps tp = {C, tap_rows, x_rows, 0, 0, zero_last_tap};
   return launch<false>(X, W, nullptr, e, out, M, C, taps * C, ldx, ldw, ldo, SANA_EPI_GATE_RES,
                        static_cast<hipStream_t>(stream), &tp);
@@ -1219,5 +1371,54 @@ SANA_API int sana_hip_dequant_w8(const int8_t* Wq, const float* scale, void* W, 
   if ((threads + 255) / 256 > 0x7fffffff) return SANA_ERR_SHAPE;
   hipLaunchKernelGGL(dequant_w8_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), Wq, scale, static_cast<uint16_t*>(W), N, K, ldw, ldo);
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+SANA_API int sana_hip_qkv_state_rows(int C, int heads, int32_t* rows, int capacity) {
+  if (C <= 0 || heads <= 0 || C != 32 * heads) return SANA_ERR_SHAPE;
+  const int q_pad = qkv_state_q_pad(C), total = qkv_state_rows_total(C, heads);
+  if (!rows) return total;
+  if (capacity < total) return SANA_ERR_ARG;
+  for (int i = 0; i < q_pad; ++i) rows[i] = i < C ? i : -1;
+  for (int i = q_pad; i < total; ++i) {
+    const int l = (i - q_pad) & 255, tile = (i - q_pad) >> 8;
+    const int head = 4 * tile + 2 * (l >> 7) + ((l >> 6) & 1), is_v = (l >> 5) & 1, e = l & 31;
+    rows[i] = head < heads ? (1 + is_v) * C + 32 * head + e : -1;
+  }
+  return total;
+}
+
+SANA_API size_t sana_hip_gemm_qkv_state_workspace_bytes(int B, int N, int heads) {
+  if (B <= 0 || N <= 0 || heads <= 0 || N % 256) return 0;
+  return (size_t)B * heads * (N / 256) * 33 * 32 * sizeof(float);
+}
+
+SANA_API int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const void* bias_tiled, void* Q, float* state,
+                                     void* workspace, size_t workspace_bytes, int B, int N, int C, int heads,
+                                     int64_t lda, int64_t ldw, int64_t ldq, void* stream) {
+  if (!A || !W_tiled || !Q || !state || B <= 0 || N <= 0 || C <= 0 || heads <= 0) return SANA_ERR_ARG;
+  if (C != 32 * heads || N % 256 || C < 64) return SANA_ERR_SHAPE;
+  if ((int64_t)B * N >= ((int64_t)1 << 31) / 2) return SANA_ERR_SHAPE;
+  const int M = B * N, rows_t = qkv_state_rows_total(C, heads);
+  if (lda < C || ldw < C || ldq < C) return SANA_ERR_ARG;
+  if (lda >= (1 << 22) || ldw >= (1 << 22) || ldq >= (1 << 22)) return SANA_ERR_SHAPE;
+  if (lda % 8 || ldw % 8 || ldq % 8 || !aligned16(A) || !aligned16(W_tiled) || !aligned16(Q) ||
+      (bias_tiled && !aligned16(bias_tiled)) || !aligned16(state))
+    return SANA_ERR_ALIGN;
+  const size_t need = sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads);
+  if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
+  if (!aligned16(workspace)) return SANA_ERR_ALIGN;
+  const int64_t tiles_t = M / BT, tiles_c = rows_t / 256;
+  if (tiles_t * tiles_c > (1 << 30)) return SANA_ERR_SHAPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const EpiArgs e = {static_cast<const uint16_t*>(bias_tiled), nullptr, nullptr, 0, 0, 1, static_cast<float*>(workspace),
+                     C, qkv_state_q_pad(C), heads, N / 256};
+  const Taps none = {0, 0, 0, 0, 0, nullptr};
+  hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_QKV_STATE, 4>), dim3((unsigned)(tiles_t * tiles_c)), dim3(256), 0, s,
+                     static_cast<const uint16_t*>(A), W_tiled, static_cast<const float*>(nullptr), e,
+                     static_cast<uint16_t*>(Q), M, rows_t, C, lda, ldw, ldq, (int)tiles_t, (int)tiles_c, none);
+  if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+  hipLaunchKernelGGL(qkv_state_reduce_kernel, dim3((unsigned)(B * heads * ((33 * 32 + 63) / 64))), dim3(256), 0, s,
+                     static_cast<const float*>(workspace), state, N / 256);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }

@@ -277,13 +277,46 @@ class LiteLA(nn.Module):
     def forward_gated(self, x, gate, residual, rotary_emb=None, **kwargs) -> torch.Tensor:
         """forward(x), or residual + gate * forward(x) with the update fused into the proj GEMM."""
         _no_grad_only(x)
-        if rotary_emb is None and x.dtype == torch.bfloat16:   # qk-norm (if any) on load inside the kernels
+        if rotary_emb is None and x.dtype == torch.bfloat16 and self._state_in_qkv_gemm(x):
+            # k and v never reach memory: their column tiles are contracted over the tokens in the qkv GEMM's epilogue
+            wt, bt = self._tiled_qkv()
+            if self.qkv.is_quantized:       # int8 weights: expanded to bf16 per call, as the plain GEMM does from 4096 rows
+                wt = ops.dequant_w8(*wt)
+            q, state = ops.gemm_qkv_state(x, wt, bt, self.heads)
+            out = ops.linattn_apply(q, state, self.eps)
+        elif rotary_emb is None and x.dtype == torch.bfloat16:   # qk-norm (if any) on load inside the kernels
             B, N, C = x.shape
             out = self._attend(self.qkv(x).view(B, N, 3, C), None)
         else:
             qkv = self._qkv_tokens(x, rotary_emb)
             out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps, head_dim=self.dim)
         return self._proj_gated(out, gate, residual)
+
+    # rows from which the qkv projection and phase 1 of the attention run as one GEMM (below it the 192-wide tiles
+    # of the plain GEMM fill the chip better than the fused kernel's 256-wide ones, and phase 1 is a few us)
+    STATE_IN_QKV_GEMM_MIN_ROWS = 4096
+
+    def _state_in_qkv_gemm(self, x) -> bool:
+        B, N, C = x.shape
+        return (x.is_cuda and self.dim == 32 and B * N >= self.STATE_IN_QKV_GEMM_MIN_ROWS
+                and isinstance(self.q_norm, nn.Identity) and isinstance(self.k_norm, nn.Identity)
+                and (self.qkv.is_quantized or self.qkv.weight.dtype == torch.bfloat16)
+                and ops.qkv_state_supported(N, C, self.heads))
+
+    def _tiled_qkv(self):
+        """The qkv weight (and bias) in the fused GEMM's row layout: derived data, rebuilt when the parameters
+        change, not part of the state_dict."""
+        quant = self.qkv.is_quantized
+        ps = (self.qkv.weight_q, self.qkv.weight_scale, self.qkv.bias) if quant else (self.qkv.weight, self.qkv.bias)
+        key = tuple((p.data_ptr(), p._version, p.device) for p in ps if p is not None)
+        cache = self.__dict__.get("_tiled_cache")
+        if cache is None or cache[0] != key:
+            with torch.no_grad():
+                tiled = [None if p is None else ops.tile_qkv_rows(p.detach(), self.heads) for p in ps]
+            # (weight, bias), the weight being the pair (int8 weight, scales) of a quantised projection
+            cache = (key, ((tiled[0], tiled[1]), tiled[2]) if quant else (tiled[0], tiled[1]))
+            self.__dict__["_tiled_cache"] = cache
+        return cache[1]
 
     def _proj_gated(self, out, gate, residual):
         """proj(out), or residual + gate * proj(out) in the GEMM epilogue; gate is [B, 1, C] or one row per

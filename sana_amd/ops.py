@@ -362,6 +362,68 @@ def dequant_w8(wq: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def qkv_state_rows(C: int, heads: int) -> torch.Tensor:
+    """Row map of the fused qkv projection's weight layout (``sana_hip_qkv_state_rows``): int64 [rows], entry i = the
+    row of the [3C, C] qkv weight that row i of the tiled weight holds, -1 for a zero row.  Host code."""
+    import ctypes
+    lib = _lib.load()
+    n = lib.sana_hip_qkv_state_rows(C, heads, None, 0)
+    if n <= 0:
+        raise SanaHipError(f"the fused qkv projection needs C == 32 * heads, got C={C}, heads={heads}")
+    buf = (ctypes.c_int32 * n)()
+    if lib.sana_hip_qkv_state_rows(C, heads, ctypes.cast(buf, ctypes.c_void_p), n) != n:
+        raise SanaHipError("sana_hip_qkv_state_rows failed")
+    return torch.tensor(list(buf), dtype=torch.int64)
+
+
+def tile_qkv_rows(t: torch.Tensor, heads: int) -> torch.Tensor:
+    """A per-output-channel tensor of the qkv projection ([3C, ...]: weight, int8 weight, bias, scales) in the fused
+    GEMM's row layout ([rows, ...], zero where the layout has no source row)."""
+    C = t.shape[0] // 3
+    rows = qkv_state_rows(C, heads).to(t.device)
+    live = rows >= 0
+    out = torch.zeros(rows.numel(), *t.shape[1:], dtype=t.dtype, device=t.device)
+    out[live] = t[rows[live]]
+    return out
+
+
+def tile_qkv_weight(weight: torch.Tensor, bias: Optional[torch.Tensor], heads: int):
+    """(W_tiled, bias_tiled) for ``gemm_qkv_state`` from the reference's [3C, C] qkv weight and [3C] bias (or None)."""
+    return tile_qkv_rows(weight, heads), None if bias is None else tile_qkv_rows(bias, heads)
+
+
+def qkv_state_supported(n_tokens: int, C: int, heads: int) -> bool:
+    return heads > 0 and C == 32 * heads and C >= 64 and n_tokens > 0 and n_tokens % 256 == 0
+
+
+def gemm_qkv_state(x: torch.Tensor, w_tiled: torch.Tensor, bias_tiled: Optional[torch.Tensor], heads: int):
+    """qkv projection with phase 1 of the linear attention in its epilogue.  x: [B, N, C] bf16 (N % 256 == 0),
+    w_tiled / bias_tiled: ``tile_qkv_weight``'s.  Returns (q [B, N, C] bf16, state [B, heads, 1, 33, 32] fp32)."""
+    _need_cuda(x, w_tiled, bias_tiled)
+    if x.dim() != 3 or x.dtype != torch.bfloat16 or w_tiled.dtype != torch.bfloat16:
+        raise SanaHipError("gemm_qkv_state needs a bf16 [B, N, C] input and a bf16 tiled weight")
+    B, N, C = x.shape
+    if not qkv_state_supported(N, C, heads):
+        raise SanaHipError(f"gemm_qkv_state needs N % 256 == 0 and C == 32 * heads, got N={N}, C={C}, heads={heads}")
+    lib = _lib.load()
+    if tuple(w_tiled.shape) != (lib.sana_hip_qkv_state_rows(C, heads, None, 0), C):
+        raise SanaHipError(f"tiled weight of shape {tuple(w_tiled.shape)} does not fit C={C}, heads={heads}")
+    if bias_tiled is not None and (bias_tiled.dtype != torch.bfloat16 or bias_tiled.numel() != w_tiled.shape[0]
+                                   or not bias_tiled.is_contiguous()):
+        raise SanaHipError("bias_tiled must be contiguous bf16 [rows]")
+    a, lda = _rows(x.reshape(B * N, C), "x")
+    w, ldw = _rows(w_tiled, "w_tiled")
+    q = torch.empty(B, N, C, dtype=torch.bfloat16, device=x.device)
+    state = torch.empty(B, heads, 1, 33, 32, dtype=torch.float32, device=x.device)
+    nbytes = lib.sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads)
+    ws = _workspace(x.device, nbytes)
+    code = lib.sana_hip_gemm_qkv_state(a.data_ptr(), w.data_ptr(), None if bias_tiled is None else bias_tiled.data_ptr(),
+                                       q.data_ptr(), state.data_ptr(), ws.data_ptr(), nbytes, B, N, C, heads,
+                                       lda, ldw, C, _stream())
+    _lib.check(code, "sana_hip_gemm_qkv_state")
+    return q, state
+
+
 def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor] = None,
                epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None,
                expand: Optional[bool] = None) -> torch.Tensor:

@@ -32,7 +32,7 @@ def test_exports_every_declared_symbol():
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.sana_hip_abi_version() == 6
+    assert lib.sana_hip_abi_version() == 7
     assert b"aligned" in lib.sana_hip_strerror(-3)
     assert b"unknown" in lib.sana_hip_strerror(-99)
 
@@ -98,3 +98,30 @@ def test_ops_refuse_cpu_tensors():
     x = torch.zeros(1, 32, 32)
     with pytest.raises(_lib.SanaHipError):
         ops.linattn_state(x, x)
+
+
+def test_qkv_state_row_map_is_a_layout_of_the_qkv_weight():
+    """sana_hip_qkv_state_rows (host code): q rows first, padded to whole 256-row tiles; then per tile of four heads
+    [K h | V h | K h+1 | V h+1] twice; every row of the [3C, C] weight exactly once, the rest -1."""
+    import ctypes
+    lib = _lib.load()
+    for heads in (1, 2, 5, 36, 70):
+        C = 32 * heads
+        n = lib.sana_hip_qkv_state_rows(C, heads, None, 0)
+        q_pad = (C + 255) // 256 * 256
+        assert n == q_pad + (heads + 3) // 4 * 256
+        buf = (ctypes.c_int32 * n)()
+        assert lib.sana_hip_qkv_state_rows(C, heads, ctypes.cast(buf, ctypes.c_void_p), n) == n
+        rows = list(buf)
+        assert rows[:C] == list(range(C)) and all(r == -1 for r in rows[C:q_pad])
+        live = sorted(r for r in rows if r >= 0)
+        assert live == list(range(3 * C))
+        for i in range(q_pad, n):
+            loc = (i - q_pad) % 256
+            head = 4 * ((i - q_pad) // 256) + 2 * (loc // 128) + (loc // 64) % 2
+            want = -1 if head >= heads else (1 + (loc // 32) % 2) * C + 32 * head + loc % 32
+            assert rows[i] == want
+    assert lib.sana_hip_qkv_state_rows(100, 3, None, 0) < 0          # C != 32 * heads
+    assert lib.sana_hip_qkv_state_rows(64, 2, ctypes.cast((ctypes.c_int32 * 4)(), ctypes.c_void_p), 4) < 0
+    assert lib.sana_hip_gemm_qkv_state_workspace_bytes(2, 512, 3) == 2 * 3 * 2 * 33 * 32 * 4
+    assert lib.sana_hip_gemm_qkv_state_workspace_bytes(2, 500, 3) == 0
