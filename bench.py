@@ -290,6 +290,14 @@ def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_onl
         add(name, "mfma", 2 * M * Nn * Kk, t_us, f"2*M*K*N, M={M} N={Nn} K={Kk}")
         t_lib = event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 20, 5)
         rows[-1]["library_gemm_us"] = round(t_lib, 2)   # hipBLASLt, plain GEMM(+bias) of the same shape, for scale only
+        if name == "gemm_qkv":
+            # the same projection with phase 1 of the attention in its epilogue (k, v never stored): one launch + the
+            # sum of the 64 per-tile partial states, against this row + linattn_state above
+            wt_, _ = ops.tile_qkv_weight(w, None, C // 32)
+            t_f = event_time_us(lambda: ops.gemm_qkv_state(a.view(B, N, Kk), wt_, None, C // 32), 20, 5)
+            add("gemm_qkv_with_attention_state", "mfma", 2 * M * Nn * Kk + 2 * M * C * 33, t_f,
+                f"2*M*K*N + 2*M*C*33 (state), M={M} N={Nn} K={Kk}; replaces gemm_qkv + linattn_state")
+            del wt_
         del a, w, o
     if cfg3_only:
         return

@@ -440,8 +440,10 @@ __device__ __forceinline__ void state_tile16(f32x4_t (&acc)[8][8], const u32x4_t
       *reinterpret_cast<u32x4_t*>(stg + row * 256 + ((fr ^ (row & 15)) << 4)) = o;
     }
   }
-  // wave-private LDS is in order: the reads below see the writes above.  hh: the wave's two heads.
-  f32x4_t S[2][2][2], Ks[2][2];
+  // wave-private LDS is in order: the reads below see the writes above.  hh: the wave's two heads.  The products
+  // are formed transposed (rows = dk, columns = dv), so that a lane ends with four consecutive dk of one dv:
+  // 16-byte stores into the [dv][dk] state.
+  f32x4_t S[2][2][2], Ks[2][2];  // S[hh][a][b]: dk 16 a + 4 fg + r, dv 16 b + fr;  Ks[hh][a]: dk 16 a + 4 fg + r
 #pragma unroll
   for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
@@ -462,31 +464,29 @@ __device__ __forceinline__ void state_tile16(f32x4_t (&acc)[8][8], const u32x4_t
         vf[b] = *reinterpret_cast<const u32x4_t*>(stg + (64 * hh + 32 + 16 * b + fr) * 256 + slot);
       }
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int a = 0; a < 2; ++a) {
         // (the builtin, not the main loop's asm statement: the compiler then places the wait states itself)
-        S[hh][0][b] = mfma_16x16x32_bf16(vf[0], kf[b], S[hh][0][b]);
-        S[hh][1][b] = mfma_16x16x32_bf16(vf[1], kf[b], S[hh][1][b]);
-        Ks[hh][b] = mfma_16x16x32_bf16(ones, kf[b], Ks[hh][b]);
+        S[hh][a][0] = mfma_16x16x32_bf16(kf[a], vf[0], S[hh][a][0]);
+        S[hh][a][1] = mfma_16x16x32_bf16(kf[a], vf[1], S[hh][a][1]);
+        Ks[hh][a] = mfma_16x16x32_bf16(kf[a], ones, Ks[hh][a]);
       }
     }
   }
   // add the two token halves: wave wt = 1 hands its 48 values per lane to wave wt = 0 of the same channel half
-  float* xch = reinterpret_cast<float*>(stg) + lane;
+  f32x4_t* xch = reinterpret_cast<f32x4_t*>(stg) + lane;
   if (wt == 1) {
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          xch[(((hh * 2 + b) * 3 + 0) * 4 + r) * 64] = S[hh][0][b][r];
-          xch[(((hh * 2 + b) * 3 + 1) * 4 + r) * 64] = S[hh][1][b][r];
-          xch[(((hh * 2 + b) * 3 + 2) * 4 + r) * 64] = Ks[hh][b][r];
-        }
+      for (int a = 0; a < 2; ++a) {
+        xch[((hh * 2 + a) * 3 + 0) * 64] = S[hh][a][0];
+        xch[((hh * 2 + a) * 3 + 1) * 64] = S[hh][a][1];
+        xch[((hh * 2 + a) * 3 + 2) * 64] = Ks[hh][a];
+      }
   }
   __syncthreads();
   if (wt == 0) {
-    const float* oth = reinterpret_cast<const float*>(smem + (wave + 2) * 32768) + lane;
+    const f32x4_t* oth = reinterpret_cast<const f32x4_t*>(smem + (wave + 2) * 32768) + lane;
     const int tile_kv = (n0 - ep.q_pad) >> 8;
     const int tile_m = m0 >> 8;
     const int bi = tile_m / ep.tiles_per_batch, split = tile_m - bi * ep.tiles_per_batch;
@@ -496,13 +496,12 @@ __device__ __forceinline__ void state_tile16(f32x4_t (&acc)[8][8], const u32x4_t
       if (head < ep.heads) {
         float* o = ep.part + (((int64_t)bi * ep.heads + head) * ep.tiles_per_batch + split) * (33 * 32);
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int a = 0; a < 2; ++a) {
+          const int dk0 = 16 * a + 4 * fg;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            o[(4 * fg + r) * 32 + 16 * b + fr] = S[hh][0][b][r] + oth[(((hh * 2 + b) * 3 + 0) * 4 + r) * 64];
-            o[(16 + 4 * fg + r) * 32 + 16 * b + fr] = S[hh][1][b][r] + oth[(((hh * 2 + b) * 3 + 1) * 4 + r) * 64];
-          }
-          if (fg == 0) o[32 * 32 + 16 * b + fr] = Ks[hh][b][0] + oth[(((hh * 2 + b) * 3 + 2) * 4 + 0) * 64];
+          for (int b = 0; b < 2; ++b)
+            *reinterpret_cast<f32x4_t*>(o + (16 * b + fr) * 32 + dk0) = S[hh][a][b] + oth[((hh * 2 + a) * 3 + b) * 64];
+          if (fr == 0) *reinterpret_cast<f32x4_t*>(o + 32 * 32 + dk0) = Ks[hh][a] + oth[((hh * 2 + a) * 3 + 2) * 64];
         }
       }
     }
