@@ -537,23 +537,43 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
   // row-contiguous, so each store instruction writes four full 256-byte row segments.  It goes in four
   // groups of 32 tokens: the stores of one group drain while the next group's activations are computed.
   if (SPLIT) {
-    // raw accumulators -> partial[z][M][N] (fp32, dense): a lane owns 16 consecutive channels of one token per
-    // MFMA tile, stored as four 16-byte pieces through a buffer resource over the wave's rows of this range's
-    // plane (rows past M fall outside it and are dropped; channel pieces past N get the idle offset)
+    // raw accumulators -> partial[z][M][N] (fp32, dense).  A lane owns 8*NI consecutive channels of one token per
+    // token tile j, but one store instruction of that layout would write 64 separate 16-byte pieces (16 rows x 4
+    // lane groups): measured, such an epilogue took as long as the 22 k-tiles in front of it.  So the sub-tile
+    // goes through the wave's 32 KB of LDS, 64 tokens at a time ([64 tokens][128 channels] fp32, 16-byte chunks
+    // XOR-swizzled by token % 16), and leaves as whole row segments: a store instruction writes two rows of 512
+    // contiguous bytes.  Rows past M fall outside the buffer resource and are dropped; chunks past N get the idle
+    // offset.
+    __syncthreads();  // every wave is done with the operand tiles
+    unsigned char* stg = smem + wave * 32768;
     const int prow0 = m0 + __builtin_amdgcn_readfirstlane(wt) * 128;
     const int prows = max(0, min(128, M - prow0));
     float* plane = reinterpret_cast<float*>(C) + ((int64_t)blockIdx.y * M + prow0) * N;
     const __amdgpu_buffer_rsrc_t rsrc_p =
         __builtin_amdgcn_make_buffer_rsrc(plane, 0, (int)((int64_t)prows * N * 4), 0x00020000);
+    const int s_chunk = lane & 31, s_rsub = lane >> 5;               // store side: 32 chunks of 4 channels, 2 rows
+    const int s_n = n0 + wc * 32 * NI + 4 * s_chunk;
+    const bool s_live = s_chunk < 8 * NI && s_n < N;
 #pragma unroll
-    for (int i = 0; i < NWT; ++i) {
-      const int n = n0 + wc * 32 * NI + 8 * NI * fg + 4 * i;  // the lane's four channels of tile i
+    for (int half = 0; half < 2; ++half) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int row_off = ((16 * j + fr) * N + n) * 4;
-        const u32x4_t o = {__float_as_uint(acc[i][j][0]), __float_as_uint(acc[i][j][1]), __float_as_uint(acc[i][j][2]),
-                           __float_as_uint(acc[i][j][3])};
-        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, n < N ? row_off : (int)0x80000000u, 0, 0);
+      for (int jj = 0; jj < 4; ++jj) {
+        const int tok = 16 * jj + fr;                                 // token of this half, 0 .. 63
+#pragma unroll
+        for (int i = 0; i < NWT; ++i) {
+          const int chunk = 2 * NI * fg + i;                          // 4 channels each: 8*NI*fg + 4*i
+          const u32x4_t o = {__float_as_uint(acc[i][4 * half + jj][0]), __float_as_uint(acc[i][4 * half + jj][1]),
+                             __float_as_uint(acc[i][4 * half + jj][2]), __float_as_uint(acc[i][4 * half + jj][3])};
+          *reinterpret_cast<u32x4_t*>(stg + tok * 512 + ((chunk ^ (tok & 15)) << 4)) = o;
+        }
+      }
+      // wave-private LDS is in order: the reads below see the writes above
+#pragma unroll
+      for (int it = 0; it < 32; ++it) {
+        const int row = 2 * it + s_rsub;                              // 0 .. 63
+        const u32x4_t o = *reinterpret_cast<const u32x4_t*>(stg + row * 512 + ((s_chunk ^ (row & 15)) << 4));
+        const int off = s_live ? ((64 * half + row) * N + s_n) * 4 : (int)0x80000000u;
+        __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_p, off, 0, 0);
       }
     }
     return;
@@ -1083,7 +1103,7 @@ GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   GemmPlan pl = {false, 1, 0, 0};
   const int KT = (K + BK - 1) / BK, cu = compute_units();
   const bool pipelined = K % 32 == 0 && K >= 64;
-  const double us_tile = pipelined ? 1.1 : 1.4, us_tile_small = 0.8, us_launch = 5.0, bytes_per_us = 3.0e6;
+  const double us_tile = pipelined ? 1.1 : 1.4, us_tile_small = 0.8, us_launch = 5.0, bytes_per_us = 6.0e6;
   double best = KT * us_tile;
   if (pipelined) {
     const int ni = pick_ni(M, N);
