@@ -796,8 +796,8 @@ def t2i_modulate(x, shift, scale):
 
 class MultiHeadCrossAttention(nn.Module):
     """Cross-attention to the text tokens (reference: sana_blocks.py:48-98, the scaled_dot_product_attention
-    branch): bf16 inference runs the attention itself as the short-key softmax kernel between stock linears;
-    everything else (other dtypes, training, more than 320 text tokens, 4-d masks) is stock ops."""
+    branch): bf16 inference runs the attention itself as the short-key softmax kernel; its linears are this library's
+    GEMM from 4096 rows and library GEMM calls below; everything else (other dtypes, training, more than 320 text tokens, 4-d masks) is stock ops."""
 
     def __init__(self, d_model, num_heads, attn_drop=0.0, proj_drop=0.0, qk_norm=False, **block_kwargs):
         super().__init__()
@@ -850,9 +850,12 @@ class MultiHeadCrossAttention(nn.Module):
                 and (mask is None or (mask.ndim == 2 and tuple(mask.shape) == (B, cond.shape[1])))
                 and self.q_linear.weight.dtype == torch.bfloat16):
             return None
-        # (q_linear and kv_linear stay library GEMM calls at their native width: at 16384 rows they take what this
-        # library's GEMM takes, at a few hundred rows they are faster, and they cost less host time per call)
-        q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
+        # (below 4096 rows q_linear and kv_linear are library GEMM calls: at a few hundred to a few thousand rows
+        # they are faster than this library's GEMM and cost less host time per call)
+        if B * N >= self.RESIDUAL_GEMM_MIN_ROWS and self.q_linear.bias is not None and x.is_contiguous():
+            q = ops.gemm_bf16(x.view(B * N, C), self.q_linear.weight, self.q_linear.bias, "bias").view(B, N, C)
+        else:
+            q = F.linear(x, self.q_linear.weight, self.q_linear.bias)
         if kv is None:
             kv = F.linear(cond, self.kv_linear.weight, self.kv_linear.bias)       # [B, Nk, 2C]
         if not isinstance(self.q_norm, nn.Identity):

@@ -82,12 +82,14 @@ def test_gemm_split_k_workspace_query():
     """Shapes with fewer output tiles than half the compute units (256 assumed without a device) are split
     along K through fp32 partial planes; shapes that fill the chip, short K loops and int8-only shapes are not."""
     lib = _lib.load()
-    # one 1024 px image at Sana-1.6B: point conv 1024 x 2240 x 5600 -> 4 x 12 tiles of 256 x 192, 88 k-tiles, 4 ranges
-    assert lib.sana_hip_gemm_workspace_bytes(1024, 2240, 5600) == 4 * 1024 * 2240 * 4
+    # one 1024 px image at Sana-1.6B: point conv 1024 x 2240 x 5600 -> 4 x 12 tiles of 256 x 192, 88 k-tiles, 5 ranges
+    assert lib.sana_hip_gemm_workspace_bytes(1024, 2240, 5600) == 5 * 1024 * 2240 * 4
+    # its proj GEMM (35 k-tiles): at most one range per 8 k-tiles
+    assert lib.sana_hip_gemm_workspace_bytes(1024, 2240, 2240) == 4 * 1024 * 2240 * 4
     # 256 tokens through the proj GEMM (35 k-tiles): at most one range per 8 k-tiles
     assert lib.sana_hip_gemm_workspace_bytes(256, 2240, 2240) == 4 * 256 * 2240 * 4
     # not split: grids that fill the chip, wide N or short K (the partial planes would cost more than the loop saves)
-    for M, N, K in ((16384, 2240, 5600), (16384, 11200, 2240), (1024, 11200, 2240), (1024, 2240, 2240),
+    for M, N, K in ((16384, 2240, 5600), (16384, 11200, 2240), (1024, 11200, 2240), (1024, 6720, 2240),
                     (1024, 3456, 1152), (1024, 2240, 512), (0, 8, 64), (256, 2244, 5600)):
         assert lib.sana_hip_gemm_workspace_bytes(M, N, K) == 0, (M, N, K)
 
