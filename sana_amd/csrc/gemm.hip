@@ -1091,7 +1091,7 @@ int mixed_split(int M, int N) {
 // units (M = 1024 tokens x N = 2240: 48 workgroups on 256 CUs) leaves most of the chip idle for the whole
 // chain; two remedies, by estimate:
 //  * split-k: S ranges of >= 8 k-tiles (S <= 8, S x tiles <= CUs) shorten the chain to ceil(KT / S) k-tiles and
-//    cost the fp32 partial planes (S x M x N x 4 bytes written and read once, about 3 bytes/ns at these sizes)
+//    cost the fp32 partial planes (S x M x N x 4 bytes written and read once, about 6 bytes/ns at these sizes)
 //    plus a second launch (about 5 us); taken when that beats the unsplit chain by 15 %.  Long-K narrow-N
 //    shapes (the point conv of a few thousand tokens or less) split, wide-N or short-K ones do not.
 //  * the 128 x 128 kernel, when its grid still fits one workgroup per CU and its chain beats the above.
