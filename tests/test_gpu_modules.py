@@ -378,6 +378,41 @@ def test_graphed_call_replays_a_chain_of_blocks(cuda):
         graphed(x[:1], y, t)
 
 
+def test_graphed_call_with_shared_conditioning_and_the_fused_routes(cuda):
+    """Two blocks at 4096 rows -- the qkv GEMM with the attention state in its epilogue, the cross-attention's
+    residual add in its projection GEMM -- with their StepConditioning evaluated inside the captured step: replays
+    equal the eager step bit for bit (every derived weight copy exists before the capture: GraphedCall warms up)."""
+    C, heads, B, HW = 288, 3, 2, (64, 32)          # cross-attention heads of 96, linear-attention heads of 32
+    blocks = []
+    for seed in (21, 22):
+        _, hb = _pair(C, heads, seed=seed)
+        blocks.append(hb.to(cuda))
+    cond = S.StepConditioning(blocks)
+    assert B * HW[0] * HW[1] >= blocks[0].attn.STATE_IN_QKV_GEMM_MIN_ROWS
+
+    def step(x, y, t):
+        for blk, c in zip(blocks, cond(y, t)):
+            x = blk(x, y, t, None, HW, None, **c)
+        return x
+
+    x, y, t = (a.bfloat16().to(cuda) for a in O.block_inputs(B, HW[0] * HW[1], C, seed=23))
+    graphed = S.GraphedCall(step, (x, y, t))
+    with torch.no_grad():
+        for r in range(3):
+            xr = torch.randn(x.shape, generator=torch.Generator().manual_seed(30 + r)).bfloat16().to(cuda)
+            yr = torch.randn(y.shape, generator=torch.Generator().manual_seed(40 + r)).bfloat16().to(cuda)
+            out = graphed(xr, yr, t)
+            torch.cuda.synchronize()
+            eager = step(xr, yr, t)
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {r}"
+        ref_blocks = [b for b in blocks]
+        own = xr
+        for blk in ref_blocks:                       # and the step without the shared conditioning: same function
+            own = blk(own, yr, t, None, HW, None)
+        assert ((eager.float() - own.float()).norm() / own.float().norm()).item() <= 2e-3
+
+
 def test_graph_replay_survives_a_larger_eager_shape(cuda):
     """A captured block holds the raw addresses of the scratch buffers it used (attention partial states, split-k
     planes).  A later, larger eager call makes the library take bigger buffers; the captured ones must stay alive
