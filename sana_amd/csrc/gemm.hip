@@ -1278,28 +1278,40 @@ int check_gate_res(const void* gate, const void* residual, int M, int N, int64_t
 }
 
 // Sum of the per-token-tile partial states of the fused qkv projection: part[bh][nsplit][33 * 32] -> state[bh][33 * 32].
-// A workgroup takes 64 elements of one (batch, head): four threads per element add every fourth tile in tile order
-// (independent loads, all in flight together), and the four sums are added in a fixed order -- deterministic.
+// One thread per element of one (batch, head) adds G-th tiles in tile order (batches of eight independent loads);
+// with G = 4 (many tiles per batch entry) four threads share an element and their sums are added in a fixed order.
+// Deterministic either way.
+template <int G>
 __global__ __launch_bounds__(256) void qkv_state_reduce_kernel(const float* __restrict__ part, float* __restrict__ state,
-                                                                int nsplit) {
-  constexpr int ELEMS = 33 * 32, SLICES = (ELEMS + 63) / 64;
-  __shared__ float red[4][64];
-  const int bh = blockIdx.x / SLICES, e = (blockIdx.x % SLICES) * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
+                                                                int nsplit, int total) {
+  constexpr int ELEMS = 33 * 32, PER = 256 / G;
+  __shared__ float red[G][PER];
+  const int local = threadIdx.x % PER, grp = threadIdx.x / PER;
+  const int gid = blockIdx.x * PER + local;  // element of the whole state array
   float s = 0.f;
-  if (e < ELEMS) {
+  if (gid < total) {
+    const int bh = gid / ELEMS, e = gid - bh * ELEMS;
     const float* p = part + ((int64_t)bh * nsplit) * ELEMS + e;
-    for (int sp0 = grp; sp0 < nsplit; sp0 += 32) {
+    for (int sp0 = grp; sp0 < nsplit; sp0 += 8 * G) {
       float v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = (sp0 + 4 * u < nsplit) ? p[(int64_t)(sp0 + 4 * u) * ELEMS] : 0.f;
+      for (int u = 0; u < 8; ++u) v[u] = (sp0 + G * u < nsplit) ? p[(int64_t)(sp0 + G * u) * ELEMS] : 0.f;
 #pragma unroll
       for (int u = 0; u < 8; ++u) s += v[u];
     }
   }
-  red[grp][threadIdx.x & 63] = s;
+  if (G == 1) {
+    if (gid < total) state[gid] = s;
+    return;
+  }
+  red[grp][local] = s;
   __syncthreads();
-  if (grp == 0 && e < ELEMS)
-    state[(int64_t)bh * ELEMS + e] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+  if (grp == 0 && gid < total) {
+    float t = red[0][local];
+#pragma unroll
+    for (int g = 1; g < G; ++g) t += red[g][local];
+    state[gid] = t;
+  }
 }
 
 // Rows of the fused qkv projection's weight layout for C = 32 * heads channels: the q rows padded to whole 256-wide
@@ -1417,7 +1429,7 @@ SANA_API int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const v
                                      int64_t lda, int64_t ldw, int64_t ldq, void* stream) {
   if (!A || !W_tiled || !Q || !state || B <= 0 || N <= 0 || C <= 0 || heads <= 0) return SANA_ERR_ARG;
   if (C != 32 * heads || N % 256 || C < 64) return SANA_ERR_SHAPE;
-  if ((int64_t)B * N >= ((int64_t)1 << 31) / 2) return SANA_ERR_SHAPE;
+  if ((int64_t)B * N >= ((int64_t)1 << 30) || (int64_t)B * heads * 33 * 32 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;
   const int M = B * N, rows_t = qkv_state_rows_total(C, heads);
   if (lda < C || ldw < C || ldq < C) return SANA_ERR_ARG;
   if (lda >= (1 << 22) || ldw >= (1 << 22) || ldq >= (1 << 22)) return SANA_ERR_SHAPE;
@@ -1437,7 +1449,12 @@ SANA_API int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const v
                      static_cast<const uint16_t*>(A), W_tiled, static_cast<const float*>(nullptr), e,
                      static_cast<uint16_t*>(Q), M, rows_t, C, lda, ldw, ldq, (int)tiles_t, (int)tiles_c, none);
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
-  hipLaunchKernelGGL(qkv_state_reduce_kernel, dim3((unsigned)(B * heads * ((33 * 32 + 63) / 64))), dim3(256), 0, s,
-                     static_cast<const float*>(workspace), state, N / 256);
+  const int total = B * heads * 33 * 32, nsplit = N / 256;
+  if (nsplit > 16)
+    hipLaunchKernelGGL(qkv_state_reduce_kernel<4>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
+                       static_cast<const float*>(workspace), state, nsplit, total);
+  else
+    hipLaunchKernelGGL(qkv_state_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const float*>(workspace), state, nsplit, total);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
