@@ -1140,38 +1140,42 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
   const int tiles_t = (M + BT - 1) / BT, tiles_c = (N + 64 * NI - 1) / (64 * NI);
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
   const Taps none = {0, 0, 0, 0, 0, nullptr};
-  if (!taps && ws) {  // split-k when it pays and the caller's workspace holds the partial planes
-    const GemmPlan pl = plan_gemm(M, N, K, W8);
-    if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
-      const Taps split = {0, 0, 0, pl.tiles, pl.rem, nullptr};
-      hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, 0, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
-                         a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
-                         split);
-      if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
-      const int64_t threads = (int64_t)M * (N / 8);
-      dim3 egrid((unsigned)((threads + 255) / 256));
+  if constexpr (NI != 2) {  // the 128-wide tile exists unsplit and without taps only
+    if (!taps && ws) {  // split-k when it pays and the caller's workspace holds the partial planes
+      const GemmPlan pl = plan_gemm(M, N, K, W8);
+      if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
+        const Taps split = {0, 0, 0, pl.tiles, pl.rem, nullptr};
+        hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, 0, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
+                           a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
+                           split);
+        if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
+        const int64_t threads = (int64_t)M * (N / 8);
+        dim3 egrid((unsigned)((threads + 255) / 256));
 #define SANA_SPLIT_EPI(EPI) \
   hipLaunchKernelGGL((splitk_epilogue_kernel<EPI>), egrid, block, 0, s, ws, pl.S, ep, c, M, N, ldc)
-      switch (epilogue) {
-        case SANA_EPI_NONE: SANA_SPLIT_EPI(SANA_EPI_NONE); break;
-        case SANA_EPI_BIAS: SANA_SPLIT_EPI(SANA_EPI_BIAS); break;
-        case SANA_EPI_BIAS_SILU: SANA_SPLIT_EPI(SANA_EPI_BIAS_SILU); break;
-        case SANA_EPI_GATE_RES: SANA_SPLIT_EPI(SANA_EPI_GATE_RES); break;
-        default: return SANA_ERR_ARG;
-      }
+        switch (epilogue) {
+          case SANA_EPI_NONE: SANA_SPLIT_EPI(SANA_EPI_NONE); break;
+          case SANA_EPI_BIAS: SANA_SPLIT_EPI(SANA_EPI_BIAS); break;
+          case SANA_EPI_BIAS_SILU: SANA_SPLIT_EPI(SANA_EPI_BIAS_SILU); break;
+          case SANA_EPI_GATE_RES: SANA_SPLIT_EPI(SANA_EPI_GATE_RES); break;
+          default: return SANA_ERR_ARG;
+        }
 #undef SANA_SPLIT_EPI
+        return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+      }
+    }
+    if (taps) {  // only the bf16 gated-residual instance exists with taps
+      if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
+      if (taps->zero_last)
+        hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
+                           lda, ldw, ldc, tiles_t, tiles_c, *taps);
+      else
+        hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 1>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
+                           lda, ldw, ldc, tiles_t, tiles_c, *taps);
       return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
     }
-  }
-  if (taps) {  // only the bf16 gated-residual instance exists with taps
-    if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
-    if (taps->zero_last)
-      hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
-                         lda, ldw, ldc, tiles_t, tiles_c, *taps);
-    else
-      hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 1>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
-                         lda, ldw, ldc, tiles_t, tiles_c, *taps);
-    return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+  } else {
+    if (taps) return SANA_ERR_ARG;
   }
 #define SANA_LAUNCH4(EPI)                                                                                         \
   hipLaunchKernelGGL((gemm4_kernel<W8, EPI, NI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
@@ -1235,6 +1239,14 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
                               scale ? scale + n_wide : nullptr, ep2, c + n_wide, M, N - n_wide, K, lda, ldw, ldc, epilogue,
                               s, nullptr, nullptr, 0);
       }
+    }
+    // Few tokens, wide N (qkv of one 1024 px image: 4 x 35 tiles of 192 channels on 256 CUs): 128-wide tiles put
+    // half as much math behind every k-tile of the chain and fill more of the chip (4 x 53 workgroups: 37 -> 31 us).
+    // bf16 weights only; taken when the 192-wide grid leaves a fifth of the CUs idle and the 128-wide one still fits.
+    if constexpr (!W8) {
+      const int64_t t128 = tiles_t * ((N + 127) / 128), t192 = tiles_t * ((N + 191) / 192);
+      if (!taps && t128 <= compute_units() && t192 < compute_units() * 4 / 5 && plan_gemm(M, N, K, W8).S == 1)
+        return launch4<W8, 2>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
     }
     return pick_ni(M, N) == 3
                ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes)

@@ -170,6 +170,32 @@ def test_gemm_mixed_channel_tiling_is_bit_identical(cuda, w8):
         assert torch.equal(whole[0, :256], head[0])
 
 
+def test_gemm_128_wide_tiles_are_bit_identical_to_the_wider_ones(cuda):
+    """1024 tokens x 6720 channels (qkv of one image) runs 128-wide tiles: 4 x 53 workgroups instead of 4 x 35 of 192
+    channels.  The same rows inside a 16384-token call run the 256- / 192-wide tiles: same k order per output, so
+    bit for bit the same; int8 weights (another instance, 192-wide) as well; every epilogue kind."""
+    from sana_amd.modules import quantize_w8
+    M, N, K = 1024, 6720, 2240
+    g = torch.Generator().manual_seed(19)
+    big = torch.randn(16384, K, generator=g).bfloat16().to(cuda)
+    a = big[5120:5120 + M]
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    wq, sc = quantize_w8(w)
+    w = (wq.float() * sc[:, None]).bfloat16().to(cuda)          # the dequantised weight: both routes see the same values
+    bias = (torch.randn(N, generator=g) * 0.5).bfloat16().to(cuda)
+    for epi in (None, "bias", "bias_silu"):
+        b = bias if epi else None
+        narrow = ops.gemm_bf16(a, w, b, epi)
+        assert torch.equal(narrow, ops.gemm_bf16(big, w, b, epi)[5120:5120 + M]), epi
+        assert torch.equal(narrow, ops.gemm_w8a16(a, wq.to(cuda), sc.to(cuda), b, epi, expand=False)), epi
+    gate = (torch.randn(1, 1, N, generator=g) * 0.5).bfloat16().to(cuda)
+    res = torch.randn(1, 16384, N, generator=g).bfloat16().to(cuda)
+    narrow = ops.gemm_gate_residual(a.view(1, M, K), w, bias, gate, res[:, 5120:5120 + M])
+    assert torch.equal(narrow[0], ops.gemm_gate_residual(big.view(1, 16384, K), w, bias, gate, res)[0, 5120:5120 + M])
+    ref = a.double() @ w.double().T + bias.double()
+    assert rel_l2(ops.gemm_bf16(a, w, bias, "bias").cpu(), ref.cpu()) <= 4e-3
+
+
 def test_gemm_exact_on_integer_inputs(cuda):
     """Small integers: every product and partial sum is exact in fp32, the result is exact in bf16."""
     g = torch.Generator().manual_seed(3)
