@@ -698,7 +698,8 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
 // wave per SIMD with the whole register file (256 accumulators + 256 VGPRs), each
 // wave a sub-tile of 128 tokens x 32*NI channels = 2*NI x 8 MFMA tiles of 16x16
 // (NI = 4: 128x128; NI = 3 narrows the workgroup's channel tile to 192 where that fills
-// the last round of workgroups better).  With a single wave per SIMD nothing
+// the last round of workgroups better, NI = 2 to 128 for few tokens and wide N, where the
+// shorter k-tile and the larger grid shorten the latency chain).  With a single wave per SIMD nothing
 // else hides a stalled memory instruction, so the main loop is one hand-ordered
 // stream (pinned with sched_barrier): a k-tile is two k-steps of 32 = 2 * 16*NI MFMA
 // slots of 16 cycles, and a lone wave issues about one other instruction per 5 cycles,
