@@ -281,7 +281,8 @@ int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_sc
  *   [3C][C] qkv weight (and entry of its bias) that row i of W_tiled holds, or -1 for a zero row.  With rows ==
  *   NULL the function returns the number of rows; with a buffer of that capacity it fills it (host code, no GPU).
  *   A: bf16 [B*N][C] (row stride lda); W_tiled: bf16 [rows][C] (row stride ldw); bias_tiled: bf16 [rows] or NULL.
- *   N % 256 == 0, C == 32 * heads.  workspace: sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads) bytes (one
+ *   C == 32 * heads; N % 256 == 0, or B == 1 and no bias (a ragged last tile's missing rows are then zeros that add
+ *   nothing to the state).  workspace: sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads) bytes (one
  *   partial state per 256 tokens, added in token order by a second launch: deterministic, no atomics). */
 int sana_hip_qkv_state_rows(int C, int heads, int32_t* rows, int capacity);
 size_t sana_hip_gemm_qkv_state_workspace_bytes(int B, int N, int heads);

@@ -1433,15 +1433,18 @@ SANA_API int sana_hip_qkv_state_rows(int C, int heads, int32_t* rows, int capaci
 }
 
 SANA_API size_t sana_hip_gemm_qkv_state_workspace_bytes(int B, int N, int heads) {
-  if (B <= 0 || N <= 0 || heads <= 0 || N % 256) return 0;
-  return (size_t)B * heads * (N / 256) * 33 * 32 * sizeof(float);
+  if (B <= 0 || N <= 0 || heads <= 0 || (N % 256 && B != 1)) return 0;
+  return (size_t)B * heads * ((N + 255) / 256) * 33 * 32 * sizeof(float);
 }
 
 SANA_API int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const void* bias_tiled, void* Q, float* state,
                                      void* workspace, size_t workspace_bytes, int B, int N, int C, int heads,
                                      int64_t lda, int64_t ldw, int64_t ldq, void* stream) {
   if (!A || !W_tiled || !Q || !state || B <= 0 || N <= 0 || C <= 0 || heads <= 0) return SANA_ERR_ARG;
-  if (C != 32 * heads || N % 256 || C < 64) return SANA_ERR_SHAPE;
+  if (C != 32 * heads || C < 64) return SANA_ERR_SHAPE;
+  // a token tile must not straddle two batch entries, and the rows of a ragged last tile must contribute nothing to
+  // the state: they read as zero activations, which stay zero only without a bias
+  if (N % 256 && (B != 1 || bias_tiled)) return SANA_ERR_SHAPE;
   if ((int64_t)B * N >= ((int64_t)1 << 30) || (int64_t)B * heads * 33 * 32 >= ((int64_t)1 << 31)) return SANA_ERR_SHAPE;
   const int M = B * N, rows_t = qkv_state_rows_total(C, heads);
   if (lda < C || ldw < C || ldq < C) return SANA_ERR_ARG;
@@ -1452,17 +1455,17 @@ SANA_API int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const v
   const size_t need = sana_hip_gemm_qkv_state_workspace_bytes(B, N, heads);
   if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
   if (!aligned16(workspace)) return SANA_ERR_ALIGN;
-  const int64_t tiles_t = M / BT, tiles_c = rows_t / 256;
+  const int64_t tiles_t = (M + BT - 1) / BT, tiles_c = rows_t / 256;
   if (tiles_t * tiles_c > (1 << 30)) return SANA_ERR_SHAPE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const EpiArgs e = {static_cast<const uint16_t*>(bias_tiled), nullptr, nullptr, 0, 0, 1, static_cast<float*>(workspace),
-                     C, qkv_state_q_pad(C), heads, N / 256};
+                     C, qkv_state_q_pad(C), heads, (N + 255) / 256};
   const Taps none = {0, 0, 0, 0, 0, nullptr};
   hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_QKV_STATE, 4>), dim3((unsigned)(tiles_t * tiles_c)), dim3(256), 0, s,
                      static_cast<const uint16_t*>(A), W_tiled, static_cast<const float*>(nullptr), e,
                      static_cast<uint16_t*>(Q), M, rows_t, C, lda, ldw, ldq, (int)tiles_t, (int)tiles_c, none);
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
-  const int total = B * heads * 33 * 32, nsplit = N / 256;
+  const int total = B * heads * 33 * 32, nsplit = (N + 255) / 256;
   if (nsplit > 16)
     hipLaunchKernelGGL(qkv_state_reduce_kernel<4>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
                        static_cast<const float*>(workspace), state, nsplit, total);

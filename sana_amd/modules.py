@@ -301,7 +301,7 @@ class LiteLA(nn.Module):
         return (x.is_cuda and self.dim == 32 and B * N >= self.STATE_IN_QKV_GEMM_MIN_ROWS
                 and isinstance(self.q_norm, nn.Identity) and isinstance(self.k_norm, nn.Identity)
                 and (self.qkv.is_quantized or self.qkv.weight.dtype == torch.bfloat16)
-                and ops.qkv_state_supported(N, C, self.heads))
+                and ops.qkv_state_supported(N, C, self.heads, B, self.qkv.bias is not None))
 
     def _tiled_qkv(self):
         """The qkv weight (and bias) in the fused GEMM's row layout: derived data, rebuilt when the parameters

@@ -392,19 +392,24 @@ def tile_qkv_weight(weight: torch.Tensor, bias: Optional[torch.Tensor], heads: i
     return tile_qkv_rows(weight, heads), None if bias is None else tile_qkv_rows(bias, heads)
 
 
-def qkv_state_supported(n_tokens: int, C: int, heads: int) -> bool:
-    return heads > 0 and C == 32 * heads and C >= 64 and n_tokens > 0 and n_tokens % 256 == 0
+def qkv_state_supported(n_tokens: int, C: int, heads: int, batch: int = 2, has_bias: bool = True) -> bool:
+    """Shapes sana_hip_gemm_qkv_state takes: whole 256-token tiles per batch entry -- or one batch entry and no bias,
+    where the ragged last tile's missing rows are zeros that add nothing to the state."""
+    return heads > 0 and C == 32 * heads and C >= 64 and n_tokens > 0 and \
+        (n_tokens % 256 == 0 or (batch == 1 and not has_bias))
 
 
 def gemm_qkv_state(x: torch.Tensor, w_tiled: torch.Tensor, bias_tiled: Optional[torch.Tensor], heads: int):
-    """qkv projection with phase 1 of the linear attention in its epilogue.  x: [B, N, C] bf16 (N % 256 == 0),
+    """qkv projection with phase 1 of the linear attention in its epilogue.  x: [B, N, C] bf16 (N % 256 == 0, or B == 1
+    and no bias),
     w_tiled / bias_tiled: ``tile_qkv_weight``'s.  Returns (q [B, N, C] bf16, state [B, heads, 1, 33, 32] fp32)."""
     _need_cuda(x, w_tiled, bias_tiled)
     if x.dim() != 3 or x.dtype != torch.bfloat16 or w_tiled.dtype != torch.bfloat16:
         raise SanaHipError("gemm_qkv_state needs a bf16 [B, N, C] input and a bf16 tiled weight")
     B, N, C = x.shape
-    if not qkv_state_supported(N, C, heads):
-        raise SanaHipError(f"gemm_qkv_state needs N % 256 == 0 and C == 32 * heads, got N={N}, C={C}, heads={heads}")
+    if not qkv_state_supported(N, C, heads, B, bias_tiled is not None):
+        raise SanaHipError(f"gemm_qkv_state needs C == 32 * heads and N % 256 == 0 (or one batch entry and no bias), "
+                           f"got B={B}, N={N}, C={C}, heads={heads}, bias {'given' if bias_tiled is not None else 'absent'}")
     lib = _lib.load()
     if tuple(w_tiled.shape) != (lib.sana_hip_qkv_state_rows(C, heads, None, 0), C):
         raise SanaHipError(f"tiled weight of shape {tuple(w_tiled.shape)} does not fit C={C}, heads={heads}")

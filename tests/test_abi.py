@@ -127,6 +127,7 @@ def test_qkv_state_row_map_is_a_layout_of_the_qkv_weight():
     assert lib.sana_hip_qkv_state_rows(64, 2, ctypes.cast((ctypes.c_int32 * 4)(), ctypes.c_void_p), 4) < 0
     assert lib.sana_hip_gemm_qkv_state_workspace_bytes(2, 512, 3) == 2 * 3 * 2 * 33 * 32 * 4
     assert lib.sana_hip_gemm_qkv_state_workspace_bytes(2, 500, 3) == 0
+    assert lib.sana_hip_gemm_qkv_state_workspace_bytes(1, 500, 3) == 3 * 2 * 33 * 32 * 4   # one entry: a ragged last tile
 
 
 def test_gemm_qkv_state_refuses_bad_arguments_before_any_launch():
@@ -139,6 +140,8 @@ def test_gemm_qkv_state_refuses_bad_arguments_before_any_launch():
     bad = lambda i, v: good[:i] + [v] + good[i + 1:]
     assert call(*bad(0, None)) == -1 and call(*bad(3, None)) == -1 and call(*bad(7, 0)) == -1     # SANA_ERR_ARG
     assert call(*bad(8, 500)) == -2 and call(*bad(10, 4)) == -2                                    # SANA_ERR_SHAPE
+    one = [P, P, P, P, P, P, ws, 1, 500, 96, 3, 96, 96, 96]      # one batch entry, ragged N: refused with a bias only
+    assert call(*one) == -2
     assert call(*bad(11, 64)) == -1                                                                # lda < C
     assert call(*bad(0, P + 2)) == -3 and call(*bad(12, 100)) == -3                                # SANA_ERR_ALIGN
     assert call(*bad(6, 1024)) == -4 and call(*bad(5, None)) == -4                                 # SANA_ERR_WORKSPACE

@@ -29,6 +29,8 @@ CASES = [
     (4, 1024, 1152, 36, True),    # cfg2 attention shape: q region padded 1152 -> 1280
     (1, 16384, 2240, 70, False),  # cfg3: 64 partial states per head
     (16, 1024, 2240, 70, False),  # 1024 px, B = 16
+    (1, 4100, 2240, 70, False),   # one batch entry, no bias: a ragged last token tile (4 rows of 256 exist)
+    (1, 300, 64, 2, False),
 ]
 
 
@@ -63,7 +65,11 @@ def test_fused_qkv_state_is_deterministic_and_rejects_other_shapes(cuda):
     q2, s2 = ops.gemm_qkv_state(x, wt, bt, 5)
     assert torch.equal(q1, q2) and torch.equal(s1, s2)
     with pytest.raises(ops.SanaHipError):
-        ops.gemm_qkv_state(x[:, :700], wt, bt, 5)              # N % 256 != 0
+        ops.gemm_qkv_state(x[:, :700], wt, bt, 5)              # N % 256 != 0 with two batch entries
+    with pytest.raises(ops.SanaHipError):
+        ops.gemm_qkv_state(x[:1, :700], wt, bt, 5)             # ... and with one, but a bias
+    q3, s3 = ops.gemm_qkv_state(x[:1, :700].contiguous(), wt, None, 5)   # one entry, no bias: taken
+    assert q3.shape == (1, 700, 160) and torch.isfinite(s3).all()
     with pytest.raises(ops.SanaHipError):
         ops.gemm_qkv_state(x, wt[:-256], bt, 5)                # a weight that is not the tiled layout of these shapes
     with pytest.raises(ops.SanaHipError):
