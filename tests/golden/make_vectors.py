@@ -1,5 +1,6 @@
 """Writes ``tests/golden/kat.npz``: known-answer vectors for the linear-attention (plain, chunk-causal, rotary) and
-depthwise-gate kernels, computed in fp64 by the plain-C quadratic-form / 9-tap restatement (``oracle/bruteforce.c``).
+depthwise-gate kernels and for the qkv projection with the attention state in its epilogue, computed in fp64 by the plain-C
+quadratic-form / 9-tap restatement (``oracle/bruteforce.c``).
 
 The reference holds no numeric fixtures for this path, so these vectors are the build's own: they
 freeze the brute-force answers on seeded inputs (all exactly representable in bf16), and both the
@@ -57,6 +58,15 @@ def main():
                     f"{tag}_chunk_of": chunk_of,
                     f"{tag}_out": cbrute.relu_attention_rope(q, k, v, freqs, 1e-8),
                     f"{tag}_cc_out": cbrute.relu_attention_rope(q, k, v, freqs, 1e-8, chunk_of)})
+    # qkv projection + attention state on small integers: every product, sum and rounding on the way is exact in
+    # bf16 / fp32 (|q|, |k|, |v| <= 128, state entries < 2^23), so the answer is THE answer, bit for bit.
+    # x [1, 512, 64], w [192, 64] (nn.Linear layout: q rows, k rows, v rows; two heads of 32)
+    x = torch.randint(-2, 3, (1, 512, 64), generator=g).double().numpy()
+    w = torch.randint(-1, 2, (192, 64), generator=g).double().numpy()
+    qkv = x @ w.T                                                     # [1, 512, 192]
+    heads = lambda t: np.ascontiguousarray(t.reshape(512, 2, 32).transpose(1, 0, 2))   # [BH = 2, N, d]
+    vec.update(qkvs_x=x, qkvs_w=w, qkvs_q=qkv[..., :64],
+               qkvs_state=cbrute.attention_state(heads(qkv[0, :, 64:128]), heads(qkv[0, :, 128:])))
     np.savez_compressed(OUT, **vec)
     print(f"wrote {OUT}: {os.path.getsize(OUT)} bytes, {len(vec)} arrays")
 

@@ -165,3 +165,29 @@ def test_kernels_rotary_family_reproduce_fixture(cuda, tag, d):
         ksum = torch.relu(k).transpose(0, 1).reshape(N, BH, d)
         want = ksum.sum(0) if chunks is None else ksum[:12].sum(0)
         assert rel_l2(state[0, :, 0, d].cpu(), want) <= 1e-6
+
+
+# ----------------------------------------------------------------------------- qkv projection + state, exact integers
+
+def test_oracle_qkv_projection_and_state_reproduce_fixture():
+    """The oracle's LiteLA pieces on the integer fixture: linear -> q, and v . relu(k)^T with the row of ones."""
+    x, w = T("qkvs_x"), T("qkvs_w")
+    qkv = F.linear(x, w)                                               # [1, N, 3C]
+    assert torch.equal(qkv[..., :64], T("qkvs_q"))
+    k, v = (qkv[0, :, 64 * i:64 * (i + 1)].reshape(-1, 2, 32).permute(1, 0, 2) for i in (1, 2))   # [h, N, d]
+    _, state = O.relu_linear_attention(k.transpose(1, 2)[None], k[None], v.transpose(1, 2)[None], 1e-8, return_state=True)
+    assert torch.equal(state[0], T("qkvs_state"))
+
+
+@pytest.mark.gpu
+def test_kernel_qkv_projection_with_state_reproduces_fixture_exactly(cuda):
+    """sana_hip_gemm_qkv_state on the integer fixture (two token tiles, two heads, one k / v column tile with two
+    dummy heads): q and the state bit for bit -- nothing on the way rounds -- and the unfused pair of launches too."""
+    from sana_amd import ops
+    x, w = T("qkvs_x").bfloat16().to(cuda), T("qkvs_w").bfloat16().to(cuda)
+    wt, _ = ops.tile_qkv_weight(w, None, 2)
+    q, state = ops.gemm_qkv_state(x, wt, None, 2)
+    assert torch.equal(q.double().cpu(), T("qkvs_q"))
+    assert torch.equal(state[0, :, 0].double().cpu(), T("qkvs_state"))
+    qkv = ops.gemm_bf16(x.view(-1, 64), w).view(1, -1, 3, 64)
+    assert torch.equal(ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2])[0, :, 0].double().cpu(), T("qkvs_state"))
