@@ -1243,8 +1243,8 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
     }
     // Few tokens, wide N (qkv of one 1024 px image: 4 x 35 tiles of 192 channels on 256 CUs): 128-wide tiles put
     // half as much math behind every k-tile of the chain and fill more of the chip (4 x 53 workgroups: 37 -> 31 us).
-    // bf16 weights only; taken when the 192-wide grid leaves a fifth of the CUs idle and the 128-wide one still fits.
-    if constexpr (!W8) {
+    // Taken when the 192-wide grid leaves a fifth of the CUs idle and the 128-wide one still fits.
+    {
       const int64_t t128 = tiles_t * ((N + 127) / 128), t192 = tiles_t * ((N + 191) / 192);
       if (!taps && t128 <= compute_units() && t192 < compute_units() * 4 / 5 && plan_gemm(M, N, K, W8).S == 1)
         return launch4<W8, 2>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);

@@ -173,7 +173,7 @@ def test_gemm_mixed_channel_tiling_is_bit_identical(cuda, w8):
 def test_gemm_128_wide_tiles_are_bit_identical_to_the_wider_ones(cuda):
     """1024 tokens x 6720 channels (qkv of one image) runs 128-wide tiles: 4 x 53 workgroups instead of 4 x 35 of 192
     channels.  The same rows inside a 16384-token call run the 256- / 192-wide tiles: same k order per output, so
-    bit for bit the same; int8 weights (another instance, 192-wide) as well; every epilogue kind."""
+    bit for bit the same; the int8-weight instances (also 128-wide here) as well; every epilogue kind."""
     from sana_amd.modules import quantize_w8
     M, N, K = 1024, 6720, 2240
     g = torch.Generator().manual_seed(19)
