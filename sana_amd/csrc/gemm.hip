@@ -887,8 +887,11 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
       fa[buf][r - 1] = *reinterpret_cast<const u32x4_t*>(st + a_off + (r - 1) * 16 * ROW_BYTES + col);
     }
   };
+  // MFMA t of a k-step: weight tile t / 8, and the token tiles in alternating direction (0..7, 7..0, ..), so that
+  // every MFMA differs from its predecessor in ONE operand -- at the end of a row of eight only the weight fragment
+  // changes, not both.  Less switching on the operand buses: the power-limited clock settles ~1 % higher.
   auto mfma = [&](int buf, int t) {  // t < 8 * NWT
-    const int i = t >> 3, j = t & 7;
+    const int i = t >> 3, j = (i & 1) ? 7 - (t & 7) : (t & 7);
     mfma_acc(acc[i][j], fw[buf][i], fa[buf][j]);
   };
 
@@ -1009,7 +1012,10 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
       for (int i = 0; i < NWT; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mfma_acc(acc[i][j], w8[i], a8[j]);
+        for (int jj = 0; jj < 8; ++jj) {
+          const int j = (i & 1) ? 7 - jj : jj;
+          mfma_acc(acc[i][j], w8[i], a8[j]);
+        }
     }
     // the MFMAs are asm statements, so the compiler does not know that their results are in flight: wait out the
     // last ones before anything reads an accumulator
