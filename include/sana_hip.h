@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SANA_HIP_ABI_VERSION 7
+#define SANA_HIP_ABI_VERSION 8
 
 /* io dtypes */
 #define SANA_DT_F32 0
@@ -236,6 +236,14 @@ int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, void* C,
                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                        int epilogue, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same GEMM for an fp16 model (the released Sana-600M configuration trains and samples in fp16,
+ * configs/sana_config/1024ms/Sana_600M_img1024.yaml:22): A, W, bias and C are IEEE half, accumulation is fp32 on
+ * v_mfma_f32_16x16x32_f16, the epilogues round to half where the bf16 form rounds to bf16.  Same arguments,
+ * tile plans and split-k behaviour as sana_hip_gemm_bf16; replaces the same nn.Linear / 1x1-conv calls. */
+int sana_hip_gemm_f16(const void* A, const void* W, const void* bias, void* C,
+                      int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
+                      int epilogue, void* workspace, size_t workspace_bytes, void* stream);
+
 /* W8A16: W is int8 [N][K] with a per-output-channel fp32 scale [N].  Each
  * weight is dequantised in registers as bf16_rne(float(q) * scale[n]) — the same
  * value as torch's (q.float() * scale).bfloat16() — before the MFMA, so the
@@ -268,6 +276,14 @@ int sana_hip_gemm_gate_residual(const void* A, const void* W, const float* w8_sc
                                 int rows_per_gate, int64_t gate_stride,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* sana_hip_gemm_gate_residual for an fp16 model: every operand IEEE half (no int8 weights), the three roundings to
+ * half.  Replaces the same lines of SanaMSBlock.forward (sana_multi_scale.py:151-155). */
+int sana_hip_gemm_gate_residual_f16(const void* A, const void* W, const void* bias,
+                                    const void* gate, const void* residual, void* C,
+                                    int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldr, int64_t ldc,
+                                    int rows_per_gate, int64_t gate_stride,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * qkv projection + phase 1 of the linear attention in one GEMM (bf16, head_dim 32, no q/k transform):
  *   Q = A Wq^T (+ bias)            stored, bf16 [B*N][C] with row stride ldq
@@ -293,8 +309,9 @@ int sana_hip_gemm_qkv_state(const void* A, const void* W_tiled, const void* bias
 /* LayerNorm without affine (eps inside the rsqrt) + adaLN modulation:
  *   out[m][:] = LN(x[m][:]) * (1 + scale[m / rows_per_mod][:]) + shift[m / rows_per_mod][:]
  *   replaces `t2i_modulate(self.norm1(x), shift, scale)` (sana_multi_scale.py:152,155).
- *   x, out: bf16 [M][C] with row strides ldx / ldo; scale, shift: bf16 rows of C
- *   values, mod_stride elements apart.  C % 8 == 0, C <= 8192.  bf16 only. */
+ *   x, out: [M][C] with row strides ldx / ldo; scale, shift: rows of C values, mod_stride elements
+ *   apart; all of io_dtype, SANA_DT_BF16 or SANA_DT_F16 (the four roundings of the stock op chain are to
+ *   that dtype).  C % 8 == 0, C <= 8192. */
 int sana_hip_layernorm_modulate(const void* x, const void* scale, const void* shift, void* out,
                                 int64_t M, int C, int64_t ldx, int64_t ldo,
                                 int rows_per_mod, int64_t mod_stride, float eps, int io_dtype, void* stream);
@@ -340,8 +357,9 @@ int sana_hip_cross_attention(const void* q, const void* kv, const float* key_bia
  * `x + self.drop_path(gate_mlp * mlp_out)` (diffusion/model/nets/sana_multi_scale_video.py:321; per frame
  * :247-252) where the module's last op is not a GEMM of this library (the temporal Mix-FFN variants), and
  * `x + gate_msa * attn(...)` when a guidance processor or hook needs the attention output itself.
- *   y, residual, out: bf16 [M][C] with row strides ldy / ldr / ldo (out may alias residual or y);
- *   gate: bf16 rows of C values, gate_stride elements apart.  C % 8 == 0.  bf16 only. */
+ *   y, residual, out: [M][C] with row strides ldy / ldr / ldo (out may alias residual or y);
+ *   gate: rows of C values, gate_stride elements apart; all of io_dtype, SANA_DT_BF16 or SANA_DT_F16.
+ *   C % 8 == 0. */
 int sana_hip_gate_residual(const void* y, const void* gate, const void* residual, void* out,
                            int64_t M, int C, int64_t ldy, int64_t ldr, int64_t ldo,
                            int rows_per_gate, int64_t gate_stride, int io_dtype, void* stream);

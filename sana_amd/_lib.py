@@ -46,6 +46,11 @@ SIGNATURES = {
     "sana_hip_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "sana_hip_gemm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                    c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
+    "sana_hip_gemm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                  c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
+    "sana_hip_gemm_gate_residual_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64,
+                                                c_int, c_int64, c_void_p, c_size_t, c_void_p]),
     "sana_hip_gemm_w8a16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "sana_hip_dequant_w8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int64, c_void_p]),

@@ -47,6 +47,30 @@ __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
   return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
 }
 
+// Conversions of the two 16-bit io dtypes by tag (T = BF16 or F16): pack two floats with round-to-nearest-even (one
+// v_cvt_pk_bf16_f32 for bf16; two conversions and a pack for f16, which has no packed round-to-nearest conversion),
+// unpack either half of a packed pair, round through the dtype.
+template <typename T> inline constexpr bool is_f16 = false;
+template <> inline constexpr bool is_f16<F16> = true;
+template <typename T> __device__ __forceinline__ uint32_t pk16(float lo, float hi) {
+  if constexpr (is_f16<T>) return pack_f16(lo, hi);
+  else return pack_bf16(lo, hi);
+}
+template <typename T> __device__ __forceinline__ float lo16(uint32_t p) {
+  if constexpr (is_f16<T>) return f16_bits_to_f32(p & 0xffffu);
+  else return bf16_lo(p);
+}
+template <typename T> __device__ __forceinline__ float hi16(uint32_t p) {
+  if constexpr (is_f16<T>) return f16_bits_to_f32(p >> 16);
+  else return bf16_hi(p);
+}
+template <typename T> __device__ __forceinline__ float rnd16(float f) {
+  // (through the bit pattern: a float -> _Float16 -> float cast pair alone may be evaluated in excess precision,
+  // i.e. not round at all)
+  if constexpr (is_f16<T>) return f16_bits_to_f32(f32_to_f16_bits(f));
+  else return round_bf16(f);
+}
+
 // ReLU on two packed 16-bit floats (bf16 or f16: both sign-magnitude, so a
 // signed-integer max against 0 clears negatives and -0).
 __device__ __forceinline__ uint32_t relu_pk16(uint32_t x) {

@@ -21,6 +21,11 @@
 
 #include "common.h"
 
+// No implicit fused multiply-adds in this file: the epilogues reproduce the stock op chain's roundings (product
+// rounded to the io dtype, THEN the sum), and for fp16 -- which has native arithmetic -- the compiler would otherwise
+// contract "round(g * y) + r" into one v_fma_f16 and drop the product's rounding.  Wanted fmas are written as fmaf.
+#pragma clang fp contract(off)
+
 // Tuning knobs: non-temporal hint on the output stores (one bit per epilogue kind: 1 none, 2 bias, 4 bias + SiLU,
 // 8 gated residual; measured on the 20-block step, all four on is best: 2.307 ms per block against 2.319-2.324 with
 // the gated-residual or the plain outputs cacheable and 2.332 with none) / on the residual loads of the pipelined
@@ -53,12 +58,17 @@ __device__ __forceinline__ int wrow_to_lds(int n) {
   return blk + 8 * ((r >> 2) & 3) + 4 * (r >> 4) + (r & 3);
 }
 
+// The GEMMs exist for the two 16-bit io dtypes, T = BF16 (also the int8-weight and the fused-state variants) or F16:
+// same loops, the MFMA of the dtype, and the dtype's own conversions in the epilogues (one v_cvt_pk_bf16_f32 per pair
+// for bf16; two conversions and a pack for f16, which has no packed round-to-nearest conversion).
 // acc += W fragment (16 channels x 32 k) . A fragment (32 k x 16 tokens), as an asm statement so that the
 // accumulator is one AGPR quad in and out: given the builtin, whose destination may differ from its addend, the
 // register allocator rotates accumulators through other registers across the loop edge (dozens of copies and
 // their wait states per k-tile in some instances).
+template <typename T>
 __device__ __forceinline__ void mfma_acc(f32x4_t& c, u32x4_t a, u32x4_t b) {
-  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  if constexpr (is_f16<T>) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
 __device__ __forceinline__ uint32_t dequant2(uint32_t q4, int which, float s, float off) {
@@ -128,16 +138,16 @@ struct Taps {
 
 // 8 outputs of one row: accumulator (+bias) -> io dtype, per the epilogue kind (everything except
 // the gated residual, which needs the row's residual and gate and is applied at store time).
-template <int EPI>
+template <int EPI, typename T = BF16>
 __device__ __forceinline__ u32x4_t epi_pack8(const float* a, const float* bv) {
   float v[8];
 #pragma unroll
   for (int r = 0; r < 8; ++r) v[r] = EPI != SANA_EPI_NONE ? a[r] + bv[r] : a[r];
   u32x4_t o;
-  o.x = pack_bf16(v[0], v[1]);
-  o.y = pack_bf16(v[2], v[3]);
-  o.z = pack_bf16(v[4], v[5]);
-  o.w = pack_bf16(v[6], v[7]);
+  o.x = pk16<T>(v[0], v[1]);
+  o.y = pk16<T>(v[2], v[3]);
+  o.z = pk16<T>(v[4], v[5]);
+  o.w = pk16<T>(v[6], v[7]);
   if (EPI == SANA_EPI_BIAS_SILU) {
     // The reference rounds the linear output to bf16 before the activation.  x * rcp(1 + 2^(-x log2 e)),
     // written stage by stage over the eight values (and pinned that way): one value at a time is a
@@ -146,8 +156,8 @@ __device__ __forceinline__ u32x4_t epi_pack8(const float* a, const float* bv) {
     float x[8], t[8];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      x[2 * p] = bf16_lo(o[p]);
-      x[2 * p + 1] = bf16_hi(o[p]);
+      x[2 * p] = lo16<T>(o[p]);
+      x[2 * p + 1] = hi16<T>(o[p]);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -165,45 +175,49 @@ __device__ __forceinline__ u32x4_t epi_pack8(const float* a, const float* bv) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) x[r] *= t[r];
     __builtin_amdgcn_sched_barrier(0);
-    o.x = pack_bf16(x[0], x[1]);
-    o.y = pack_bf16(x[2], x[3]);
-    o.z = pack_bf16(x[4], x[5]);
-    o.w = pack_bf16(x[6], x[7]);
+    o.x = pk16<T>(x[0], x[1]);
+    o.y = pk16<T>(x[2], x[3]);
+    o.z = pk16<T>(x[4], x[5]);
+    o.w = pk16<T>(x[6], x[7]);
   }
   return o;
 }
+template <typename T = BF16>
 __device__ __forceinline__ uint32_t gate_res2(uint32_t y, uint32_t g, uint32_t r) {
-  const float t0 = round_bf16(bf16_lo(g) * bf16_lo(y)), t1 = round_bf16(bf16_hi(g) * bf16_hi(y));
-  return pack_bf16(bf16_lo(r) + t0, bf16_hi(r) + t1);
+  const float t0 = rnd16<T>(lo16<T>(g) * lo16<T>(y)), t1 = rnd16<T>(hi16<T>(g) * hi16<T>(y));
+  return pk16<T>(lo16<T>(r) + t0, hi16<T>(r) + t1);
 }
 // y: 8 linear outputs (already rounded to bf16), g / r: the gate and residual values of the same 8 columns
+template <typename T = BF16>
 __device__ __forceinline__ u32x4_t gate_res8v(u32x4_t y, u32x4_t g, u32x4_t r) {
   u32x4_t o;
-  o.x = gate_res2(y.x, g.x, r.x);
-  o.y = gate_res2(y.y, g.y, r.y);
-  o.z = gate_res2(y.z, g.z, r.z);
-  o.w = gate_res2(y.w, g.w, r.w);
+  o.x = gate_res2<T>(y.x, g.x, r.x);
+  o.y = gate_res2<T>(y.y, g.y, r.y);
+  o.z = gate_res2<T>(y.z, g.z, r.z);
+  o.w = gate_res2<T>(y.w, g.w, r.w);
   return o;
 }
 // the same with the gate values already unpacked (they are the same for every row a lane handles)
+template <typename T = BF16>
 __device__ __forceinline__ u32x4_t gate_res8f(u32x4_t y, const float* g, u32x4_t r) {
   u32x4_t o;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const uint32_t t = pack_bf16(g[2 * e] * bf16_lo(y[e]), g[2 * e + 1] * bf16_hi(y[e]));  // one convert rounds both
-    o[e] = pack_bf16(bf16_lo(r[e]) + bf16_lo(t), bf16_hi(r[e]) + bf16_hi(t));
+    const uint32_t t = pk16<T>(g[2 * e] * lo16<T>(y[e]), g[2 * e + 1] * hi16<T>(y[e]));  // one convert rounds both
+    o[e] = pk16<T>(lo16<T>(r[e]) + lo16<T>(t), hi16<T>(r[e]) + hi16<T>(t));
   }
   return o;
 }
 // y: 8 linear outputs (already rounded to bf16) of row m, columns n..n+7
+template <typename T = BF16>
 __device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m, int n) {
   const u32x4_t g = *reinterpret_cast<const u32x4_t*>(e.gate + (int64_t)(m / e.rows_per_gate) * e.gate_stride + n);
   const u32x4_t r = *reinterpret_cast<const u32x4_t*>(e.res + (int64_t)m * e.ldr + n);
   u32x4_t o;
-  o.x = gate_res2(y.x, g.x, r.x);
-  o.y = gate_res2(y.y, g.y, r.y);
-  o.z = gate_res2(y.z, g.z, r.z);
-  o.w = gate_res2(y.w, g.w, r.w);
+  o.x = gate_res2<T>(y.x, g.x, r.x);
+  o.y = gate_res2<T>(y.y, g.y, r.y);
+  o.z = gate_res2<T>(y.z, g.z, r.z);
+  o.w = gate_res2<T>(y.w, g.w, r.w);
   return o;
 }
 
@@ -215,7 +229,7 @@ __device__ __forceinline__ u32x4_t gate_res8(u32x4_t y, const EpiArgs& e, int m,
 // (three register sets in rotation), because with so little math per k-tile the chain is otherwise one global
 // load latency per k-tile.  Every output sums its k products in the same order in all of these kernels, so
 // they agree bit for bit.
-template <bool W8, int EPI, int TT = 4, int TC = 4>
+template <bool W8, int EPI, int TT = 4, int TC = 4, typename T = BF16>
 __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const uint16_t* __restrict__ A, const void* __restrict__ Wv,
                                                    const float* __restrict__ scale, const EpiArgs ep,
                                                    uint16_t* __restrict__ C,
@@ -361,8 +375,7 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
       for (int i = 0; i < TC; ++i)
 #pragma unroll
         for (int j = 0; j < TT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw[i]),
-                                                             __builtin_bit_cast(bf16x8_t, fa[j]), acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_32x32x16<T>(fw[i], fa[j], acc[i][j]);
     }
     store_tile((d + 1) % DEPTH, cur ^ 1);
     __syncthreads();
@@ -378,7 +391,7 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
     float bv[16];
     if (HAS_BIAS) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? bf16_bits_to_f32(ep.bias[n + r]) : 0.f;
+      for (int r = 0; r < 16; ++r) bv[r] = (ep.bias && n + r < N) ? lo16<T>(ep.bias[n + r]) : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < TT; ++j) {
@@ -391,8 +404,8 @@ __global__ __launch_bounds__(256, (TT * TC <= 4 ? 2 : 1)) void gemm_kernel(const
           float a8[8];
 #pragma unroll
           for (int r = 0; r < 8; ++r) a8[r] = acc[i][j][8 * half + r];
-          u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a8, bv + 8 * half);
-          if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n + 8 * half);
+          u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI, T>(a8, bv + 8 * half);
+          if (EPI == SANA_EPI_GATE_RES) o = gate_res8<T>(o, ep, m, n + 8 * half);
           *reinterpret_cast<u32x4_t*>(cp + 8 * half) = o;
         }
       }
@@ -511,14 +524,14 @@ __device__ __forceinline__ void state_tile16(f32x4_t (&acc)[8][8], const u32x4_t
 // Epilogue of the pipelined kernels.  acc[i][j][r] (MFMA 16x16 tiles: i = channel tile of the wave, j = token tile):
 // token m0 + wt*128 + 16*j + lane%16, channel n0 + wc*32*NI + 8*NI*(lane/16) + 4*i + r.  bpk: the lane's 8*NI bias
 // values, packed (the caller requests them ahead of its last k-tile so that their latency hides behind its MFMAs).
-template <int EPI, int NI, bool SPLIT>
+template <int EPI, int NI, bool SPLIT, typename T = BF16>
 __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u32x4_t (&bpk)[NI], unsigned char* smem,
                                               const EpiArgs& ep, uint16_t* __restrict__ C, int M, int N, int64_t ldc,
                                               int m0, int n0) {
   constexpr int NWT = 2 * NI;
   constexpr bool HAS_BIAS = EPI != SANA_EPI_NONE;
   if constexpr (EPI == SANA_EPI_QKV_STATE) {
-    static_assert(NI == 4 && !SPLIT, "the fused qkv projection runs 256-wide tiles, unsplit");
+    static_assert(NI == 4 && !SPLIT && !is_f16<T>, "the fused qkv projection runs 256-wide bf16 tiles, unsplit");
     if (n0 >= ep.q_pad) {  // uniform per workgroup: a k / v tile
       state_tile16(acc, bpk, smem, ep, m0, n0);
       return;
@@ -613,8 +626,8 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
     for (int c = 0; c < NI; ++c)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        bv[c][2 * e] = bf16_lo(bpk[c][e]);
-        bv[c][2 * e + 1] = bf16_hi(bpk[c][e]);
+        bv[c][2 * e] = lo16<T>(bpk[c][e]);
+        bv[c][2 * e + 1] = hi16<T>(bpk[c][e]);
       }
   }
   // Software-pipelined over the four groups of 32 tokens: step s of phase j converts piece s of group j
@@ -628,7 +641,7 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
     float a8[8];
 #pragma unroll
     for (int r = 0; r < 4; ++r) a8[r] = acc[2 * c][j][r], a8[4 + r] = acc[2 * c + 1][j][r];
-    const u32x4_t o = epi_pack8<(EPI == SANA_EPI_GATE_RES || EPI == SANA_EPI_QKV_STATE) ? SANA_EPI_BIAS : EPI>(a8, bv[c]);
+    const u32x4_t o = epi_pack8<(EPI == SANA_EPI_GATE_RES || EPI == SANA_EPI_QKV_STATE) ? SANA_EPI_BIAS : EPI, T>(a8, bv[c]);
     const int chunk = NI * fg + c;
     *reinterpret_cast<u32x4_t*>(stg + tok * 256 + ((chunk ^ (tok & 15)) << 4)) = o;
   };
@@ -656,8 +669,8 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
           const u32x4_t gate = *reinterpret_cast<const u32x4_t*>(ep.gate + (int64_t)g_first * ep.gate_stride + o_n);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            gf[2 * e] = bf16_lo(gate[e]);
-            gf[2 * e + 1] = bf16_hi(gate[e]);
+            gf[2 * e] = lo16<T>(gate[e]);
+            gf[2 * e + 1] = hi16<T>(gate[e]);
           }
         }
       }
@@ -671,7 +684,7 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
       if (j < 4 && st < 2 * NI) convert_piece(j, st);
       __builtin_amdgcn_sched_barrier(0);
       if (js >= 0) {
-        if (EPI == SANA_EPI_GATE_RES) o = gate_res8f(o, gf, res[js][st]);
+        if (EPI == SANA_EPI_GATE_RES) o = gate_res8f<T>(o, gf, res[js][st]);
         __builtin_amdgcn_raw_buffer_store_b128(o, rsrc_c, c_off0 + (8 * js + st) * c_step, 0, ((SANA_GEMM_NT_STORE >> EPI) & 1) ? kBufferNt : 0);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -686,7 +699,7 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
               u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, r_off0 + (8 * js + it) * r_step, 0, 0));
           const u32x4_t g2 = *reinterpret_cast<const u32x4_t*>(
               ep.gate + (int64_t)(m / ep.rows_per_gate) * ep.gate_stride + o_n);
-          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v(y, g2, r), rsrc_c, c_off0 + (8 * js + it) * c_step, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(gate_res8v<T>(y, g2, r), rsrc_c, c_off0 + (8 * js + it) * c_step, 0, 0);
         }
       }
     }
@@ -721,7 +734,7 @@ __device__ __forceinline__ void finish_tile16(f32x4_t (&acc)[2 * NI][8], const u
 // k-tiles and stores the raw fp32 accumulators to C taken as float [gridDim.y][M][N]; splitk_epilogue_kernel
 // adds the ranges up in order and applies the epilogue.
 // TAPS: 0 = plain A operand, 1 = tap-concatenated A operand, 2 = the same with per-row-block zero_last flags.
-template <bool W8, int EPI, int NI, int TAPS = 0, bool SPLIT = false>
+template <bool W8, int EPI, int NI, int TAPS = 0, bool SPLIT = false, typename T = BF16>
 __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__ A_, const void* __restrict__ Wv_,
                                                     const float* __restrict__ scale, const EpiArgs ep,
                                                     uint16_t* __restrict__ C, int M, int N, int K_, int64_t lda,
@@ -892,7 +905,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   // changes, not both.  Less switching on the operand buses: the power-limited clock settles ~1 % higher.
   auto mfma = [&](int buf, int t) {  // t < 8 * NWT
     const int i = t >> 3, j = (i & 1) ? 7 - (t & 7) : (t & 7);
-    mfma_acc(acc[i][j], fw[buf][i], fa[buf][j]);
+    mfma_acc<T>(acc[i][j], fw[buf][i], fa[buf][j]);
   };
 
   const int KT = (K + BK - 1) / BK;
@@ -936,6 +949,15 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
   static_assert(W8 || (QSTRIDE >= 2 && 1 + (NQ - 1) * QSTRIDE < BAR - 2 && RSTR >= 1 && BAR + 1 + (NFR - 1) * RSTR < TS),
                 "staging does not fit in front of the barrier");
   static_assert(!W8 || (4 * 7 + 1 < BAR && PSTR >= 1), "staging does not fit in front of the barrier");
+  // The MFMAs below are asm statements: the compiler neither knows that they read the accumulators through the
+  // matrix pipe nor places the wait states such a read needs behind the VALU writes that zeroed them.  Pin the
+  // order by hand: every accumulator passes through an empty asm statement (its zeroing is complete, in program
+  // order, in front of it), then eight wait states, then the first MFMA -- whatever the compiler puts in between.
+#pragma unroll
+  for (int i = 0; i < NWT; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+  asm volatile("s_nop 7" ::: "memory");
   for (int kt = 0; kt < KT - 1; ++kt) {
     const int cur = kt & 1;
     const unsigned char* st = smem + cur * 2 * TILE_BYTES;
@@ -1014,7 +1036,7 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) {
           const int j = (i & 1) ? 7 - jj : jj;
-          mfma_acc(acc[i][j], w8[i], a8[j]);
+          mfma_acc<T>(acc[i][j], w8[i], a8[j]);
         }
     }
     // the MFMAs are asm statements, so the compiler does not know that their results are in flight: wait out the
@@ -1022,12 +1044,12 @@ __global__ __launch_bounds__(256) void gemm4_kernel(const uint16_t* __restrict__
     asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
   }
 
-  finish_tile16<EPI, NI, SPLIT>(acc, bpk, smem, ep, C, M, N, ldc, m0, n0);
+  finish_tile16<EPI, NI, SPLIT, T>(acc, bpk, smem, ep, C, M, N, ldc, m0, n0);
 }
 
 // Second half of a split-k GEMM: partial[S][M][N] (fp32) -> C = epilogue(sum over the S k-ranges, added in
 // order).  One thread per row and 8 channels; the same epilogue functions as the fused path.
-template <int EPI>
+template <int EPI, typename T = BF16>
 __global__ __launch_bounds__(256) void splitk_epilogue_kernel(const float* __restrict__ partial, int S,
                                                                const EpiArgs ep, uint16_t* __restrict__ C, int M, int N,
                                                                int64_t ldc) {
@@ -1048,12 +1070,12 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(const float* __res
     const u32x4_t b = *reinterpret_cast<const u32x4_t*>(ep.bias + n);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      bv[2 * e] = bf16_lo(b[e]);
-      bv[2 * e + 1] = bf16_hi(b[e]);
+      bv[2 * e] = lo16<T>(b[e]);
+      bv[2 * e + 1] = hi16<T>(b[e]);
     }
   }
-  u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI>(a, bv);
-  if (EPI == SANA_EPI_GATE_RES) o = gate_res8(o, ep, m, n);
+  u32x4_t o = epi_pack8<EPI == SANA_EPI_GATE_RES ? SANA_EPI_BIAS : EPI, T>(a, bv);
+  if (EPI == SANA_EPI_GATE_RES) o = gate_res8<T>(o, ep, m, n);
   *reinterpret_cast<u32x4_t*>(C + (int64_t)m * ldc + n) = o;
 }
 
@@ -1140,7 +1162,7 @@ GemmPlan plan_gemm(int M, int N, int K, bool w8) {
 }
 size_t split_bytes(const GemmPlan& pl, int M, int N) { return pl.S > 1 ? (size_t)pl.S * M * N * sizeof(float) : 0; }
 
-template <bool W8, int NI>
+template <bool W8, int NI, typename T = BF16>
 int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N, int K,
             int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr,
             float* ws = nullptr, size_t ws_bytes = 0) {
@@ -1152,14 +1174,14 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
       const GemmPlan pl = plan_gemm(M, N, K, W8);
       if (pl.S > 1 && ws_bytes >= split_bytes(pl, M, N)) {
         const Taps split = {0, 0, 0, pl.tiles, pl.rem, nullptr};
-        hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, 0, true>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
+        hipLaunchKernelGGL((gemm4_kernel<W8, SANA_EPI_NONE, NI, 0, true, T>), dim3(grid.x, (unsigned)pl.S), block, 0, s,
                            a, W, scale, ep, reinterpret_cast<uint16_t*>(ws), M, N, K, lda, ldw, ldc, tiles_t, tiles_c,
                            split);
         if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
         const int64_t threads = (int64_t)M * (N / 8);
         dim3 egrid((unsigned)((threads + 255) / 256));
 #define SANA_SPLIT_EPI(EPI) \
-  hipLaunchKernelGGL((splitk_epilogue_kernel<EPI>), egrid, block, 0, s, ws, pl.S, ep, c, M, N, ldc)
+  hipLaunchKernelGGL((splitk_epilogue_kernel<EPI, T>), egrid, block, 0, s, ws, pl.S, ep, c, M, N, ldc)
         switch (epilogue) {
           case SANA_EPI_NONE: SANA_SPLIT_EPI(SANA_EPI_NONE); break;
           case SANA_EPI_BIAS: SANA_SPLIT_EPI(SANA_EPI_BIAS); break;
@@ -1172,7 +1194,7 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
       }
     }
     if (taps) {  // only the bf16 gated-residual instance exists with taps
-      if (W8 || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
+      if (W8 || is_f16<T> || epilogue != SANA_EPI_GATE_RES) return SANA_ERR_ARG;
       if (taps->zero_last)
         hipLaunchKernelGGL((gemm4_kernel<false, SANA_EPI_GATE_RES, NI, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K,
                            lda, ldw, ldc, tiles_t, tiles_c, *taps);
@@ -1185,7 +1207,7 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
     if (taps) return SANA_ERR_ARG;
   }
 #define SANA_LAUNCH4(EPI)                                                                                         \
-  hipLaunchKernelGGL((gemm4_kernel<W8, EPI, NI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+  hipLaunchKernelGGL((gemm4_kernel<W8, EPI, NI, 0, false, T>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
                      tiles_t, tiles_c, none)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH4(SANA_EPI_NONE); break;
@@ -1198,13 +1220,13 @@ int launch4(const uint16_t* a, const void* W, const float* scale, const EpiArgs&
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
-template <bool W8>
+template <bool W8, typename T = BF16>
 int launch_small(const uint16_t* a, const void* W, const float* scale, const EpiArgs& ep, uint16_t* c, int M, int N,
                  int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s) {
   const int tiles_t = (M + 127) / 128, tiles_c = (N + 127) / 128;
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
 #define SANA_LAUNCH_S(EPI)                                                                                          \
-  hipLaunchKernelGGL((gemm_kernel<W8, EPI, 2, 2>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+  hipLaunchKernelGGL((gemm_kernel<W8, EPI, 2, 2, T>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
                      tiles_t, tiles_c)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH_S(SANA_EPI_NONE); break;
@@ -1217,7 +1239,7 @@ int launch_small(const uint16_t* a, const void* W, const float* scale, const Epi
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
-template <bool W8>
+template <bool W8, typename T = BF16>
 int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, void* C, int M, int N, int K,
            int64_t lda, int64_t ldw, int64_t ldc, int epilogue, hipStream_t s, const Taps* taps = nullptr,
            void* workspace = nullptr, size_t workspace_bytes = 0) {
@@ -1226,7 +1248,7 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
   const uint16_t* a = static_cast<const uint16_t*>(A);
   uint16_t* c = static_cast<uint16_t*>(C);
   if (!taps && plan_gemm(M, N, K, W8).small)
-    return launch_small<W8>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
+    return launch_small<W8, T>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s);
   if (K % 32 == 0 && K >= 64) {  // the pipelined kernel; the generic one takes any K % 8 == 0 (int8: K % 16 == 0)
     float* ws = aligned16(workspace) ? static_cast<float*>(workspace) : nullptr;
     // Mixed channel tiling: the first n_wide channels in 256-wide tiles, the rest in 192-wide ones, as two launches
@@ -1236,13 +1258,13 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
     if (!taps && plan_gemm(M, N, K, W8).S == 1) {
       const int n_wide = mixed_split(M, N);
       if (n_wide > 0) {
-        const int rc = launch4<W8, 4>(a, W, scale, ep, c, M, n_wide, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
+        const int rc = launch4<W8, 4, T>(a, W, scale, ep, c, M, n_wide, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
         if (rc != SANA_OK) return rc;
         EpiArgs ep2 = ep;
         if (ep2.bias) ep2.bias += n_wide;
         if (ep2.gate) ep2.gate += n_wide;
         if (ep2.res) ep2.res += n_wide;
-        return launch4<W8, 3>(a, static_cast<const char*>(W) + (int64_t)n_wide * ldw * (W8 ? 1 : 2),
+        return launch4<W8, 3, T>(a, static_cast<const char*>(W) + (int64_t)n_wide * ldw * (W8 ? 1 : 2),
                               scale ? scale + n_wide : nullptr, ep2, c + n_wide, M, N - n_wide, K, lda, ldw, ldc, epilogue,
                               s, nullptr, nullptr, 0);
       }
@@ -1253,17 +1275,17 @@ int launch(const void* A, const void* W, const float* scale, const EpiArgs& ep, 
     {
       const int64_t t128 = tiles_t * ((N + 127) / 128), t192 = tiles_t * ((N + 191) / 192);
       if (!taps && t128 <= compute_units() && t192 < compute_units() * 4 / 5 && plan_gemm(M, N, K, W8).S == 1)
-        return launch4<W8, 2>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
+        return launch4<W8, 2, T>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, nullptr, nullptr, 0);
     }
     return pick_ni(M, N) == 3
-               ? launch4<W8, 3>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes)
-               : launch4<W8, 4>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes);
+               ? launch4<W8, 3, T>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes)
+               : launch4<W8, 4, T>(a, W, scale, ep, c, M, N, K, lda, ldw, ldc, epilogue, s, taps, ws, workspace_bytes);
   }
   if (taps) return SANA_ERR_SHAPE;
   const int tiles_c = (N + BC - 1) / BC;
   dim3 grid((unsigned)(tiles_t * tiles_c)), block(256);
 #define SANA_LAUNCH(EPI)                                                                                        \
-  hipLaunchKernelGGL((gemm_kernel<W8, EPI>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
+  hipLaunchKernelGGL((gemm_kernel<W8, EPI, 4, 4, T>), grid, block, 0, s, a, W, scale, ep, c, M, N, K, lda, ldw, ldc, \
                      (int)tiles_t, tiles_c)
   switch (epilogue) {
     case SANA_EPI_NONE: SANA_LAUNCH(SANA_EPI_NONE); break;
@@ -1365,6 +1387,16 @@ SANA_API int sana_hip_gemm_bf16(const void* A, const void* W, const void* bias, 
                        static_cast<hipStream_t>(stream), nullptr, workspace, workspace_bytes);
 }
 
+SANA_API int sana_hip_gemm_f16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,
+                               int64_t lda, int64_t ldw, int64_t ldc, int epilogue, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  if (epilogue == SANA_EPI_GATE_RES) return SANA_ERR_ARG;
+  const int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, epilogue, 8, 8);
+  if (rc != SANA_OK) return rc;
+  return launch<false, F16>(A, W, nullptr, plain_epi(bias), C, M, N, K, lda, ldw, ldc, epilogue,
+                            static_cast<hipStream_t>(stream), nullptr, workspace, workspace_bytes);
+}
+
 SANA_API int sana_hip_gemm_w8a16(const void* A, const int8_t* Wq, const float* scale, const void* bias, void* C,
                                  int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue,
                                  void* workspace, size_t workspace_bytes, void* stream) {
@@ -1392,6 +1424,21 @@ SANA_API int sana_hip_gemm_gate_residual(const void* A, const void* W, const flo
                            workspace_bytes)
             : launch<false>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, s, nullptr, workspace,
                             workspace_bytes);
+}
+
+SANA_API int sana_hip_gemm_gate_residual_f16(const void* A, const void* W, const void* bias, const void* gate,
+                                             const void* residual, void* C, int M, int N, int K, int64_t lda,
+                                             int64_t ldw, int64_t ldr, int64_t ldc, int rows_per_gate,
+                                             int64_t gate_stride, void* workspace, size_t workspace_bytes,
+                                             void* stream) {
+  int rc = check_common(A, W, bias, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES, 8, 8);
+  if (rc != SANA_OK) return rc;
+  rc = check_gate_res(gate, residual, M, N, ldr, rows_per_gate, gate_stride);
+  if (rc != SANA_OK) return rc;
+  const EpiArgs e = {static_cast<const uint16_t*>(bias), static_cast<const uint16_t*>(gate),
+                     static_cast<const uint16_t*>(residual), ldr, gate_stride, rows_per_gate, nullptr, 0, 0, 0, 0};
+  return launch<false, F16>(A, W, nullptr, e, C, M, N, K, lda, ldw, ldc, SANA_EPI_GATE_RES,
+                            static_cast<hipStream_t>(stream), nullptr, workspace, workspace_bytes);
 }
 
 SANA_API int sana_hip_tconv_residual(const void* X, const void* W, void* out, int M, int C, int taps,

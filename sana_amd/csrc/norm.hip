@@ -13,6 +13,11 @@
 // reproduced in registers.
 #include "common.h"
 
+// No implicit fused multiply-adds in this file: the epilogues reproduce the stock op chain's roundings (product
+// rounded to the io dtype, THEN the sum), and for fp16 -- which has native arithmetic -- the compiler would otherwise
+// contract "round(g * y) + r" into one v_fma_f16 and drop the product's rounding.  Wanted fmas are written as fmaf.
+#pragma clang fp contract(off)
+
 #ifndef SANA_LN_NT_LOAD
 #define SANA_LN_NT_LOAD 0
 #endif
@@ -31,7 +36,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // NCH: 16-byte chunks per lane (C <= 512 * NCH).  ADD: the row is x + y (rounded to bf16, as the stock add
 // stores it) and is written to `sum` as well: the residual update in front of the norm, in the same pass.
-template <int NCH, bool ADD>
+template <int NCH, bool ADD, typename T>
 __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __restrict__ x,
                                                           const uint16_t* __restrict__ y,
                                                           const uint16_t* __restrict__ scale,
@@ -62,7 +67,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
         const u32x4_t b = load_stream<SANA_LN_NT_LOAD != 0>(reinterpret_cast<const u32x4_t*>(yr + 8 * ch));
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          raw[i][e] = pack_bf16(bf16_lo(raw[i][e]) + bf16_lo(b[e]), bf16_hi(raw[i][e]) + bf16_hi(b[e]));
+          raw[i][e] = pk16<T>(lo16<T>(raw[i][e]) + lo16<T>(b[e]), hi16<T>(raw[i][e]) + hi16<T>(b[e]));
         store_stream<SANA_LN_NT_STORE != 0>(raw[i], reinterpret_cast<u32x4_t*>(sr + 8 * ch));
       }
     }
@@ -71,7 +76,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) s += bf16_lo(raw[i][e]) + bf16_hi(raw[i][e]);
+    for (int e = 0; e < 4; ++e) s += lo16<T>(raw[i][e]) + hi16<T>(raw[i][e]);
   const float mean = wave_sum(s) / (float)C;
   float v = 0.f;
 #pragma unroll
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
     if (lane + 64 * i < nchunks) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float a = bf16_lo(raw[i][e]) - mean, b = bf16_hi(raw[i][e]) - mean;
+        const float a = lo16<T>(raw[i][e]) - mean, b = hi16<T>(raw[i][e]) - mean;
         v = fmaf(a, a, v);
         v = fmaf(b, b, v);
       }
@@ -97,10 +102,10 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
       u32x4_t o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const uint32_t ln = pack_bf16((bf16_lo(raw[i][e]) - mean) * rstd, (bf16_hi(raw[i][e]) - mean) * rstd);
-        const uint32_t s1 = pack_bf16(1.0f + bf16_lo(sc[e]), 1.0f + bf16_hi(sc[e]));
-        const uint32_t t = pack_bf16(bf16_lo(ln) * bf16_lo(s1), bf16_hi(ln) * bf16_hi(s1));
-        o[e] = pack_bf16(bf16_lo(t) + bf16_lo(sh[e]), bf16_hi(t) + bf16_hi(sh[e]));
+        const uint32_t ln = pk16<T>((lo16<T>(raw[i][e]) - mean) * rstd, (hi16<T>(raw[i][e]) - mean) * rstd);
+        const uint32_t s1 = pk16<T>(1.0f + lo16<T>(sc[e]), 1.0f + hi16<T>(sc[e]));
+        const uint32_t t = pk16<T>(lo16<T>(ln) * lo16<T>(s1), hi16<T>(ln) * hi16<T>(s1));
+        o[e] = pk16<T>(lo16<T>(t) + lo16<T>(sh[e]), hi16<T>(t) + hi16<T>(sh[e]));
       }
       store_stream<SANA_LN_NT_STORE != 0>(o, reinterpret_cast<u32x4_t*>(orow + 8 * ch));
     }
@@ -110,6 +115,7 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const uint16_t* __rest
 // out = res + gate[row / rows_per_gate] * y with the two roundings of the stock op pair (product, then sum):
 // the gated residual update behind a module whose last op is not one of this library's GEMMs.  One thread per
 // 8 channels; three streams (y, res, out), HBM bound.
+template <typename T>
 __global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __restrict__ y,
                                                             const uint16_t* __restrict__ gate,
                                                             const uint16_t* __restrict__ res,
@@ -127,8 +133,8 @@ __global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __re
   u32x4_t o;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const uint32_t t = pack_bf16(bf16_lo(gv[e]) * bf16_lo(yv[e]), bf16_hi(gv[e]) * bf16_hi(yv[e]));
-    o[e] = pack_bf16(bf16_lo(rv[e]) + bf16_lo(t), bf16_hi(rv[e]) + bf16_hi(t));
+    const uint32_t t = pk16<T>(lo16<T>(gv[e]) * lo16<T>(yv[e]), hi16<T>(gv[e]) * hi16<T>(yv[e]));
+    o[e] = pk16<T>(lo16<T>(rv[e]) + lo16<T>(t), hi16<T>(rv[e]) + hi16<T>(t));
   }
   store_stream<SANA_LN_NT_STORE != 0>(o, reinterpret_cast<u32x4_t*>(out + m * ldo + n));
 }
@@ -144,7 +150,7 @@ static int ln_impl(const void* x, const void* y, const void* scale, const void* 
                    float eps, int io_dtype, void* stream) {
   if (!x || !scale || !shift || !out || M <= 0 || C <= 0 || rows_per_mod <= 0) return SANA_ERR_ARG;
   if (ADD && (!y || !sum)) return SANA_ERR_ARG;
-  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
   if (C % 8 || C > 8192) return SANA_ERR_SHAPE;
   if (ldx < C || ldo < C || mod_stride < 0 || (ADD && (ldy < C || lds < C))) return SANA_ERR_ARG;
   if (ldx % 8 || ldo % 8 || mod_stride % 8 || !aligned16(x) || !aligned16(out) || !aligned16(scale) ||
@@ -161,9 +167,15 @@ static int ln_impl(const void* x, const void* y, const void* scale, const void* 
   uint16_t* sp = static_cast<uint16_t*>(sum);
   uint16_t* op = static_cast<uint16_t*>(out);
   const int nch = (C / 8 + 63) / 64;
-#define SANA_LN(NCH)                                                                                              \
-  hipLaunchKernelGGL((ln_modulate_kernel<NCH, ADD>), grid, block, 0, s, xp, yp, sc, sh, sp, op, M, C, ldx, ldy, lds, \
-                     ldo, rows_per_mod, mod_stride, eps)
+#define SANA_LN(NCH)                                                                                          \
+  do {                                                                                                        \
+    if (io_dtype == SANA_DT_F16)                                                                              \
+      hipLaunchKernelGGL((ln_modulate_kernel<NCH, ADD, F16>), grid, block, 0, s, xp, yp, sc, sh, sp, op, M, C, \
+                         ldx, ldy, lds, ldo, rows_per_mod, mod_stride, eps);                                  \
+    else                                                                                                      \
+      hipLaunchKernelGGL((ln_modulate_kernel<NCH, ADD, BF16>), grid, block, 0, s, xp, yp, sc, sh, sp, op, M, C, \
+                         ldx, ldy, lds, ldo, rows_per_mod, mod_stride, eps);                                  \
+  } while (0)
   if (nch <= 2) SANA_LN(2);
   else if (nch <= 3) SANA_LN(3);
   else if (nch <= 5) SANA_LN(5);
@@ -192,7 +204,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_gate_residual(
     const void* y, const void* gate, const void* residual, void* out, int64_t M, int C, int64_t ldy, int64_t ldr,
     int64_t ldo, int rows_per_gate, int64_t gate_stride, int io_dtype, void* stream) {
   if (!y || !gate || !residual || !out || M <= 0 || C <= 0 || rows_per_gate <= 0) return SANA_ERR_ARG;
-  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  if (io_dtype != SANA_DT_BF16 && io_dtype != SANA_DT_F16) return SANA_ERR_DTYPE;
   if (C % 8) return SANA_ERR_SHAPE;
   if (ldy < C || ldr < C || ldo < C || gate_stride < 0) return SANA_ERR_ARG;
   if (ldy % 8 || ldr % 8 || ldo % 8 || gate_stride % 8 || !aligned16(y) || !aligned16(gate) || !aligned16(residual) ||
@@ -200,9 +212,15 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_gate_residual(
     return SANA_ERR_ALIGN;
   const int64_t threads = M * (C / 8);
   if ((threads + 255) / 256 > 0x7fffffff) return SANA_ERR_SHAPE;
-  hipLaunchKernelGGL(gate_residual_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(y),
-                     static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(residual),
-                     static_cast<uint16_t*>(out), M, C, ldy, ldr, ldo, rows_per_gate, gate_stride);
+  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (io_dtype == SANA_DT_F16)
+    hipLaunchKernelGGL(gate_residual_kernel<F16>, grid, block, 0, s, static_cast<const uint16_t*>(y),
+                       static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(residual),
+                       static_cast<uint16_t*>(out), M, C, ldy, ldr, ldo, rows_per_gate, gate_stride);
+  else
+    hipLaunchKernelGGL(gate_residual_kernel<BF16>, grid, block, 0, s, static_cast<const uint16_t*>(y),
+                       static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(residual),
+                       static_cast<uint16_t*>(out), M, C, ldy, ldr, ldo, rows_per_gate, gate_stride);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }

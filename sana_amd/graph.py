@@ -25,16 +25,24 @@ class GraphedCall:
     def __init__(self, fn: Callable[..., torch.Tensor], example: Sequence[torch.Tensor], warmup: int = 2):
         if not example or not all(torch.is_tensor(t) and t.is_cuda for t in example):
             raise ValueError("GraphedCall needs device tensors as example arguments")
+        if warmup < 1:
+            raise ValueError("GraphedCall needs at least one warm-up call: lazy allocations, host-to-device copies of "
+                             "derived tables and the library's scratch buffer must exist before the capture starts")
         self._inputs = list(example)   # the example tensors ARE the captured input buffers
         with torch.no_grad():
-            side = torch.cuda.Stream(device=example[0].device)
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):          # warm-up off the capturing stream: lazy allocations, table caches
+            # One stream of this object's own for the warm-up AND the capture.  The library keeps its scratch buffer
+            # per (device, stream): warming up on the stream that is captured afterwards creates that buffer eagerly,
+            # in the ordinary memory pool, before the capture begins (allocated during the capture it would belong to
+            # this graph's private pool while other graphs used it), and a stream per object gives every graph a
+            # scratch buffer of its own, so two graphs replayed on different streams do not share one.
+            self._stream = torch.cuda.Stream(device=example[0].device)
+            self._stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(self._stream):
                 for _ in range(warmup):
                     fn(*self._inputs)
-            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.current_stream().wait_stream(self._stream)
             self._graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self._graph):
+            with torch.cuda.graph(self._graph, stream=self._stream):
                 self._output = fn(*self._inputs)
 
     def __call__(self, *tensors: torch.Tensor) -> torch.Tensor:

@@ -12,10 +12,10 @@ Forward only (inference).  The modules run on a GPU through ``libsana_hip.so``;
 there is no CPU path: a configuration the kernels do not cover raises
 ``NotImplementedError`` at construction or call time.  Cross-attention is stock
 PyTorch-ROCm ops by design.  A few options keep the HIP attention / depthwise
-kernels but take a stock op for one stage (fp16 / fp32 models: library GEMM for the
+kernels but take a stock op for one stage (fp32 models: library GEMM for the
 linears; the real-valued pre-ReLU rotary embedding of ``LiteLA``; the temporal
 conv with a frame mask, C % 64 != 0 or a dtype other than bf16; the unfused
-LayerNorm / modulate / gate / residual seams outside bf16 inference).  Each of
+LayerNorm / modulate / gate / residual seams outside bf16 / fp16 inference).  Each of
 those logs one line per process and reason on the ``sana_amd`` logger
 (:func:`stock_path`), so nothing leaves the fast path silently.
 """
@@ -48,6 +48,27 @@ def stock_path(where: str, why: str) -> None:
 
 
 
+def _version(t: torch.Tensor):
+    """The tensor's in-place version counter, or None for a tensor created under ``torch.inference_mode()``
+    (such tensors do not track one and reading it raises; an in-place edit of one is then not noticed by the
+    caches of derived data below, which key on it)."""
+    return None if t.is_inference() else t._version
+
+
+def _sources_unchanged(entry, tensors) -> bool:
+    """``entry`` = (source tensors, their versions) of a derived-data cache: true when ``tensors`` are the very
+    same objects (not merely tensors at the same address: the allocator hands a freed address to the next
+    parameter) with unchanged version counters."""
+    if entry is None or len(entry[0]) != len(tensors):
+        return False
+    return all(a is b for a, b in zip(entry[0], tensors)) and entry[1] == tuple(
+        None if t is None else _version(t) for t in tensors)
+
+
+def _source_entry(tensors):
+    return (tuple(tensors), tuple(None if t is None else _version(t) for t in tensors))
+
+
 def _no_grad_only(*tensors):
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise SanaHipError("the HIP path is forward-only: call it under torch.no_grad() / inference_mode()")
@@ -57,12 +78,12 @@ def _no_grad_only(*tensors):
 
 
 class HipLinear(nn.Linear):
-    """``nn.Linear`` whose bf16 GPU forward is the hand-written MFMA GEMM.
+    """``nn.Linear`` whose bf16 / fp16 GPU forward is the hand-written MFMA GEMM.
 
     Keys ``weight`` / ``bias`` as in ``nn.Linear``.  After :meth:`quantize_w8_`
     the bf16 weight is dropped and replaced by ``weight_q`` (int8 [out, in]) and
     ``weight_scale`` (fp32 [out]); the forward then runs the W8A16 GEMM.
-    Other dtypes (fp16 / fp32 models) use the stock library GEMM.
+    fp32 models use the stock library GEMM.
     """
 
     def quantize_w8_(self) -> "HipLinear":
@@ -89,23 +110,25 @@ def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None,
     lead = x.shape[:-1]
     K = x.shape[-1]
     if gate is not None:
-        if x.dtype == torch.bfloat16 and gate.dtype == x.dtype and residual.dtype == x.dtype and x.is_cuda \
-                and x.dim() == 3 and epilogue is None:
+        if x.dtype in ops.IO16 and gate.dtype == x.dtype and residual.dtype == x.dtype and x.is_cuda \
+                and x.dim() == 3 and epilogue is None and (weight_q is None or x.dtype == torch.bfloat16):
             w = weight_q if weight_q is not None else weight
             return ops.gemm_gate_residual(x, w, bias, gate, residual, weight_scale if weight_q is not None else None)
-        stock_path("gated residual behind a linear", f"the fused epilogue needs bf16 [B, N, C] device input, gate and "
+        stock_path("gated residual behind a linear", f"the fused epilogue needs bf16 / fp16 [B, N, C] device input, gate and "
                    f"residual and no activation; got x {x.dtype} {x.dim()}-d, gate {gate.dtype}, residual "
                    f"{residual.dtype}, epilogue {epilogue!r}")
         return residual + gate * hip_linear(x, weight, bias, epilogue, weight_q, weight_scale)
-    if x.dtype == torch.bfloat16 and x.is_cuda:
+    if x.dtype in ops.IO16 and x.is_cuda and (weight_q is not None or weight.dtype == x.dtype):
         x2 = x.reshape(-1, K)
         if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
             x2 = x2.contiguous()
         epi = {None: "bias" if bias is not None else None, "silu": "bias_silu"}[epilogue]
         if epilogue == "silu" and bias is None:
             bias = torch.zeros(weight_q.shape[0] if weight_q is not None else weight.shape[0],
-                               dtype=torch.bfloat16, device=x.device)
+                               dtype=x.dtype, device=x.device)
         if weight_q is not None:
+            if x.dtype != torch.bfloat16:
+                raise SanaHipError("W8A16 needs bf16 activations")
             y = ops.gemm_w8a16(x2, weight_q, weight_scale, bias, epi, out=out)
         else:
             y = ops.gemm_bf16(x2, weight.reshape(weight.shape[0], -1), bias, epi, out=out)
@@ -114,8 +137,9 @@ def hip_linear(x, weight, bias, epilogue=None, weight_q=None, weight_scale=None,
         raise SanaHipError("the HIP path needs device tensors (no CPU path exists)")
     if weight_q is not None:
         raise SanaHipError("W8A16 needs bf16 activations")
-    # fp16 / fp32 models: plain library GEMM (hipBLASLt), activation as a stock op
-    stock_path("linear / 1x1 conv", f"the hand-written GEMM is bf16 only, input is {x.dtype} (library GEMM instead)")
+    # fp32 models (or activations and weights of different dtypes): plain library GEMM, activation as a stock op
+    stock_path("linear / 1x1 conv", f"the hand-written GEMM takes bf16 or fp16 operands of one dtype, got input {x.dtype} "
+               f"and weight {weight.dtype} (library GEMM instead)")
     y = F.linear(x, weight.reshape(weight.shape[0], -1), bias)
     return F.silu(y) if epilogue == "silu" else y
 
@@ -176,7 +200,7 @@ _ROPE_TABLE_LIMIT = 16
 
 def _rope_table_cached(rotary_emb: torch.Tensor, N: int, device, head_dim: int) -> torch.Tensor:
     key = (rotary_emb.untyped_storage().data_ptr(), rotary_emb.storage_offset(), tuple(rotary_emb.shape),
-           tuple(rotary_emb.stride()), rotary_emb.dtype, rotary_emb.device, rotary_emb._version, N,
+           tuple(rotary_emb.stride()), rotary_emb.dtype, rotary_emb.device, _version(rotary_emb), N,
            torch.device(device), head_dim)
     capturing = rotary_emb.is_cuda and torch.cuda.is_current_stream_capturing()
     entry = _ROPE_TABLES.get(key)
@@ -308,13 +332,12 @@ class LiteLA(nn.Module):
         change, not part of the state_dict."""
         quant = self.qkv.is_quantized
         ps = (self.qkv.weight_q, self.qkv.weight_scale, self.qkv.bias) if quant else (self.qkv.weight, self.qkv.bias)
-        key = tuple((p.data_ptr(), p._version, p.device) for p in ps if p is not None)
         cache = self.__dict__.get("_tiled_cache")
-        if cache is None or cache[0] != key:
+        if cache is None or not _sources_unchanged(cache[0], ps):
             with torch.no_grad():
                 tiled = [None if p is None else ops.tile_qkv_rows(p.detach(), self.heads) for p in ps]
             # (weight, bias), the weight being the pair (int8 weight, scales) of a quantised projection
-            cache = (key, ((tiled[0], tiled[1]), tiled[2]) if quant else (tiled[0], tiled[1]))
+            cache = (_source_entry(ps), ((tiled[0], tiled[1]), tiled[2]) if quant else (tiled[0], tiled[1]))
             self.__dict__["_tiled_cache"] = cache
         return cache[1]
 
@@ -621,12 +644,11 @@ class GLUMBConvTemp(GLUMBConv):
         """t_conv.weight [C, C, t, 1] -> [C, t*C] with k = tap * C + input channel (derived data, rebuilt when
         the parameter changes; not part of the state_dict)."""
         w = self.t_conv.weight
-        key = (w.data_ptr(), w._version, w.device)
         cache = self.__dict__.get("_tconv_cache")
-        if cache is None or cache[0] != key:
+        if cache is None or not _sources_unchanged(cache[0], (w,)):
             with torch.no_grad():
                 w2 = w[:, :, :, 0].permute(0, 2, 1).reshape(w.shape[0], -1).contiguous()
-            cache = (key, w2)
+            cache = (_source_entry((w,)), w2)
             self.__dict__["_tconv_cache"] = cache
         return cache[1]
 
@@ -824,9 +846,8 @@ class MultiHeadCrossAttention(nn.Module):
     def _padded(self, pad_to):
         ps = (self.q_linear.weight, self.q_linear.bias, self.kv_linear.weight, self.kv_linear.bias,
               self.proj.weight)
-        key = tuple((p.data_ptr(), p._version, p.dtype, p.device) for p in ps) + (pad_to,)
         cache = self.__dict__.get("_pad_cache")
-        if cache is None or cache[0] != key:
+        if cache is None or cache[2] != pad_to or not _sources_unchanged(cache[0], ps):
             H, d, C, e = self.num_heads, self.head_dim, self.d_model, pad_to - self.head_dim
             with torch.no_grad():
                 wq = F.pad(ps[0].view(H, d, C), (0, 0, 0, e)).reshape(H * pad_to, C)
@@ -834,7 +855,8 @@ class MultiHeadCrossAttention(nn.Module):
                 wkv = F.pad(ps[2].view(2, H, d, C), (0, 0, 0, e)).reshape(2 * H * pad_to, C)
                 bkv = F.pad(ps[3].view(2, H, d), (0, e)).reshape(-1)
                 wo = F.pad(ps[4].view(C, H, d), (0, e)).reshape(C, H * pad_to)
-            cache = (key, (wq.contiguous(), bq.contiguous(), wkv.contiguous(), bkv.contiguous(), wo.contiguous()))
+            cache = (_source_entry(ps), (wq.contiguous(), bq.contiguous(), wkv.contiguous(), bkv.contiguous(),
+                                         wo.contiguous()), pad_to)
             self.__dict__["_pad_cache"] = cache
         return cache[1]
 
@@ -904,7 +926,7 @@ class MultiHeadCrossAttention(nn.Module):
             k, v = kv[:, :, 0].transpose(1, 2), kv[:, :, 1].transpose(1, 2)
         else:
             q = self.q_linear(x)
-            kv = self.kv_linear(cond).view(B, -1, 2, C)
+            kv = (self.kv_linear(cond) if kv is None else kv).view(B, -1, 2, C)   # the caller's kv_linear(cond), if given
             k, v = kv.unbind(2)
             q = self.q_norm(q).view(B, -1, H, d).transpose(1, 2)
             k = self.k_norm(k).view(B, -1, H, d).transpose(1, 2)
@@ -961,7 +983,7 @@ class SanaMSBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = modulation.chunk(6, dim=1)
         # (conditioning in another dtype than x -- an fp32 t with a bf16 x -- promotes in the stock op chain; the
         # fused kernels read the modulation rows as x's dtype, so that case takes the stock composition below)
-        if x.is_cuda and x.dtype == torch.bfloat16 and shift_msa.dtype == x.dtype and C % 8 == 0 and C <= 8192 \
+        if x.is_cuda and x.dtype in ops.IO16 and shift_msa.dtype == x.dtype and C % 8 == 0 and C <= 8192 \
                 and not torch.is_grad_enabled():
             # fused seams: LayerNorm + modulate in one kernel, gate * out + residual in the GEMM epilogue
             h = ops.layernorm_modulate(x, scale_msa, shift_msa, self.norm1.eps)
@@ -980,7 +1002,7 @@ class SanaMSBlock(nn.Module):
                                                    self.norm2.eps)
             return self.mlp.forward_gated(h, HW, gate_mlp, x)
         stock_path("SanaMSBlock LayerNorm / modulate / gate / residual seams",
-                   f"the fused seams are bf16 inference only (C % 8 == 0, C <= 8192); got x {x.dtype}, t {t.dtype}, C = {C}, "
+                   f"the fused seams are bf16 / fp16 inference only (C % 8 == 0, C <= 8192); got x {x.dtype}, t {t.dtype}, C = {C}, "
                    f"grad {'on' if torch.is_grad_enabled() else 'off'}")
         x = x + self.drop_path(
             gate_msa * self.attn(t2i_modulate(self.norm1(x), shift_msa, scale_msa), HW=HW, rotary_emb=image_rotary_emb))
@@ -1017,13 +1039,13 @@ class StepConditioning:
 
     def _stacked(self):
         ps = [(b.cross_attn.kv_linear.weight, b.cross_attn.kv_linear.bias, b.scale_shift_table) for b in self.blocks]
-        key = tuple((p.data_ptr(), p._version) for trio in ps for p in trio)
-        if key != self._key:
+        flat = tuple(p for trio in ps for p in trio)
+        if not _sources_unchanged(self._key, flat):
             with torch.no_grad():
                 self._w = torch.cat([w for w, _, _ in ps])                     # [L * 2C, C]
                 self._b = torch.cat([b for _, b, _ in ps])                     # [L * 2C]
                 self._tab = torch.stack([s for _, _, s in ps])[:, None]        # [L, 1, 6, C]
-            self._key = key
+            self._key = _source_entry(flat)
         return self._w, self._b, self._tab
 
     def __call__(self, y, t):
@@ -1036,8 +1058,13 @@ class StepConditioning:
             return [{} for _ in self.blocks]
         w, b, tab = self._stacked()
         B, Nk, C = y.shape
-        kv = ops.gemm_bf16(y.reshape(B * Nk, C), w, b, "bias").view(B, Nk, L, 2 * C)
         mod = tab + t.reshape(1, B, 6, -1)                                     # [L, B, 6, C]
+        # the stacked kv GEMM only where the blocks' cross-attention consumes it: the stock composition for 96 <
+        # head_dim < 128 applies kv_linear with a padded copy of its weight and would discard the result
+        if not all(ops.cross_attention_supported(b.cross_attn.head_dim, Nk) or not 96 < b.cross_attn.head_dim < 128
+                   for b in self.blocks):
+            return [dict(modulation=mod[i]) for i in range(L)]
+        kv = ops.gemm_bf16(y.reshape(B * Nk, C), w, b, "bias").view(B, Nk, L, 2 * C)
         return [dict(text_kv=kv[:, :, i], modulation=mod[i]) for i in range(L)]
 
 

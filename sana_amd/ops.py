@@ -13,6 +13,7 @@ from . import _lib
 from ._lib import DT_BF16, DT_F16, DT_F32, SanaHipError
 
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
+IO16 = (torch.bfloat16, torch.float16)   # the 16-bit io dtypes of the GEMMs and of the block's fused seams
 HEAD_DIM = 32
 HEAD_DIMS = (32, 112)   # head dims with kernels: 32 (all dtypes), 112 (bf16; the video configurations)
 
@@ -311,10 +312,12 @@ def _gemm_workspace(lib, device, M: int, N: int, K: int) -> Tuple[Optional[int],
 
 def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
               epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """a: [M, K] bf16; weight: [N, K] bf16 (nn.Linear layout).  Returns epilogue(a @ weight.T) [M, N] bf16."""
+    """a: [M, K]; weight: [N, K] (nn.Linear layout); both bf16, or both fp16 (``sana_hip_gemm_f16``: the same
+    kernels on the fp16 MFMA).  Returns epilogue(a @ weight.T) [M, N] in that dtype."""
     _need_cuda(a, weight, bias)
-    if a.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-        raise SanaHipError("gemm_bf16 needs bf16 operands")
+    dt = a.dtype
+    if dt not in IO16 or weight.dtype != dt:
+        raise SanaHipError(f"the GEMM needs bf16 or fp16 operands of one dtype, got {a.dtype} and {weight.dtype}")
     a, lda = _rows(a, "a")
     weight, ldw = _rows(weight, "weight")
     M, K = a.shape
@@ -324,18 +327,19 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     epi = _EPI[epilogue]
     if bias is not None and epi == _lib.EPI_NONE:
         epi = _lib.EPI_BIAS
-    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
-        raise SanaHipError("bias must be contiguous bf16 [N]")
+    if bias is not None and (bias.dtype != dt or bias.numel() != N or not bias.is_contiguous()):
+        raise SanaHipError(f"bias must be contiguous {dt} [N]")
     if out is None:
-        out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+        out = torch.empty(M, N, dtype=dt, device=a.device)
     out, ldc = _rows(out, "out")
-    if tuple(out.shape) != (M, N) or out.dtype != torch.bfloat16:
+    if tuple(out.shape) != (M, N) or out.dtype != dt:
         raise SanaHipError("out has the wrong shape or dtype")
     if M == 0:
         return out
     lib = _lib.load()
     ws, nbytes = _gemm_workspace(lib, a.device, M, N, K)
-    code = lib.sana_hip_gemm_bf16(a.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
+    fn = lib.sana_hip_gemm_f16 if dt == torch.float16 else lib.sana_hip_gemm_bf16
+    code = fn(a.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
                                   out.data_ptr(), M, N, K, lda, ldw, ldc, epi, ws, nbytes, _stream())
     _lib.check(code, "sana_hip_gemm_bf16")
     return out
@@ -468,7 +472,7 @@ def gemm_w8a16(a: torch.Tensor, wq: torch.Tensor, scale: torch.Tensor, bias: Opt
 
 # --------------------------------------------------------------------------- fused seams of the block
 
-def _mod_rows(t: torch.Tensor, B: int, C: int, what: str, dtype=torch.bfloat16) -> Tuple[torch.Tensor, int]:
+def _mod_rows(t: torch.Tensor, B: int, C: int, what: str, dtype) -> Tuple[torch.Tensor, int]:
     """Per-batch row vectors [B, 1, C] / [B, C] with unit inner stride -> (tensor, batch stride)."""
     if t.dtype != dtype:     # the kernels read these rows as 16-bit values: another dtype would be misread
         raise SanaHipError(f"{what} must be {dtype} like the activations, got {t.dtype}")
@@ -489,26 +493,35 @@ def gemm_gate_residual(a: torch.Tensor, weight: torch.Tensor, bias: Optional[tor
     if weight_scale is not None and (expand or (expand is None and B * Ntok >= W8_EXPAND_MIN_ROWS)):
         weight, weight_scale = dequant_w8(weight.reshape(weight.shape[0], -1), weight_scale), None
     C = weight.shape[0]
-    if a.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or gate.dtype != torch.bfloat16:
-        raise SanaHipError("gemm_gate_residual is bf16 only")
-    if weight_scale is None and weight.dtype != torch.bfloat16:
-        raise SanaHipError(f"weight must be bf16 (or int8 together with weight_scale), got {weight.dtype}")
+    dt = a.dtype
+    if dt not in IO16 or residual.dtype != dt or gate.dtype != dt:
+        raise SanaHipError("gemm_gate_residual needs bf16 or fp16 activations, gate and residual of one dtype")
+    if weight_scale is not None and dt != torch.bfloat16:
+        raise SanaHipError("W8A16 needs bf16 activations")
+    if weight_scale is None and weight.dtype != dt:
+        raise SanaHipError(f"weight must be {dt} (or int8 together with weight_scale), got {weight.dtype}")
     if weight_scale is not None and (weight.dtype != torch.int8 or weight_scale.dtype != torch.float32
                                      or weight_scale.numel() != C or not weight_scale.is_contiguous()):
         raise SanaHipError("W8A16 needs an int8 weight and contiguous fp32 scales, one per output channel")
-    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != C or not bias.is_contiguous()):
-        raise SanaHipError("bias must be contiguous bf16 [C]")
+    if bias is not None and (bias.dtype != dt or bias.numel() != C or not bias.is_contiguous()):
+        raise SanaHipError(f"bias must be contiguous {dt} [C]")
     if weight.reshape(C, -1).shape[1] != K:
         raise SanaHipError(f"K mismatch: a {tuple(a.shape)} vs weight {tuple(weight.shape)}")
     a2, lda = _rows(a.reshape(B * Ntok, K), "a")
     w2, ldw = _rows(weight.reshape(C, -1), "weight")
     r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
-    g2, gstride = _mod_rows(gate, B, C, "gate")
-    out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=a.device)
+    g2, gstride = _mod_rows(gate, B, C, "gate", dt)
+    out = torch.empty(B * Ntok, C, dtype=dt, device=a.device)
     if B * Ntok == 0:
         return out.view(B, Ntok, C)
     lib = _lib.load()
     ws, nbytes = _gemm_workspace(lib, a.device, B * Ntok, C, K)
+    if dt == torch.float16:
+        code = lib.sana_hip_gemm_gate_residual_f16(
+            a2.data_ptr(), w2.data_ptr(), bias.data_ptr() if bias is not None else None, g2.data_ptr(), r2.data_ptr(),
+            out.data_ptr(), B * Ntok, C, K, lda, ldw, ldr, C, Ntok, gstride, ws, nbytes, _stream())
+        _lib.check(code, "sana_hip_gemm_gate_residual_f16")
+        return out.view(B, Ntok, C)
     code = lib.sana_hip_gemm_gate_residual(
         a2.data_ptr(), w2.data_ptr(), weight_scale.data_ptr() if weight_scale is not None else None,
         bias.data_ptr() if bias is not None else None, g2.data_ptr(), r2.data_ptr(), out.data_ptr(),
@@ -659,17 +672,16 @@ def gate_residual(y: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor) -
     """residual + gate * y in one pass with the stock op pair's two roundings; y, residual: [B, N, C] bf16;
     gate: [B, 1, C], or one row per group of consecutive tokens, [B, G, 1, C]."""
     _need_cuda(y, gate, residual)
-    if y.shape != residual.shape or y.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or \
-            gate.dtype != torch.bfloat16:
-        raise SanaHipError("gate_residual needs bf16 y and residual of one shape and a bf16 gate")
+    if y.shape != residual.shape or y.dtype not in IO16 or residual.dtype != y.dtype or gate.dtype != y.dtype:
+        raise SanaHipError("gate_residual needs bf16 or fp16 y, residual (of one shape) and gate of one dtype")
     B, Ntok, C = y.shape
     groups = gate.numel() // max(B * C, 1)
     if groups < 1 or gate.numel() != B * groups * C or Ntok % groups:
         raise SanaHipError(f"gate {tuple(gate.shape)} does not divide the {Ntok} tokens of {B} batch entries")
     y2, ldy = _rows(y.reshape(B * Ntok, C), "y")
     r2, ldr = _rows(residual.reshape(B * Ntok, C), "residual")
-    g2, gstride = _mod_rows(gate.reshape(B * groups, 1, C), B * groups, C, "gate")
-    out = torch.empty(B * Ntok, C, dtype=torch.bfloat16, device=y.device)
+    g2, gstride = _mod_rows(gate.reshape(B * groups, 1, C), B * groups, C, "gate", y.dtype)
+    out = torch.empty(B * Ntok, C, dtype=y.dtype, device=y.device)
     if B * Ntok == 0:
         return out.view(B, Ntok, C)
     code = _lib.load().sana_hip_gate_residual(y2.data_ptr(), g2.data_ptr(), r2.data_ptr(), out.data_ptr(), B * Ntok, C,

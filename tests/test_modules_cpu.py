@@ -181,7 +181,50 @@ def test_stock_paths_are_logged_once_and_wrappers_reject_foreign_dtypes(caplog):
     assert len(caplog.records) == 2 and "stock PyTorch ops" in caplog.records[0].getMessage()
     rows32 = torch.zeros(2, 1, 64)
     with pytest.raises(SanaHipError, match="must be torch.bfloat16"):
-        ops._mod_rows(rows32, 2, 64, "scale")
-    assert ops._mod_rows(rows32.bfloat16(), 2, 64, "scale")[1] == 64
+        ops._mod_rows(rows32, 2, 64, "scale", torch.bfloat16)
+    assert ops._mod_rows(rows32.bfloat16(), 2, 64, "scale", torch.bfloat16)[1] == 64
     # device checks come first for real calls; the dtype checks of the GEMM wrapper are reachable with meta-free
     # CPU tensors only up to the device check, so the rest is exercised on the GPU (tests/test_gpu_modules.py)
+
+
+def test_derived_data_caches_work_under_inference_mode_and_follow_replaced_parameters():
+    """The reference pipelines run under torch.inference_mode() (app/sana_pipeline.py:166): tensors created there
+    have no version counter.  The caches of derived data (rope table, tiled qkv weight, stacked step conditioning)
+    must work on such tensors, and a parameter REPLACED by another tensor is a miss even when the allocator hands
+    the new tensor the old address."""
+    from sana_amd import modules as M
+    with torch.inference_mode():
+        ang = torch.rand(1, 1, 8, 16) * 6.28
+        rot = torch.polar(torch.ones_like(ang), ang)
+        assert rot.is_inference()
+        t1 = M._rope_table_cached(rot, 8, "cpu", 32)
+        assert M._rope_table_cached(rot, 8, "cpu", 32) is t1
+        assert torch.allclose(t1[..., 0], torch.cos(ang)[0, 0], atol=1e-6) and torch.allclose(t1[..., 1], torch.sin(ang)[0, 0], atol=1e-6)
+        la = S.LiteLA(64, 64, dim=32)
+        w1, b1 = la._tiled_qkv()
+        assert la._tiled_qkv()[0] is w1 and b1 is None
+        blocks = [S.SanaMSBlock(64, 4, mlp_ratio=2.5, attn_type="linear", ffn_type="glumbconv") for _ in range(2)]
+        for b in blocks:   # parameters created inside inference mode
+            assert b.scale_shift_table.is_inference()
+        sc = S.StepConditioning(blocks)
+        w, bias, tab = sc._stacked()
+        assert sc._stacked()[0] is w and tuple(w.shape) == (2 * 128, 64) and tuple(tab.shape) == (2, 1, 6, 64)
+    # outside inference mode: an in-place edit and a replaced parameter both rebuild
+    la = S.LiteLA(64, 64, dim=32)
+    w1, _ = la._tiled_qkv()
+    with torch.no_grad():
+        la.qkv.weight.mul_(2.0)
+    w2, _ = la._tiled_qkv()
+    assert w2 is not w1 and torch.equal(w2, 2.0 * w1)
+    old = la.qkv.weight
+    la.qkv.weight = torch.nn.Parameter(old.detach().clone() * 0.5)     # same shape, version 0, maybe the same address later
+    w3, _ = la._tiled_qkv()
+    assert w3 is not w2 and torch.equal(w3, w1)
+
+
+def test_graphed_call_needs_a_warm_up():
+    from sana_amd.graph import GraphedCall
+    with pytest.raises(ValueError):
+        GraphedCall(lambda x: x, [torch.zeros(1)], warmup=1)      # CPU tensors
+    src = inspect.getsource(GraphedCall.__init__)
+    assert "warmup < 1" in src
