@@ -25,9 +25,12 @@ summaries under profiles/ were taken with).  ``roofline.traffic`` is not
 measurable from inside the process: it is the HBM byte count of one launch of
 the dominant kernel from two ``rocprofv3 --pmc`` runs of ``--kernels-only --cfg3-only``
 (FETCH_SIZE, WRITE_SIZE), read at run time from profiles/kernels_cfg3_hbm_traffic.txt.
-``configs`` holds the two small configurations of the benchmark definition beside the
-headline: cfg1 (the LiteLA op alone, fp32, eps 1e-15) and cfg2 (one Sana-600M block,
-B=4), each with the oracle timed on the host cores.
+``configs`` holds the other configurations of the benchmark definition beside the
+headline: cfg1 (the LiteLA op alone, fp32, eps 1e-15), cfg2 (one Sana-600M block,
+B=4), cfg4 (the W8A16 block at B=16 x 1024 tokens) and cfg5 (chunk-causal attention
+with 70 heads of 32 on 21 x 30 x 52 tokens + the per-frame Mix-FFN), each with the
+oracle timed on the host cores; ``kernels`` also lists cfg2's four GEMMs with the
+library's time beside each.
 """
 from __future__ import annotations
 
@@ -155,6 +158,8 @@ def kernel_rooflines(dev, iters=50, warmup=10, stock_conv=False, cfg3_only=False
     if not cfg3_only:
         _kernel_rooflines_other_shapes(dev, add, qkv, state, out, la_bytes, g, iters, warmup)
     _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_only)
+    if not cfg3_only:
+        _kernel_rows_qk_norm_and_cfg2(dev, add, rows, g)
     # plain device copy as a bandwidth yardstick of this box
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
@@ -322,6 +327,55 @@ def _kernel_rooflines_ffn(dev, add, rows, g, iters, warmup, stock_conv, cfg3_onl
     del buf, ot
 
 
+def _kernel_rows_qk_norm_and_cfg2(dev, add, rows, g):
+    """litela_qk_norm_cfg3: what LiteLA with qk_norm=True (every Sana-1.5 configuration) runs between its qkv GEMM
+    and its proj GEMM -- the per-token 1/rms pass and the two attention phases with the norm applied on load --
+    as one timed sequence.  Then the four GEMMs of cfg2 (Sana-600M width, B=4 x 1024 tokens = 4096 rows) with
+    the library's plain GEMM of the same shape beside each."""
+    from sana_amd import ops
+
+    B, N, M = 1, 16384, 16384
+    qkv = torch.randn(B, N, 3, C, generator=g).bfloat16().to(dev)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    wn = (1 + 0.1 * torch.randn(C, generator=g)).bfloat16().to(dev)
+    out = torch.empty(B, N, C, dtype=torch.bfloat16, device=dev)
+
+    def qk_norm_attention():
+        rq, rk = ops.qk_rms(q, k, 1e-5)
+        st = ops.linattn_state(k, v, pre=ops.QkPre(rk, wn, None))
+        ops.linattn_apply(q, st, 1e-8, out=out, pre=ops.QkPre(rq, wn, None))
+
+    add("litela_qk_norm_cfg3", "hbm", 2 * M * C * 2 + 2 * (2 * M * C * 2) + 3 * 2 * M * 4 + 2 * (C // 32) * 33 * 32 * 4,
+        event_time_us(qk_norm_attention, 30, 5),
+        "qk_rms + linattn_state + linattn_apply with q/k RMSNorm on load (4 launches): q, k read twice, v read, out "
+        "written; beyond the plain qkv GEMM (the fused qkv+state route needs the whole k row's 1/rms before it can "
+        "contract a token, so it does not apply)")
+    del qkv, out
+    Cc, Hc, Mc = 1152, 2880, 4096
+    x_res = torch.randn(4, 1024, Cc, generator=g).bfloat16().to(dev)
+    mod = (torch.randn(4, 6, Cc, generator=g) * 0.5).bfloat16().to(dev)
+    for name, Nn, Kk, epi in (("cfg2_gemm_qkv", 3 * Cc, Cc, None), ("cfg2_gemm_proj_gate_residual", Cc, Cc, "gate_res"),
+                              ("cfg2_gemm_inverted", 2 * Hc, Cc, "bias_silu"),
+                              ("cfg2_gemm_point_gate_residual", Cc, Hc, "gate_res")):
+        a = torch.randn(Mc, Kk, generator=g).bfloat16().to(dev)
+        w = (torch.randn(Nn, Kk, generator=g) * 0.02).bfloat16().to(dev)
+        bias = torch.zeros(Nn, dtype=torch.bfloat16, device=dev) if epi else None
+        o = torch.empty(Mc, Nn, dtype=torch.bfloat16, device=dev)
+        if epi == "gate_res":
+            fn = lambda: ops.gemm_gate_residual(a.view(4, 1024, Kk), w, bias, mod[:, 2:3], x_res)
+        else:
+            fn = lambda: ops.gemm_bf16(a, w, bias, epi, out=o)
+        add(name, "mfma", 2 * Mc * Nn * Kk, event_time_us(fn, 50, 10), f"2*M*K*N, M={Mc} N={Nn} K={Kk} (cfg2: B=4 x 1024 tokens)")
+        rows[-1]["library_gemm_us"] = round(event_time_us(lambda: torch.nn.functional.linear(a, w, bias), 50, 10), 2)
+        if name == "cfg2_gemm_qkv":
+            wt_, _ = ops.tile_qkv_weight(w, None, Cc // 32)
+            add("cfg2_gemm_qkv_with_attention_state", "mfma", 2 * Mc * Nn * Kk + 2 * Mc * Cc * 33,
+                event_time_us(lambda: ops.gemm_qkv_state(a.view(4, 1024, Kk), wt_, None, Cc // 32), 50, 10),
+                f"2*M*K*N + state, M={Mc} N={Nn} K={Kk}: the route the cfg2 block takes (replaces cfg2_gemm_qkv + phase 1)")
+            del wt_
+        del a, w, o
+
+
 _STATES = {}
 
 
@@ -480,6 +534,96 @@ def small_configs(dev):
     return res
 
 
+def _cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return ""
+
+
+def config4(dev, ips_w8: float, ips_bf16: float):
+    """cfg4: W8A16 Sana-1.6B at 1024px, B=16 x 1024 tokens; GPU figures from the images/s legs, host: ONE oracle
+    block on the dequantised weights in fp32 at the same shape."""
+    from oracle import sana_oracle as O
+
+    B, HW = 16, (32, 32)
+    blk = O.SanaMSBlock(C, HEADS_X, mlp_ratio=MLP_RATIO, attn_type="linear", ffn_type="glumbconv")
+    blk.load_state_dict({k: v.float() for k, v in O.dequantized_block_state(make_state(0)).items()})
+    blk.attn.fp32_attention = True
+    x, y, t = make_inputs(B, HW[0] * HW[1])
+    with torch.no_grad():
+        blk(x, y, t, HW=HW)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            blk(x, y, t, HW=HW)
+        t_cpu = (time.perf_counter() - t0) / 3 * 1e3
+    return {"workload": "W8A16 (int8 per-output-channel qkv / proj / 1x1-conv weights, bf16 activations) Sana-1.6B block, "
+                        "B=16 images of N=32x32=1024 tokens, C=2240, 300 text tokens, random init",
+            "gpu_block_ms": round(B / ips_w8 / DEPTH * 1e3, 4), "gpu_block_ms_bf16_weights": round(B / ips_bf16 / DEPTH * 1e3, 4),
+            "images_per_s": round(ips_w8, 2),
+            "note": "gpu_block_ms = step time of the 20 chained W8A16 blocks / 20 (the images_per_s_1024px leg)",
+            "cpu_baseline": {"value": round(t_cpu, 2), "unit": "ms per block forward", "cores": torch.get_num_threads(),
+                             "kind": "port", "sample": "1 of the 20 blocks at the same shape (B=16, N=1024) on the dequantised "
+                                                       f"weights, fp32, 3 timed iterations after 1 warm-up; cpu='{_cpu_model()}'"}}
+
+
+def config5(dev):
+    """cfg5: ChunkCausalAttention at C=2240 with 70 heads of 32 on 21 x 30 x 52 tokens, then the GLUMBConv Mix-FFN with
+    the depthwise 3x3 per frame -- the two modules as the configuration words them, GPU and host (oracle, fp32)."""
+    import sana_amd as S
+    from oracle import sana_oracle as O
+
+    T, H, W = 21, 30, 52
+    N = T * H * W
+    g = torch.Generator().manual_seed(9)
+
+    def tn(p):
+        return torch.nn.init.trunc_normal_(torch.empty(p.shape), std=0.02, generator=g)
+
+    oa = O.ChunkCausalAttention(C, C, heads=C // 32, eps=1e-8)
+    om = O.GLUMBConv(C, HID, use_bias=(True, True, False), norm=(None, None, None), act=("silu", "silu", None))
+    with torch.no_grad():
+        for m in (oa, om):
+            for n_, p_ in m.named_parameters():
+                p_.copy_(tn(p_) if p_.dim() > 1 else torch.zeros_like(p_))
+    oa.fp32_attention = True
+    ha = S.ChunkCausalAttention(C, C, heads=C // 32, eps=1e-8).bfloat16()
+    hm = S.GLUMBConv(C, HID, use_bias=(True, True, False), norm=(None, None, None), act=("silu", "silu", None)).bfloat16()
+    ha.load_state_dict({k: v.bfloat16() for k, v in oa.state_dict().items()})
+    hm.load_state_dict({k: v.bfloat16() for k, v in om.state_dict().items()})
+    ha, hm = ha.to(dev), hm.to(dev)
+    x = torch.randn(1, N, C, generator=g)
+    xd = x.bfloat16().to(dev)
+    every_frame = list(range(T))
+    res = {"workload": "chunk-causal linear attention module (qkv + attention + proj), bf16 io / fp32 state, C=2240, 70 heads x 32, "
+                       "21 frames x 30x52 tokens (N=32760), B=1, followed by the GLUMBConv Mix-FFN (hidden 5600) with the "
+                       "depthwise 3x3 per frame"}
+    with torch.no_grad():
+        res["gpu_attention_ms_21_chunks"] = round(event_time_us(
+            lambda: ha(xd, HW=(T, H, W), chunk_index=every_frame), 10, 3) / 1e3, 4)
+        res["gpu_attention_ms_chunks_0_11"] = round(event_time_us(
+            lambda: ha(xd, HW=(T, H, W), chunk_index=[0, 11]), 10, 3) / 1e3, 4)
+        res["gpu_mix_ffn_ms"] = round(event_time_us(lambda: hm(xd, HW=(T, H, W)), 10, 3) / 1e3, 4)
+        oa(x, HW=(T, H, W), chunk_index=[0, 11])
+        t0 = time.perf_counter()
+        for _ in range(2):
+            oa(x, HW=(T, H, W), chunk_index=[0, 11])
+        t_att = (time.perf_counter() - t0) / 2 * 1e3
+        om(x, HW=(T, H, W))
+        t0 = time.perf_counter()
+        for _ in range(2):
+            om(x, HW=(T, H, W))
+        t_ffn = (time.perf_counter() - t0) / 2 * 1e3
+    res["cpu_baseline"] = {"value": round(t_att + t_ffn, 1), "attention_ms": round(t_att, 1), "mix_ffn_ms": round(t_ffn, 1),
+                           "unit": "ms per pass of the two modules", "cores": torch.get_num_threads(), "kind": "port",
+                           "sample": "the whole workload (chunk_index [0, 11]) in fp32, 2 timed iterations after 1 warm-up; "
+                                     f"cpu='{_cpu_model()}'"}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -570,6 +714,9 @@ def main():
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
         "configs": None if args.no_cpu_baseline else small_configs(dev),
     }
+    if line["configs"] is not None:
+        line["configs"]["cfg4"] = config4(dev, ips_w8, ips_bf16)
+        line["configs"]["cfg5"] = config5(dev)
     print(json.dumps(line))
 
 

@@ -65,11 +65,15 @@ def test_cfg3_all_twenty_blocks_and_chain_drift(cuda):
     per-block parity at the full shape.  Beside it the HIP chain runs freely from x0; its distance from the oracle
     chain is the accumulated drift: bounded by 3e-3 * sqrt(blocks) in rel-L2 (one block contributes ~2e-3, mostly
     the bf16 rounding of the residual stream it hands on; independent roundings add in quadrature: measured
-    1.8e-3 after one block, 1.06e-2 after all twenty)."""
+    1.8e-3 after one block, 1.06e-2 after all twenty).
+    A third chain shows whose drift that is: the oracle itself in bf16 on the GPU (stock PyTorch ops with
+    ``fp32_attention``: the reference's own arithmetic at the precision it runs in), free-running from the same x0.
+    The HIP chain must end no further from the fp32 chain than 1.1 x that stock bf16 chain does."""
     HW = (128, 128)
     x, y, t = (a.bfloat16() for a in bench.make_inputs(1, HW[0] * HW[1]))
     yd, td = y.to(cuda), t.to(cuda)
-    ref_run, hip_run = x.float(), x.to(cuda)
+    ref_run, hip_run, stock_run = x.float(), x.to(cuda), x.to(cuda)
+    drift = stock_drift = 0.0
     with torch.no_grad():
         for i in range(bench.DEPTH):
             state = bench.make_state(i)
@@ -79,10 +83,15 @@ def test_cfg3_all_twenty_blocks_and_chain_drift(cuda):
             rl = check_block(hb(xin.to(cuda), yd, td, HW=HW), ref_run, f"cfg3 block {i}")
             hip_run = hb(hip_run, yd, td, HW=HW)
             drift = rel_l2(hip_run.cpu(), ref_run)
-            print(f"block {i:2d}: rel-L2 on the oracle's input {rl:.2e}; free-running chain drift {drift:.2e}; "
-                  f"|x| rms {ref_run.pow(2).mean().sqrt().item():.2f}", flush=True)
+            ob16 = ob.bfloat16().to(cuda)             # the same block as stock bf16 ops on the GPU
+            ob16.attn.fp32_attention = True
+            stock_run = ob16(stock_run, yd, td, HW=HW)
+            stock_drift = rel_l2(stock_run.cpu(), ref_run)
+            print(f"block {i:2d}: rel-L2 on the oracle's input {rl:.2e}; free-running chain drift {drift:.2e} "
+                  f"(stock bf16 chain: {stock_drift:.2e}); |x| rms {ref_run.pow(2).mean().sqrt().item():.2f}", flush=True)
             assert drift <= 3e-3 * math.sqrt(i + 1), f"chain drift after {i + 1} blocks: {drift:.3e}"
-            del ob, hb
+            del ob, hb, ob16
+    assert drift <= 1.1 * stock_drift, f"HIP chain drift {drift:.3e} against the stock bf16 chain's {stock_drift:.3e}"
 
 
 def test_step_conditioning_shared_by_the_blocks(cuda):
