@@ -164,6 +164,27 @@ int sana_hip_linattn_apply_pre(const void* q, const float* state, void* out,
                                void* stream);
 
 /* ---------------------------------------------------------------------------
+ * The transform order of LiteLA.forward itself (diffusion/model/nets/sana_blocks.py:274-286): q and k are
+ * RMS-normalised over all channels (`self.q_norm(q)`, :274-275), rotated BEFORE the ReLU by the real-valued rotary
+ * embedding (`apply_rotary_emb(q, rotary_emb, use_real_unbind_dim=-2)`, :282-284 and :1549-1582: channel pairs
+ * (2i, 2i+1) of a head, out = x * cos + rot(x) * sin in fp32, rounded to the io dtype), and only then enter
+ * attn_matmul (:286), whose ReLU, vk, ksum row and denominator all see the rotated values.
+ *   rope  [N][d/2][2] fp32 (cos, sin) of pair i -- the reference's cos / sin tables [N][d] with their two entries
+ *         per pair equal (what its table builders produce) -- or NULL;  rinv / weight as for the *_pre entry points.
+ * One chunk (LiteLA is not chunk-causal), head_dim 32, bf16 io (SANA_ERR_SHAPE / SANA_ERR_DTYPE otherwise); with
+ * rope NULL these are sana_hip_linattn_state_pre / sana_hip_linattn_apply_pre. */
+int sana_hip_litela_state(const void* k, const void* v, float* state,
+                          void* workspace, size_t workspace_bytes,
+                          int B, int N, int h, int d, int64_t stride_b, int64_t stride_n, int io_dtype,
+                          const float* k_rinv, const void* k_weight, const float* rope, void* stream);
+
+int sana_hip_litela_apply(const void* q, const float* state, void* out,
+                          int B, int N, int h, int d,
+                          int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
+                          float eps, int io_dtype, int out_dtype,
+                          const float* q_rinv, const void* q_weight, const float* rope, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Phase 1 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  *

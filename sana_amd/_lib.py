@@ -33,6 +33,12 @@ SIGNATURES = {
                                            c_int, c_int, c_int, c_int, c_int64, c_int64,
                                            c_void_p, c_int, c_int, c_int, c_int,
                                            c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sana_hip_litela_state": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                      c_int, c_int, c_int, c_int, c_int64, c_int64, c_int,
+                                      c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sana_hip_litela_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                      c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int,
+                                      c_void_p, c_void_p, c_void_p, c_void_p]),
     "sana_hip_linattn_state_noalloc": (c_int, [c_void_p, c_void_p, c_void_p,
                                                c_int, c_int, c_int, c_int, c_int64, c_int64,
                                                c_void_p, c_int, c_int, c_int, c_int,

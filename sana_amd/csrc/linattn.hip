@@ -50,7 +50,8 @@ constexpr int TILE = 32;                  // tokens per phase-1 tile
 // grid: x = nsplit, y = n_chunks, z = B * pairs;  block 256
 // dst: when nsplit == 1 the final state, else partial[(bh*n_chunks + c)*nsplit + split][1056]
 // ----------------------------------------------------------------------------
-// PRE: on-load transforms as compile-time bits (1 = q/k RMSNorm, 2 = rotary embedding)
+// PRE: on-load transforms as compile-time bits (1 = q/k RMSNorm, 2 = rotary embedding, 4 = the rotation comes before
+// the ReLU and ksum is taken from the rotated values: QkPre::rope_first)
 template <typename T, int PRE>
 __global__ __launch_bounds__(256) void linattn_state16_kernel(
     const uint16_t* __restrict__ K, const uint16_t* __restrict__ V, float* __restrict__ dst,
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
   }
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
 
-  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0, rope_first = (PRE & 4) != 0;
   u32x4_t kreg[4], vreg[4];
   // PRE: per-token 1/rms and this lane's four (cos, sin) pairs travel with the tile; the norm weight
   // of the lane's 8 channels is loop-invariant; ksum is accumulated here, per lane and channel,
@@ -137,13 +138,14 @@ __global__ __launch_bounds__(256) void linattn_state16_kernel(
       u32x4_t kk = kreg[i];
       if (PRE) {
         if (has_norm) kk = rms_scale8(kk, rin[i], kw);
+        if (rope_first) kk = rope8(kk, cs[i][0], cs[i][1]);
         kk = relu_pk16(kk);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           ks8[2 * e] += bf16_lo(kk[e]);
           ks8[2 * e + 1] += bf16_hi(kk[e]);
         }
-        if (has_rope) kk = rope8(kk, cs[i][0], cs[i][1]);
+        if (has_rope && !rope_first) kk = rope8(kk, cs[i][0], cs[i][1]);
       } else {
         kk = relu_pk16(kk);
       }
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
   }
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
+  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0, rope_first = (PRE & 4) != 0;
   u32x4_t qw[2] = {zero4, zero4};
   if (has_norm) {
 #pragma unroll
@@ -426,8 +428,9 @@ __global__ __launch_bounds__(256) void linattn_apply_bf16_kernel(
       for (int hh = 0; hh < 2; ++hh) {
         u32x4_t qd = *reinterpret_cast<const u32x4_t*>(stage + u * 2048 + slot_r[hh]);
         if (has_norm) qd = rms_scale8(qd, rin[u], qw[hh]);
+        if (rope_first) qd = rope8(qd, cs[u][0], cs[u][1]);              // rotated first: both operands
         qd = relu_pk16(qd);                                              // denominator operand
-        const u32x4_t qb = has_rope ? rope8(qd, cs[u][0], cs[u][1]) : qd;  // numerator operand
+        const u32x4_t qb = (has_rope && !rope_first) ? rope8(qd, cs[u][0], cs[u][1]) : qd;  // numerator operand
         f32x4_t acc[3];
 #pragma unroll
         for (int rb = 0; rb < 3; ++rb) {
@@ -625,6 +628,7 @@ static int check_pre(const QkPre& pre, int io_dtype) {
   if (!pre.rinv && !pre.rope) return SANA_OK;
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
   if (pre.rinv && !pre.weight) return SANA_ERR_ARG;
+  if (pre.rope_first && !pre.rope) return SANA_ERR_ARG;
   if ((pre.weight && !aligned16(pre.weight)) || (pre.rope && !aligned16(pre.rope))) return SANA_ERR_ALIGN;
   return SANA_OK;
 }
@@ -647,6 +651,7 @@ static int state_impl(const void* k, const void* v, float* state, void* workspac
   const int esz = io_dtype == SANA_DT_F32 ? 4 : 2;
   if (!aligned16(k) || !aligned16(v) || !aligned16(state) || (stride_n * esz) % 16 || (stride_b * esz) % 16)
     return SANA_ERR_ALIGN;
+  if (d == 112 && pre.rope_first) return SANA_ERR_SHAPE;  // the rotate-first order exists for head_dim 32 only
   if (d == 112)
     return launch_state112(k, v, state, workspace, workspace_bytes, B, N, h, stride_b, stride_n, chunk_starts, n_chunks,
                            max_chunk_tokens, causal, io_dtype, pre, static_cast<hipStream_t>(stream));
@@ -666,12 +671,14 @@ static int state_impl(const void* k, const void* v, float* state, void* workspac
                        pl.split_tokens, stride_b, stride_n);
   } else {
     dim3 grid(pl.nsplit, n_chunks, B * ((h + 1) / 2));
-    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0) | (pre.rope_first ? 4 : 0);
 #define SANA_STATE16(T, PRE)                                                                                  \
   hipLaunchKernelGGL((linattn_state16_kernel<T, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(k), \
                      static_cast<const uint16_t*>(v), dst, chunk_starts, N, h, n_chunks, pl.nsplit,           \
                      pl.split_tokens, stride_b, stride_n, pre)
     if (io_dtype == SANA_DT_F16) SANA_STATE16(F16, 0);
+    else if (mode == 7) SANA_STATE16(BF16, 7);
+    else if (mode == 6) SANA_STATE16(BF16, 6);
     else if (mode == 3) SANA_STATE16(BF16, 3);
     else if (mode == 2) SANA_STATE16(BF16, 2);
     else if (mode == 1) SANA_STATE16(BF16, 1);
@@ -693,7 +700,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state(
     const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N, int h, int d,
     int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens, int causal,
     int io_dtype, void* stream) {
-  const QkPre none = {nullptr, nullptr, nullptr};
+  const QkPre none = {nullptr, nullptr, nullptr, 0};
   return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, chunk_starts, n_chunks,
                     max_chunk_tokens, causal, io_dtype, none, stream);
 }
@@ -702,9 +709,18 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state_pre
     const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N, int h, int d,
     int64_t stride_b, int64_t stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens, int causal,
     int io_dtype, const float* k_rinv, const void* k_weight, const float* rope, void* stream) {
-  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope};
+  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope, 0};
   return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, chunk_starts, n_chunks,
                     max_chunk_tokens, causal, io_dtype, pre, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_litela_state(
+    const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N, int h, int d,
+    int64_t stride_b, int64_t stride_n, int io_dtype, const float* k_rinv, const void* k_weight, const float* rope,
+    void* stream) {
+  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope, rope ? 1 : 0};
+  return state_impl(k, v, state, workspace, workspace_bytes, B, N, h, d, stride_b, stride_n, nullptr, 1, N, 0, io_dtype,
+                    pre, stream);
 }
 
 // ---------------------------------------------------------------------------- phase 1 without a workspace argument
@@ -750,7 +766,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_state_noa
   if (!ws) return SANA_ERR_RUNTIME;
   // every partial state the reduction reads is written by the launch before it (empty splits write zeros), so the
   // array's old contents never reach a result and nothing has to be cleared
-  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope};
+  const QkPre pre = {k_rinv, static_cast<const uint16_t*>(k_weight), rope, 0};
   return state_impl(k, v, state, ws, (size_t)SANA_HIP_NOALLOC_SCRATCH_BYTES, B, N, h, d, stride_b, stride_n,
                     chunk_starts, n_chunks, max_chunk_tokens, causal, io_dtype, pre, stream);
 }
@@ -806,6 +822,7 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
       (o_stride_n * osz) % 16 || (o_stride_b * osz) % 16)
     return SANA_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d == 112 && pre.rope_first) return SANA_ERR_SHAPE;
   if (d == 112)
     return launch_apply112(q, state, out, B, N, h, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
                            n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, pre, s);
@@ -824,14 +841,18 @@ static int apply_impl(const void* q, const float* state, void* out, int B, int N
   hipLaunchKernelGGL((linattn_apply_bf16_kernel<F32, PRE>), grid, dim3(256), 0, s, static_cast<const uint16_t*>(q), \
                      state, out, chunk_starts, N, h, n_chunks, wg_tokens, q_stride_b, q_stride_n, o_stride_b,     \
                      o_stride_n, eps, pre, (int)gx, ngroups)
-    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+    const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0) | (pre.rope_first ? 4 : 0);
     if (out_dtype == SANA_DT_F32) {
-      if (mode == 3) SANA_APPLY(true, 3);
+      if (mode == 7) SANA_APPLY(true, 7);
+      else if (mode == 6) SANA_APPLY(true, 6);
+      else if (mode == 3) SANA_APPLY(true, 3);
       else if (mode == 2) SANA_APPLY(true, 2);
       else if (mode == 1) SANA_APPLY(true, 1);
       else SANA_APPLY(true, 0);
     } else {
-      if (mode == 3) SANA_APPLY(false, 3);
+      if (mode == 7) SANA_APPLY(false, 7);
+      else if (mode == 6) SANA_APPLY(false, 6);
+      else if (mode == 3) SANA_APPLY(false, 3);
       else if (mode == 2) SANA_APPLY(false, 2);
       else if (mode == 1) SANA_APPLY(false, 1);
       else SANA_APPLY(false, 0);
@@ -859,7 +880,7 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply(
     const void* q, const float* state, void* out, int B, int N, int h, int d, int64_t q_stride_b, int64_t q_stride_n,
     int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
     float eps, int io_dtype, int out_dtype, void* stream) {
-  const QkPre none = {nullptr, nullptr, nullptr};
+  const QkPre none = {nullptr, nullptr, nullptr, 0};
   return apply_impl(q, state, out, B, N, h, d, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
                     n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, none, stream);
 }
@@ -869,7 +890,16 @@ extern "C" __attribute__((visibility("default"))) int sana_hip_linattn_apply_pre
     int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts, int n_chunks, int max_chunk_tokens,
     float eps, int io_dtype, int out_dtype, const float* q_rinv, const void* q_weight, const float* rope,
     void* stream) {
-  const QkPre pre = {q_rinv, static_cast<const uint16_t*>(q_weight), rope};
+  const QkPre pre = {q_rinv, static_cast<const uint16_t*>(q_weight), rope, 0};
   return apply_impl(q, state, out, B, N, h, d, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts,
                     n_chunks, max_chunk_tokens, eps, io_dtype, out_dtype, pre, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int sana_hip_litela_apply(
+    const void* q, const float* state, void* out, int B, int N, int h, int d, int64_t q_stride_b, int64_t q_stride_n,
+    int64_t o_stride_b, int64_t o_stride_n, float eps, int io_dtype, int out_dtype, const float* q_rinv,
+    const void* q_weight, const float* rope, void* stream) {
+  const QkPre pre = {q_rinv, static_cast<const uint16_t*>(q_weight), rope, rope ? 1 : 0};
+  return apply_impl(q, state, out, B, N, h, d, q_stride_b, q_stride_n, o_stride_b, o_stride_n, nullptr, 1, N, eps,
+                    io_dtype, out_dtype, pre, stream);
 }

@@ -28,6 +28,10 @@ struct QkPre {
   const float* rinv;       // [B][N], or null
   const uint16_t* weight;  // [h*d] bf16, with rinv
   const float* rope;       // [N][d/2][2] (cos, sin) per token and pair of a head, or null
+  // 0: rotation after the ReLU, numerator operands only (LiteLAReLURope and the chunk-causal family);
+  // 1: rotation BEFORE the ReLU, rounded to the io dtype, and everything -- numerator, ksum row, denominator --
+  //    uses the rotated values (LiteLA.forward with image_rotary_emb, sana_blocks.py:282-286).  head_dim 32 only.
+  int rope_first;
 };
 
 // bf16(w * (x * rinv)): the float chain of the reference RMSNorm, rounded once at the end

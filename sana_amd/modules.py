@@ -216,6 +216,26 @@ def _rope_table_cached(rotary_emb: torch.Tensor, N: int, device, head_dim: int) 
     return entry[1]
 
 
+def _rope_real_table_cached(rotary_emb, N: int, device, head_dim: int):
+    """:func:`ops.rope_table_real` of a ``(cos, sin)`` pair through the same cache as the complex tables (an entry
+    may be None: a table whose pair entries differ is checked once, not on every call)."""
+    cos, sin = rotary_emb
+    key = ("real",) + tuple((t.untyped_storage().data_ptr(), t.storage_offset(), tuple(t.shape), tuple(t.stride()),
+                            t.dtype, t.device, _version(t)) for t in (cos, sin)) + (N, torch.device(device), head_dim)
+    capturing = torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+    entry = _ROPE_TABLES.get(key)
+    if entry is None:
+        entry = [(cos, sin), ops.rope_table_real(cos, sin, N, device, head_dim), capturing]
+        _ROPE_TABLES[key] = entry
+        if len(_ROPE_TABLES) > _ROPE_TABLE_LIMIT:
+            for old in [k for k, e in _ROPE_TABLES.items() if not e[2]][:len(_ROPE_TABLES) - _ROPE_TABLE_LIMIT]:
+                del _ROPE_TABLES[old]
+    else:
+        _ROPE_TABLES.move_to_end(key)
+        entry[2] = entry[2] or capturing
+    return entry[1]
+
+
 def _as_token_major(t: torch.Tensor, token_dim: int) -> torch.Tensor:
     """(B, h, d, N) [token_dim=3] or (B, h, N, d) [token_dim=2] -> [B, N, h*d] with
     unit channel stride, without a copy when the memory already is token-major."""
@@ -289,7 +309,8 @@ class LiteLA(nn.Module):
             qkv[:, :, 1].copy_(self.k_norm(qkv[:, :, 1]))
         if rotary_emb is not None:
             stock_path("LiteLA rotary embedding", "the real-valued pre-ReLU rotation of LiteLA.forward "
-                       "(sana_blocks.py:282-284) has no kernel; applied in place on the qkv buffer")
+                       "(sana_blocks.py:282-284) runs inside the kernels for bf16, head_dim 32 and (cos, sin) tables whose "
+                       "two entries per channel pair are equal; applied in place on the qkv buffer otherwise")
             _rotary_real_tokens_(qkv[:, :, 0], rotary_emb)
             _rotary_real_tokens_(qkv[:, :, 1], rotary_emb)
         return qkv
@@ -311,6 +332,17 @@ class LiteLA(nn.Module):
         elif rotary_emb is None and x.dtype == torch.bfloat16:   # qk-norm (if any) on load inside the kernels
             B, N, C = x.shape
             out = self._attend(self.qkv(x).view(B, N, 3, C), None)
+        elif x.dtype == torch.bfloat16 and x.is_cuda and self.dim == 32 and \
+                (table := _rope_real_table_cached(rotary_emb, x.shape[1], x.device, self.dim)) is not None:
+            # LiteLA.forward's own order (sana_blocks.py:274-286): norm, rotation BEFORE the ReLU, everything rotated --
+            # applied on load inside the two attention kernels, nothing written back to the qkv buffer
+            B, N, C = x.shape
+            qkv = self.qkv(x).view(B, N, 3, C)
+            pre_q, pre_k = self._pre(qkv, None)
+            pre_q = ops.QkPre(pre_q.rinv if pre_q else None, pre_q.weight if pre_q else None, table, rope_first=True)
+            pre_k = ops.QkPre(pre_k.rinv if pre_k else None, pre_k.weight if pre_k else None, table, rope_first=True)
+            state = ops.linattn_state(qkv[:, :, 1], qkv[:, :, 2], pre=pre_k, head_dim=self.dim)
+            out = ops.linattn_apply(qkv[:, :, 0], state, self.eps, pre=pre_q)
         else:
             qkv = self._qkv_tokens(x, rotary_emb)
             out = ops.relu_linear_attention(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], self.eps, head_dim=self.dim)

@@ -94,14 +94,18 @@ class QkPre:
     """Transforms applied to q or k on load inside the attention kernels (bf16 io):
     RMSNorm over all channels (``rinv`` [B, N] fp32 from :func:`qk_rms` and the bf16
     ``weight`` [C]) before the ReLU, rotary embedding (``rope`` [N, head_dim/2, 2] fp32 from
-    :func:`rope_table`) after it, on the numerator operands only."""
+    :func:`rope_table`) after it, on the numerator operands only.  ``rope_first=True`` is the order of
+    ``LiteLA.forward`` instead (sana_blocks.py:282-286): the rotation comes BEFORE the ReLU and every
+    operand -- numerator, ksum row, denominator -- sees the rotated values (head_dim 32, one chunk)."""
 
-    __slots__ = ("rinv", "weight", "rope")
+    __slots__ = ("rinv", "weight", "rope", "rope_first")
 
-    def __init__(self, rinv=None, weight=None, rope=None):
+    def __init__(self, rinv=None, weight=None, rope=None, rope_first: bool = False):
         if (rinv is None) != (weight is None):
             raise SanaHipError("rinv and weight go together")
-        self.rinv, self.weight, self.rope = rinv, weight, rope
+        if rope_first and rope is None:
+            raise SanaHipError("rope_first needs a rope table")
+        self.rinv, self.weight, self.rope, self.rope_first = rinv, weight, rope, bool(rope_first)
 
     def check(self, x: torch.Tensor, head_dim: int = HEAD_DIM) -> Tuple[Optional[int], Optional[int], Optional[int]]:
         B, N, C = x.shape
@@ -151,6 +155,19 @@ def rope_table(freqs: torch.Tensor, N: int, device, head_dim: int = HEAD_DIM) ->
     return torch.view_as_real(f.to(torch.complex64)).to(device=device, dtype=torch.float32).contiguous()
 
 
+def rope_table_real(cos: torch.Tensor, sin: torch.Tensor, N: int, device, head_dim: int = HEAD_DIM) -> Optional[torch.Tensor]:
+    """The real-valued rotary tables ``LiteLA.forward`` receives -- ``(cos, sin)``, each [N, d], applied to the channel
+    pairs (2i, 2i+1) of a head (sana_blocks.py:1572-1582) -- as the kernels' fp32 (cos, sin) table [N, d/2, 2], or None
+    when the two entries of some pair differ (the reference's builders repeat every angle for its pair; a table
+    that does not is not a rotation of the pair and has no kernel form)."""
+    if cos.shape != sin.shape or cos.dim() != 2 or tuple(cos.shape) != (N, head_dim):
+        raise SanaHipError(f"rotary_emb must be (cos, sin) of shape {(N, head_dim)}, got {tuple(cos.shape)} / {tuple(sin.shape)}")
+    c, sn = cos.to(torch.float32), sin.to(torch.float32)
+    if not (torch.equal(c[:, 0::2], c[:, 1::2]) and torch.equal(sn[:, 0::2], sn[:, 1::2])):
+        return None
+    return torch.stack([c[:, 0::2], sn[:, 0::2]], dim=-1).to(device=device).contiguous()
+
+
 def _head_dim(d: int) -> int:
     if d not in HEAD_DIMS:
         raise SanaHipError(f"head_dim {d} has no kernel (supported: {HEAD_DIMS})")
@@ -193,6 +210,16 @@ def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: b
     shape = (B, N, h, d, sb, sn, tab.data_ptr() if tab is not None else None, n_chunks, longest,
              1 if causal else 0, _dt(k))
     pre_args = pre.check(k, d) if pre is not None else (None, None, None)
+    if pre is not None and pre.rope_first:
+        if n_chunks != 1 or noalloc:
+            raise SanaHipError("the rotate-before-ReLU order (LiteLA.forward) is not chunk-causal and has no no-alloc form")
+        nbytes = lib.sana_hip_linattn_workspace_bytes(B, h, d, 1, N, _dt(k))
+        ws = _workspace(k.device, nbytes)
+        code = lib.sana_hip_litela_state(k.data_ptr(), v.data_ptr(), state.data_ptr(),
+                                         ws.data_ptr() if ws is not None else None, nbytes, B, N, h, d, sb, sn, _dt(k),
+                                         *pre_args, _stream())
+        _lib.check(code, "sana_hip_litela_state")
+        return state
     if noalloc:
         code = lib.sana_hip_linattn_state_noalloc(k.data_ptr(), v.data_ptr(), state.data_ptr(), *shape, *pre_args,
                                                   _stream())
@@ -249,6 +276,13 @@ def linattn_apply(q: torch.Tensor, state: torch.Tensor, eps: float, chunk_tokens
         return out
     args = (q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, d, qsb, qsn, osb, osn,
             tab.data_ptr() if tab is not None else None, n_chunks, longest, float(eps), _dt(q), _DT[out_dtype])
+    if pre is not None and pre.rope_first:
+        if n_chunks != 1:
+            raise SanaHipError("the rotate-before-ReLU order (LiteLA.forward) is not chunk-causal")
+        code = _lib.load().sana_hip_litela_apply(q.data_ptr(), state.data_ptr(), out.data_ptr(), B, N, h, d, qsb, qsn,
+                                                osb, osn, float(eps), _dt(q), _DT[out_dtype], *pre.check(q, d), _stream())
+        _lib.check(code, "sana_hip_litela_apply")
+        return out
     if pre is None:
         code = _lib.load().sana_hip_linattn_apply(*args, _stream())
     else:

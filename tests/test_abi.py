@@ -32,7 +32,7 @@ def test_exports_every_declared_symbol():
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.sana_hip_abi_version() == 7
+    assert lib.sana_hip_abi_version() == 8
     assert b"aligned" in lib.sana_hip_strerror(-3)
     assert b"unknown" in lib.sana_hip_strerror(-99)
 

@@ -180,3 +180,90 @@ def test_cached_stream_equals_chunk_causal(cuda):
             acc_ref = cache_ref if acc_ref is None else [acc_ref[0] + cache_ref[0], acc_ref[1] + cache_ref[1]]
             check(out, ref, f"cached chunk {a}:{b}")
             assert rel_l2(cache[0].cpu(), cache_ref[0]) <= 1e-2 and rel_l2(cache[1].cpu(), cache_ref[1]) <= 1e-2
+
+
+# ---------------------------------------------------------------- LiteLA.forward's own order: rotation BEFORE the ReLU
+
+
+def real_tables(N, seed, head_dim=32, pair_equal=True):
+    """(cos, sin) [N, head_dim] as LiteLA.forward receives them (sana_blocks.py:282-284); generic angles."""
+    g = torch.Generator().manual_seed(seed)
+    if pair_equal:
+        theta = (torch.rand(N, head_dim // 2, generator=g) * 6.283).repeat_interleave(2, 1)
+    else:
+        theta = torch.rand(N, head_dim, generator=g) * 6.283
+    return torch.cos(theta), torch.sin(theta)
+
+
+@pytest.mark.parametrize("B,N,C,qk_norm", [(2, 1024, 1152, False), (2, 1024, 1152, True), (1, 16384, 2240, True),
+                                           (3, 77, 96, True)])
+def test_litela_pre_relu_rotary_runs_in_the_kernels(cuda, caplog, B, N, C, qk_norm):
+    """LiteLA with image_rotary_emb: RMSNorm, the real-valued rotation before the ReLU and the ReLU happen on load in
+    the two attention kernels (no stock-op pass over the qkv buffer is logged), within the attention tolerance of the
+    oracle module in fp64 on the same bf16 weights and inputs."""
+    import logging
+    om, hm = make("LiteLA", C, qk_norm, seed=N + C)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(5)).bfloat16()
+    cos, sin = real_tables(N, 7)
+    with torch.no_grad():
+        ref = ref64(om, x, rotary_emb=(cos.double(), sin.double()))
+        S.modules._stock_paths_seen.clear()
+        with caplog.at_level(logging.WARNING, logger="sana_amd"):
+            out = hm(x.to(cuda), rotary_emb=(cos.to(cuda), sin.to(cuda)))
+    assert not [r for r in caplog.records if "LiteLA" in r.getMessage()], [r.getMessage() for r in caplog.records]
+    check(out, ref, f"LiteLA pre-ReLU rotary, qk_norm={qk_norm}")
+
+
+def test_litela_pre_relu_rotary_state_and_output_against_explicit_rotation(cuda):
+    """The kernels' rotate-first order against the same kernels WITHOUT transforms on explicitly rotated inputs
+    (rotation in fp32 with the fmas of the kernel, rounded to bf16): the vk block of the state is bit-identical (same
+    MFMA operands, same order), its ksum row and the output agree to fp32 summation order.  A rotation pins what the
+    order means: rotating AFTER the ReLU (the LiteLAReLURope order) on the same inputs gives another state."""
+    B, N, h = 2, 1000, 6
+    C = 32 * h
+    g = torch.Generator().manual_seed(3)
+    q, k, v = ((torch.randn(B, N, C, generator=g) * 1.3).bfloat16().to(cuda) for _ in range(3))
+    cos, sin = real_tables(N, 11)
+    table = ops.rope_table_real(cos, sin, N, cuda)
+    assert table is not None and tuple(table.shape) == (N, 16, 2)
+    assert ops.rope_table_real(*real_tables(N, 11, pair_equal=False), N, cuda) is None
+
+    def rotate(t):
+        x = t.float().view(B, N, h, 16, 2)
+        c, s = table[None, :, None, :, 0], table[None, :, None, :, 1]
+        x0, x1 = x[..., 0], x[..., 1]
+        r0 = torch.addcmul(-(x1 * s), x0, c)      # fma(x0, c, -(x1 * s))
+        r1 = torch.addcmul(x1 * c, x0, s)         # fma(x0, s, x1 * c)
+        return torch.stack([r0, r1], dim=-1).view(B, N, C).bfloat16()
+
+    pre = ops.QkPre(rope=table, rope_first=True)
+    st = ops.linattn_state(k, v, pre=pre)
+    st_ref = ops.linattn_state(rotate(k), v)
+    # fma contraction on the host may differ from the kernel's in the last fp32 bit of a rotated value, which can flip
+    # its bf16 rounding: compare the states at the level of a few such flips
+    assert rel_l2(st[:, :, :, :32], st_ref[:, :, :, :32]) <= 2e-4
+    assert rel_l2(st[:, :, :, 32:], st_ref[:, :, :, 32:]) <= 2e-4
+    out = ops.linattn_apply(q, st_ref, 1e-8, pre=pre)
+    out_ref = ops.linattn_apply(rotate(q), st_ref, 1e-8)
+    assert rel_l2(out, out_ref) <= 2e-3 and (out.float() - out_ref.float()).abs().max().item() <= 2e-2
+    st_after = ops.linattn_state(k, v, pre=ops.QkPre(rope=table))           # ReLU first, then the rotation
+    assert rel_l2(st_after[:, :, :, :32], st_ref[:, :, :, :32]) > 0.1
+
+
+def test_litela_rotary_tables_without_pair_structure_take_the_stock_pass(cuda, caplog):
+    """cos / sin tables whose two entries per channel pair differ are no rotation of the pair: the module applies them
+    with stock ops on the qkv buffer (logged) and still matches the oracle."""
+    import logging
+    B, N, C = 2, 200, 96
+    om, hm = make("LiteLA", C, True, seed=9)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(5)).bfloat16()
+    cos, sin = real_tables(N, 7, pair_equal=False)
+    with torch.no_grad():
+        ref = ref64(om, x, rotary_emb=(cos.double(), sin.double()))
+        S.modules._stock_paths_seen.clear()
+        with caplog.at_level(logging.WARNING, logger="sana_amd"):
+            out = hm(x.to(cuda), rotary_emb=(cos.to(cuda), sin.to(cuda)))
+    assert any("LiteLA rotary embedding" in r.getMessage() for r in caplog.records)
+    check(out, ref, "LiteLA generic real tables")
