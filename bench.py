@@ -403,15 +403,21 @@ def chain_step(blocks, cond, x, y, t, HW):
     return h
 
 
-def images_per_s(dev, blocks, steps: int, warmup: int, B: int = 16) -> float:
-    """1024px shape of Sana-1.6B: B images of N=1024 tokens; the DEPTH DiT blocks of one denoising step only."""
+def images_per_s(dev, blocks, steps: int, warmup: int, B: int = 16, graphed: bool = False) -> float:
+    """1024px shape of Sana-1.6B: B images of N=1024 tokens; the DEPTH DiT blocks of one denoising step only.
+    ``graphed``: the step's launches replayed from one captured HIP graph (sana_amd.GraphedCall) instead of being
+    issued from Python."""
     import sana_amd as S
 
     HW = (32, 32)
     cond = S.StepConditioning(blocks)
     x, y, t = (a.bfloat16().to(dev) for a in make_inputs(B, HW[0] * HW[1]))
     with torch.no_grad():
-        t_us = event_time_us(lambda: chain_step(blocks, cond, x, y, t, HW), steps, warmup)
+        if graphed:
+            step = S.GraphedCall(lambda a, b, c: chain_step(blocks, cond, a, b, c, HW), (x, y, t))
+            t_us = event_time_us(lambda: step(x, y, t), steps, warmup)
+        else:
+            t_us = event_time_us(lambda: chain_step(blocks, cond, x, y, t, HW), steps, warmup)
     return B / (t_us * 1e-6)
 
 
@@ -677,6 +683,7 @@ def main():
         kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev, stock_conv=args.stock_conv)
         ips_bf16 = images_per_s(dev, blocks, 5, 2)
         one_image_ms = 1e3 / images_per_s(dev, blocks, 20, 5, B=1)   # 20 blocks on one image: latency, not throughput
+        one_image_ms_graph = 1e3 / images_per_s(dev, blocks, 20, 5, B=1, graphed=True)
         del cond, blocks
         blocks = make_blocks(dev, w8=True)
         ips_w8 = images_per_s(dev, blocks, 5, 2)
@@ -700,10 +707,11 @@ def main():
                                "C=2240, 70x32 heads, Mix-FFN hidden 5600, 300 text tokens, random init"},
         "images_per_s_1024px": {"bf16": round(ips_bf16, 2), "w8a16": round(ips_w8, 2),
                                 "one_image_step_ms_bf16": round(one_image_ms, 3),
+                                "one_image_step_ms_bf16_hip_graph": round(one_image_ms_graph, 3),
                                 "one_image_step_ms_w8a16": round(one_image_ms_w8, 3),
                                 "note": "B=16, N=1024: B / time of the 20 chained blocks; DiT blocks of one denoising step only "
                                         "(no text encoder, VAE, embedders, step count or CFG doubling); "
-                                        "one_image_step_ms: the same 20 blocks at B=1"},
+                                        "one_image_step_ms: the same 20 blocks at B=1 (hip_graph: replayed from one captured HIP graph)"},
         "video_block_ms": {"value": round(video_ms, 3),
                            "note": "one SanaVideoMSBlock forward, bf16: N=21x30x52=32760 tokens, C=2240, 20 heads of 112, "
                                    "q/k RMSNorm + rotary embedding, chunk_index [0, 11], ChunkGLUMBConvTemp, 300 text tokens"},

@@ -361,13 +361,23 @@ __global__ __launch_bounds__(64 * NW, 16 / NW) void dwconv_gate16_lds_kernel(con
   const __amdgpu_buffer_rsrc_t rsrc_y = __builtin_amdgcn_make_buffer_rsrc(
       static_cast<char*>(y) + (int64_t)slab * 128 * ESZ + img * Ch * ESZ, 0, H * W * opix_b - slab * 128 * ESZ, 0x00020000);
   const unsigned char* my = ring + (4 * wave) * DWL_PIXB + lane_b;        // this wave's first footprint pixel, this lane's pair
+  // The ring is read with asm loads: to the compiler an ordinary LDS read may alias the LDS-writing global loads
+  // still in flight (the next group's), and it would wait for ALL of them (vmcnt(0)) in front of the first read --
+  // which empties the ring at every group.  Which loads must have landed is this kernel's own business (the counted
+  // waits and barriers of the main loop); the wait for the reads themselves is tied to their results below.
+  const uint32_t my_lds = (uint32_t)(size_t)(__attribute__((address_space(3))) const unsigned char*)my;
   auto take_row = [&](int slot, uint32_t (&row)[TW + 1][4]) {
     uint32_t ra[TW + 2], rg[TW + 2];
+    const uint32_t base = my_lds + slot * DWL_ROWB;
 #pragma unroll
     for (int i = 0; i < TW + 2; ++i) {
-      ra[i] = *reinterpret_cast<const uint32_t*>(my + slot * DWL_ROWB + i * DWL_PIXB);
-      rg[i] = *reinterpret_cast<const uint32_t*>(my + slot * DWL_ROWB + i * DWL_PIXB + 256);
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(ra[i]) : "v"(base), "n"(i * DWL_PIXB));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(rg[i]) : "v"(base), "n"(i * DWL_PIXB + 256));
     }
+    static_assert(TW + 2 == 6, "the wait below names the six pixels of a row");
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(ra[0]), "+v"(ra[1]), "+v"(ra[2]), "+v"(ra[3]), "+v"(ra[4]), "+v"(ra[5]), "+v"(rg[0]), "+v"(rg[1]),
+                   "+v"(rg[2]), "+v"(rg[3]), "+v"(rg[4]), "+v"(rg[5]));
 #pragma unroll
     for (int i = 0; i < TW + 1; ++i) {
       row[i][0] = __builtin_amdgcn_perm(ra[i + 1], ra[i], 0x05040100u);
@@ -424,7 +434,8 @@ __global__ __launch_bounds__(64 * NW, 16 / NW) void dwconv_gate16_lds_kernel(con
       if (g + 1 >= NGRP) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       else if (wave < NFULL) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PMAX) : "memory");
       else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PMAX - 1) : "memory");
-      __syncthreads();                                                     // and so have everyone else's
+      __builtin_amdgcn_s_barrier();                                        // and so have everyone else's (no fence: the
+                                                                           // next group's loads stay in flight)
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
         const int t = 2 * g + r;
@@ -434,7 +445,7 @@ __global__ __launch_bounds__(64 * NW, 16 / NW) void dwconv_gate16_lds_kernel(con
           if (t >= 2 && wave_ok) compute(y0 + t - 2, win[(s3 + 1) % 3], win[(s3 + 2) % 3], win[s3]);
         }
       }
-      __syncthreads();  // every wave has taken the group's rows: its slots may be refilled
+      __builtin_amdgcn_s_barrier();  // every wave has taken the group's rows (its reads are waited for): the slots may be refilled
       if (g + 2 < NGRP) issue_group(g + 2);
     }
   }

@@ -13,6 +13,9 @@
 //            of the state (two bf16 terms of the fp32 values as MFMA 16x16x32 A operands for bf16 output,
 //            three for fp32 output) plus a row block that carries ksum in every row, so each lane gets
 //            its token's denominator.
+#include <algorithm>
+#include <type_traits>
+
 #include "common.h"
 #include "linattn_common.h"
 
@@ -24,289 +27,528 @@ constexpr int SE = (DH + 1) * DH;       // 12656 state elements per (batch, head
 constexpr int NCH = DH / 8;             // 14 16-byte chunks per token and head
 constexpr int TILE = 32;
 
-// Workgroup index -> (unit of four adjacent heads, head within it).  Four 224-byte head rows are seven whole
-// 128-byte lines; a single head's row shares its first / last line with a neighbour.  Workgroup i runs on XCD
-// i % 8, so the four heads of a unit take consecutive slots of ONE XCD: the shared lines are then fetched into
-// one L2, once, instead of into two.  Returns false for the padding of the grid.
+// Workgroup index -> (unit, head).  Heads are taken four at a time: four 224-byte head rows are seven whole
+// 128-byte lines, while a single head's row shares its first / last line with a neighbour.  Workgroup i runs on
+// XCD i % 8, each XCD has its own L2: the (unit, head group) pairs are cut into 8 contiguous blocks, one per XCD,
+// and the four heads of a group take consecutive slots of the XCD.  Shared lines are then fetched into one L2,
+// once, and so is what all heads of a unit read alike (the tokens' rotary factors, 1 / rms): a unit's head groups
+// sit on one XCD, two where a block boundary cuts through.  Returns false for the padding of the grid.
 struct HeadUnit {
   int unit, head;
 };
+// a wave-uniform value into a scalar register, whatever the compiler thinks of it (integer division runs on the
+// vector unit and its result, and all that is derived from it -- buffer resources, loop bounds -- would otherwise
+// be handled as per-lane data)
+__device__ __forceinline__ int uniform(int x) {
+  int r;
+  asm volatile("s_mov_b32 %0, %1" : "=s"(r) : "s"(x));
+  return r;
+}
 __device__ __forceinline__ bool head_unit(int idx, int units, int h, HeadUnit& u) {
   const int xcd = idx & 7, slot = idx >> 3;
   const int hgroups = (h + 3) >> 2;
-  const int un = (slot >> 2) * 8 + xcd;
-  u.unit = un / hgroups;
+  const int total = units * hgroups;
+  const int un = (xcd * total) / 8 + (slot >> 2);
+  u.unit = uniform(un / hgroups);
   u.head = (un - u.unit * hgroups) * 4 + (slot & 3);
-  return un < units * hgroups && u.head < h;
+  return un < ((xcd + 1) * total) / 8 && u.head < h;
 }
-inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) / 4) + 7) / 8 * 8 * 4; }
+inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) / 4) + 7) / 8 * 8 * 4; }  // 8 x 4 x the largest block
 
 // ----------------------------------------------------------------------------
-// phase 1.  1-D grid over units (batch, chunk, token split) x heads, see head_unit; block 256.
-// partial[(bh * n_chunks + c) * nsplit + split][SE]
+// phase 1.  grid.x over token ranges x heads, see head_unit, grid.y = batch; block 512 = eight waves.
+//
+// A workgroup walks ONE contiguous token range of a (batch, head) -- ranges are cut by token count, not by chunk,
+// so every workgroup has the same work whatever the chunking -- in tiles of 32 tokens that never straddle a chunk
+// boundary, and writes one record (113 x 112 fp32) per chunk its range touches:
+//   record[(bh * n_chunks + c) * nslot + (range - first range touching c)]
+// reduce112_kernel adds a chunk's records in range order (and runs the prefix over chunks when causal).
+//
+// Everything a tile needs comes global -> LDS by direct loads (`buffer_load_dwordx4 ... lds`, 16 bytes per lane,
+// no staging registers) into rings: K and V rows of the head (224 bytes = 14 pieces, stored back to back: a row
+// stride of 56 banks makes the transposing operand reads below conflict free as it is, and every lane of every load
+// instruction carries data) and the tokens' 1 / rms in a ring of NKV stages, the tokens' rotary factors (448
+// bytes) in a ring of NKV - 1.  Tokens past the tile's limit (the chunk or range end) are loaded through an offset
+// outside the buffer resource, i.e. as zeros: they add nothing.  The bytes in flight per compute unit are what
+// the rings hold, independent of registers.
+//
+// The state is 8 x 8 tiles of v_mfma_f32_16x16x32 (113 x 112 padded to 128 x 128); wave w < 4 owns rows (dv)
+// [64 (w & 1), + 64) x columns (dk) [64 (w >> 1), + 64): 4 x 4 accumulator tiles, 8 operands per tile of tokens
+// (the LDS operand traffic, which runs at half the plain read rate, is what the split minimises), no cross-wave
+// reduction.  The operands are read from the token-major stage with ds_read_b64_tr_b16 (a 16-lane
+// group reads a 4-token x 16-channel block and every lane receives the 4 tokens of ONE channel -- the transpose
+// the contraction over tokens needs -- 2 instructions per operand quad).  Row block and column block 112..127 are
+// padding and never read from LDS: the column block's operand is zero, the row block's A operand is a constant
+// (row 0 all ones), so its accumulator row 0 is sum_n relu(k_n) = row 112 of the state, the "1" column the
+// reference pads onto V.
+//
+// One barrier per tile.  Between two barriers every wave refills the ring entries consumed a tile ago, waves 0..3
+// read the operands of tile i and run its MFMAs, and with on-load transforms (q/k RMSNorm, rotary embedding) waves
+// 4..7 rewrite the K rows of tile i + 1 in place (16-byte pieces, two per thread): transform arithmetic and MFMA
+// operand traffic of consecutive tiles run side by side in different waves.  With a rotary embedding the MFMA
+// operands are rotated and ksum must not be, so it is accumulated per thread in the transform and folded through
+// the tile's own (consumed) rotary slot when a chunk ends.
 // ----------------------------------------------------------------------------
-constexpr int LR = 160;  // LDS tile row stride in elements: 320 B puts the two token groups of a read 16 banks apart
-constexpr int SMEM_BYTES = 2 * 128 * 128 * 4;  // two padded fp32 accumulator images for the wave reduction
-                                             // (>= 4 waves x 2 tiles x 33 x LR x 2 B of staging)
-static_assert(SMEM_BYTES >= 4 * 2 * (TILE + 1) * LR * 2, "staging must fit");
+constexpr int S2_ROW = NCH * 16;                // bytes per token row of K / V in a stage
+constexpr int S2_KV = 2 * TILE * S2_ROW;        // K rows, then V rows: 14336 bytes
+constexpr int S2_ROPE = TILE * DH * 4;          // rotary factors of a tile: 14336 bytes
+template <int PRE>
+struct Stage2 {
+  static constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
+  static constexpr int kv_bytes = S2_KV + (has_norm ? 1024 : 0);  // (a load instruction always fills 64 slots)
+  static constexpr int n_kv = 2 * TILE * NCH / 64, n_rope = has_rope ? TILE * 28 / 64 : 0;   // load instructions: 14, 14
+  static constexpr int n_instr = n_kv + n_rope + (has_norm ? 1 : 0);
+  static constexpr int NKV = 6;   // ring depth (measured: 4 .. 10 make no difference, the kernel is not bound by latency)
+  static constexpr int NR = has_rope ? NKV - 1 : 0;
+  static constexpr int bytes = NKV * kv_bytes + NR * S2_ROPE;
+  static constexpr int per_wave = (n_instr + 3) / 4;   // load instructions per tile of issuing waves < n_instr % 4; the others one less
+  static_assert(bytes <= 160 * 1024, "LDS");
+  static_assert((NKV - 2) * per_wave < 64, "vmcnt range");
+};
 
-// PRE: on-load transforms, compile-time so that the tile code stays one branch-free block: bit 0 = q/k RMSNorm,
-// bit 1 = rotary embedding
+template <typename T>
+__device__ __forceinline__ f32x4_t mfma16(u32x4_t a, u32x4_t b, f32x4_t c) {
+  if constexpr (is_f16<T>)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return mfma_16x16x32_bf16(a, b, c);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// The rings are read with asm statements: to the compiler an ordinary LDS read may alias the LDS-writing global
+// loads still in flight (the stages further down the ring) and it would wait for ALL of them (vmcnt(0)) in front of
+// the first read, which would empty the ring at every tile.  Which loads must have landed is the kernel's own
+// business (counted waits + barriers); the waits for the LDS reads themselves are tied to their results.
+// addr: LDS byte address, OFF: immediate byte offset.
+//
+// read_tr16: 4 tokens x 16 channels of a token-major tile -> this lane's channel, 4 tokens; addr points at the
+// lane's 4-channel segment of its token
+template <int OFF>
+__device__ __forceinline__ u32x2_t read_tr16(uint32_t addr) {
+  u32x2_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read128(uint32_t addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+__device__ __forceinline__ float lds_read32(uint32_t addr) {
+  float v;
+  asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write128(uint32_t addr, u32x4_t v) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(size_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+struct TileCur {  // walks the tiles of a token range: 32 tokens at a time, never across a chunk boundary
+  int t, c, seg_end;
+};
+struct Tile112 {
+  int start, limit, c;
+  bool last;  // of its chunk within the range
+};
+struct Ops112 {  // MFMA operands of one tile of tokens: [operand][token half]
+  u32x2_t v[4][2], k[4][2];
+};
+
 template <typename T, int PRE>
-__global__ __launch_bounds__(256) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
+__global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
                                                        float* __restrict__ partial,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int nsplit, int split_tokens, int units,
-                                                       int64_t stride_b, int64_t stride_n, const QkPre pre) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+                                                       int n_chunks, int nslot, int range_tokens, int units,
+                                                       int nranges, int64_t stride_b, int64_t stride_n, const QkPre pre) {
+  typedef Stage2<PRE> ST;
+  constexpr bool has_norm = ST::has_norm, has_rope = ST::has_rope;
+  constexpr int NKV = ST::NKV, NR = ST::NR;
+  constexpr int AHEAD = PRE ? 1 : 0;  // the transform works one tile ahead of the operand reads
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[ST::bytes];
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   HeadUnit hu;
   if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
   const int head = hu.head;
-  const int split = hu.unit % nsplit, c = (hu.unit / nsplit) % n_chunks, b = hu.unit / (nsplit * n_chunks);
-  const ChunkRange cr = chunk_range(chunk_starts, c, N);
-  const int t0 = cr.begin + split * split_tokens;
-  const int t1 = min(cr.end, t0 + split_tokens);
-  // tokens per tile: 32, or 16 with transforms (their operands -- rotary factors above all -- travel with the
-  // tile, and a 32-token tile of them does not fit the registers next to the accumulator)
-  constexpr int TT_ = PRE ? 16 : TILE;
-  constexpr int TROWS = TT_ + 1;  // one spare row per tile: where the idle lanes of the transform mapping write
-  uint16_t* lds_k = reinterpret_cast<uint16_t*>(smem) + wave * (2 * TROWS * LR);
-  uint16_t* lds_v = lds_k + TROWS * LR;
-  // channels 112..127 of every tile row are written once, as zeros, and never again
-  for (int i = lane; i < 2 * TROWS * 2; i += 64) {  // (K rows, V rows) x 2 chunks of 8
-    const int row = i >> 1, chunk = NCH + (i & 1);
-    *reinterpret_cast<u32x4_t*>(lds_k + row * LR + chunk * 8) = u32x4_t{0u, 0u, 0u, 0u};
-  }
+  const int rg = hu.unit, b = blockIdx.y;
+  const int r0 = rg * range_tokens, r1 = min(N, r0 + range_tokens);
+  if (r0 >= r1) return;
+  auto chunk_end = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c + 1] : N; };
+  auto chunk_begin = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c] : 0; };
+  int c0 = 0;
+  while (chunk_end(c0) <= r0) ++c0;  // the chunk of the range's first token (uniform; a few dozen chunks at most)
+  const uint32_t smem_addr = lds_addr(smem);
+  const uint32_t rope_ring = smem_addr + NKV * ST::kv_bytes;
 
-  // load mapping, consecutive lanes on consecutive 16-byte pieces of a token's 224-byte head row:
-  //   plain      piece id = lane + 64 i (i < 7): token id / 14, piece id % 14
-  //   transforms lanes 0..55: token 4 i + lane / 14 (i < 4), piece lane % 14 -- a lane keeps ONE piece, so its norm
-  //              weights are loop invariant and its ksum is 8 registers; the other 8 lanes load nothing (zeros)
-  //              and write them to the spare row
-  constexpr int NSLOT = PRE ? 4 : 7;
-  const bool lane_ok = !PRE || lane < 4 * NCH;
-  int ld_tok[NSLOT], ld_ch[NSLOT];
+  // ---- global -> LDS.  Load instruction q of a tile fills slots [64 q', 64 q' + 64) of 16 bytes of its ring entry;
+  // wave w < 4 issues q = w, w + 4, ... (a wave that issues loads stalls while the memory pipeline is full, which
+  // in a kernel bound by memory is most of the time: the waves that run the transforms must not be among them).
+  // Slots: K rows (32 x 14), V rows (32 x 14), 1 / rms (8) | rotary factors (32 x 28)
+  const int row_b = (int)stride_n * 2;
+  const int64_t tok_bytes = (int64_t)N * stride_n * 2;
+  const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(K + (int64_t)b * stride_b + head * DH), 0, (int)(tok_bytes - (int64_t)head * DH * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(V + (int64_t)b * stride_b + head * DH), 0, (int)(tok_bytes - (int64_t)head * DH * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(has_norm ? pre.rinv + (int64_t)b * N : nullptr), 0, has_norm ? N * 4 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(pre.rope), 0, has_rope ? N * (DH * 4) : 0, 0x00020000);
+  const int idle = (int)0x80000000u;
+  // per load instruction of this wave: token row (within the tile) of the lane's slot and its byte offset from the
+  // tile's first token
+  int ld_row[ST::per_wave], ld_off[ST::per_wave];
 #pragma unroll
-  for (int i = 0; i < NSLOT; ++i) {
-    const int id = PRE ? 4 * NCH * i + lane : lane + 64 * i;
-    ld_tok[i] = lane_ok ? id / NCH : TT_;
-    ld_ch[i] = lane_ok ? id - (id / NCH) * NCH : lane - 4 * NCH;
+  for (int j = 0; j < ST::per_wave; ++j) {
+    const int q = wave + 4 * j;
+    ld_row[j] = 0;
+    ld_off[j] = idle;
+    if (q < ST::n_kv) {
+      const int s = (q % (ST::n_kv / 2)) * 64 + lane, row = s / NCH, col = s - row * NCH;
+      ld_row[j] = row;
+      ld_off[j] = row * row_b + col * 16;
+    } else if (q < ST::n_kv + ST::n_rope) {
+      const int s = (q - ST::n_kv) * 64 + lane;  // the tile's factors are one contiguous run
+      ld_row[j] = s / 28;
+      ld_off[j] = s * 16;
+    } else if (q < ST::n_instr) {  // 1 / rms: 8 pieces of 4 tokens
+      ld_row[j] = 0;   // (tokens past the limit read whatever statistic is there, or zero past the tensor: their K rows are zeros)
+      ld_off[j] = lane < 8 ? lane * 16 : idle;
+    }
   }
-  const uint16_t* kbase = K + (int64_t)b * stride_b + head * DH;
-  const uint16_t* vbase = V + (int64_t)b * stride_b + head * DH;
-  constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
+  int issued = 0;  // tiles whose loads have been issued; tile t lives in K/V stage t % NKV and rotary slot t % NR
+  auto issue = [&](int start, int limit) __attribute__((always_inline)) {
+    if (wave >= 4) {
+      ++issued;
+      return;
+    }
+    unsigned char* kvb = smem + (issued % NKV) * ST::kv_bytes;
+    unsigned char* rpb = smem + NKV * ST::kv_bytes + (has_rope ? (issued % (NR ? NR : 1)) * S2_ROPE : 0);
+#pragma unroll
+    for (int j = 0; j < ST::per_wave; ++j) {
+      const int q = wave + 4 * j;  // wave-uniform
+      if (q >= ST::n_instr) break;
+      // the tile's first token goes into the scalar offset, the lane's part is constant; rows past the limit and
+      // idle lanes get an offset outside the resource
+      const int voff = ld_row[j] < limit - start ? ld_off[j] : idle;
+      if (q < ST::n_kv) {
+        auto dst = (__attribute__((address_space(3))) void*)(kvb + q * 1024);
+        if (q < ST::n_kv / 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, dst, 16, voff, start * row_b, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, dst, 16, voff, start * row_b, 0, 0);
+      } else if (q < ST::n_kv + ST::n_rope) {
+        auto dst = (__attribute__((address_space(3))) void*)(rpb + (q - ST::n_kv) * 1024);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_c, dst, 16, voff, start * (DH * 4), 0, 0);
+      } else {
+        auto dst = (__attribute__((address_space(3))) void*)(kvb + S2_KV);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_r, dst, 16, voff, start * 4, 0, 0);
+      }
+    }
+    ++issued;
+  };
+  const bool more_loads = ST::n_instr % 4 == 0 || wave < ST::n_instr % 4;  // this wave issues per_wave loads per tile
+  // waits until this wave's loads of all but the `keep` youngest tiles have landed; `keep` as a template argument
+  // when it is the steady-state figure, everything otherwise (prologue and tail of short ranges)
+  auto wait_tiles = [&](auto keep_c, int keep) __attribute__((always_inline)) {
+    constexpr int KEEP = decltype(keep_c)::value;
+    if (wave >= 4) return;  // nothing of its own in flight
+    if (keep == KEEP) {
+      if (more_loads) wait_vmcnt<KEEP * ST::per_wave>();
+      else wait_vmcnt<KEEP * (ST::per_wave - 1)>();
+    } else {
+      wait_vmcnt<0>();
+    }
+  };
 
-  f32x16_t acc[4][4];
+  auto has_tile = [&](const TileCur& cur) __attribute__((always_inline)) { return cur.t < r1; };
+  auto next_tile = [&](TileCur& cur) __attribute__((always_inline)) {
+    Tile112 tl;
+    tl.start = cur.t;
+    tl.limit = cur.seg_end;
+    tl.c = cur.c;
+    const int nt = min(cur.t + TILE, cur.seg_end);
+    tl.last = nt == cur.seg_end;
+    cur.t = nt;
+    if (tl.last && nt < r1) {
+      ++cur.c;
+      cur.seg_end = min(chunk_end(cur.c), r1);
+    }
+    return tl;
+  };
+  TileCur icur = {r0, c0, min(chunk_end(c0), r1)}, ccur = icur, tcur = icur;
+#pragma unroll 1
+  for (int i = 0; i < NKV - 1 && has_tile(icur); ++i) {
+    const Tile112 tl = next_tile(icur);
+    issue(tl.start, tl.limit);
+  }
+  auto record_of = [&](int c) __attribute__((always_inline)) {
+    const int first = uniform(chunk_begin(c) / range_tokens);  // first range touching the chunk
+    const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nslot + (rg - first);
+    return partial + slot * SE;
+  };
+
+  // ---- roles.  Waves 0..3 run the MFMAs, waves 4..7 the transforms; all eight issue loads.
+  const bool mma_role = wave < 4;  // wave-uniform
+
+  // ---- transform side: 16-byte piece i of a tile = piece i % 14 of token i / 14; thread tid - 256 takes pieces
+  // tid - 256 and tid (the second one exists for tid < 448)
+  const int tq = tid - 256;
+  bool tp_ok[2];
+  int tp_tok[2];
+  u32x4_t kw[2];
+  float ks8[2][8];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = tq + 256 * u;
+    tp_ok[u] = PRE && !mma_role && i < TILE * NCH;
+    tp_tok[u] = i / NCH;
+    kw[u] = u32x4_t{0u, 0u, 0u, 0u};
+    if (has_norm && tp_ok[u]) kw[u] = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + (i - tp_tok[u] * NCH) * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ks8[u][e] = 0.f;
+  }
+  int tdone = 0;  // tiles transformed
+  // Rewrites the K rows of the next tile of the transform cursor in place; all of its loads have landed and nobody
+  // else touches it before the next barrier.  Every wave calls it (the cursor and the barrier of the ksum fold are
+  // workgroup business), the transform waves do the work.
+  auto transform_next = [&]() __attribute__((always_inline)) {
+    const Tile112 tl = next_tile(tcur);
+    const uint32_t sa = smem_addr + (tdone % NKV) * ST::kv_bytes;
+    const uint32_t ra = rope_ring + (has_rope ? (tdone % (NR ? NR : 1)) * S2_ROPE : 0);
+    if (!mma_role) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {  // (one piece after the other: the registers of both at once do not fit)
+        if (!tp_ok[u]) continue;
+        const int i = tq + 256 * u;
+        u32x4_t x = lds_read128<0>(sa + i * 16);
+        float rin = 0.f;
+        f32x4_t cs0 = {0.f, 0.f, 0.f, 0.f}, cs1 = cs0;
+        if (has_norm) rin = lds_read32(sa + S2_KV + tp_tok[u] * 4);
+        if (has_rope) {
+          cs0 = __builtin_bit_cast(f32x4_t, lds_read128<0>(ra + i * 32));
+          cs1 = __builtin_bit_cast(f32x4_t, lds_read128<16>(ra + i * 32));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x), "+v"(rin), "+v"(cs0), "+v"(cs1));
+        if (has_norm) x = rms_scale8(x, rin, kw[u]);
+        x = relu_pk16(x);
+        if (has_rope) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ks8[u][2 * e] += bf16_lo(x[e]);
+            ks8[u][2 * e + 1] += bf16_hi(x[e]);
+          }
+          x = rope8(x, cs0, cs1);
+        }
+        lds_write128<0>(sa + i * 16, x);
+      }
+    }
+    if (has_rope && tl.last) {  // uniform: a chunk (or the range) ends with this tile: its ksum row
+      // fold area = the tile's rotary slot: every thread overwrites exactly the bytes it alone has read
+      if (!mma_role) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          if (!tp_ok[u]) continue;
+          const uint32_t fa = ra + (tq + 256 * u) * 32;
+          lds_write128<0>(fa, __builtin_bit_cast(u32x4_t, f32x4_t{ks8[u][0], ks8[u][1], ks8[u][2], ks8[u][3]}));
+          lds_write128<16>(fa, __builtin_bit_cast(u32x4_t, f32x4_t{ks8[u][4], ks8[u][5], ks8[u][6], ks8[u][7]}));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ks8[u][e] = 0.f;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      if (tq >= 0 && tq < DH) {  // channel tq: piece tq / 8 of the 32 tokens
+        const float* fold = reinterpret_cast<const float*>(smem + NKV * ST::kv_bytes + (tdone % (NR ? NR : 1)) * S2_ROPE);
+        const int p = tq >> 3, e = tq & 7;
+        float sum = 0.f;
+#pragma unroll 4
+        for (int tk = 0; tk < TILE; ++tk) sum += fold[(tk * NCH + p) * 8 + e];
+        record_of(tl.c)[DH * DH + tq] = sum;
+        // stores share the counter the rings wait on (and need not retire in order with the loads)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+    }
+    ++tdone;
+  };
+
+  // ---- MFMA side: lane = 16 g + R; tokens 16 hh + 4 g + R / 4 (hh = 0, 1) are this lane group's 8 contraction
+  // slots; both operands use the same map.  Wave w < 4: rows (dv) [64 (w & 1), + 64) x columns (dk) [64 (w >> 1), + 64)
+  const int g = lane >> 4, R = lane & 15;
+  const int dvh = wave & 1, dkh = (wave >> 1) & 1;   // wave-uniform
+  const bool v3_real = dvh == 0, k3_real = dkh == 0;  // row block 112..127 / column block 112..127 are padding
+  f32x4_t acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int tr_off = (4 * g + (R >> 2)) * S2_ROW + (R & 3) * 8;
+  const uint32_t v_off = TILE * S2_ROW + tr_off + dvh * 128, k_off = tr_off + dkh * 128;
+  const uint32_t one2 = is_f16<T> ? 0x3c003c00u : 0x3f803f80u;
+  const u32x2_t ones2 = R == 0 ? u32x2_t{one2, one2} : u32x2_t{0u, 0u};
+  auto read_ops = [&](int tile, Ops112& o) __attribute__((always_inline)) {
+    const uint32_t sa = smem_addr + (tile % NKV) * ST::kv_bytes;
+    const uint32_t vb = sa + v_off, kb = sa + k_off;
+    o.v[0][0] = read_tr16<0>(vb), o.v[0][1] = read_tr16<16 * S2_ROW>(vb);
+    o.v[1][0] = read_tr16<32>(vb), o.v[1][1] = read_tr16<32 + 16 * S2_ROW>(vb);
+    o.v[2][0] = read_tr16<64>(vb), o.v[2][1] = read_tr16<64 + 16 * S2_ROW>(vb);
+    if (v3_real) o.v[3][0] = read_tr16<96>(vb), o.v[3][1] = read_tr16<96 + 16 * S2_ROW>(vb);
+    else o.v[3][0] = o.v[3][1] = ones2;
+    o.k[0][0] = read_tr16<0>(kb), o.k[0][1] = read_tr16<16 * S2_ROW>(kb);
+    o.k[1][0] = read_tr16<32>(kb), o.k[1][1] = read_tr16<32 + 16 * S2_ROW>(kb);
+    o.k[2][0] = read_tr16<64>(kb), o.k[2][1] = read_tr16<64 + 16 * S2_ROW>(kb);
+    if (k3_real) o.k[3][0] = read_tr16<96>(kb), o.k[3][1] = read_tr16<96 + 16 * S2_ROW>(kb);
+    else o.k[3][0] = o.k[3][1] = u32x2_t{0u, 0u};
+  };
+  auto wait_ops = [&](Ops112& o) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(o.v[0][0]), "+v"(o.v[0][1]), "+v"(o.v[1][0]), "+v"(o.v[1][1]), "+v"(o.v[2][0]), "+v"(o.v[2][1]),
+                   "+v"(o.v[3][0]), "+v"(o.v[3][1]), "+v"(o.k[0][0]), "+v"(o.k[0][1]), "+v"(o.k[1][0]), "+v"(o.k[1][1]),
+                   "+v"(o.k[2][0]), "+v"(o.k[2][1]), "+v"(o.k[3][0]), "+v"(o.k[3][1])
+                 :
+                 : "memory");
+    if (!PRE) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  float acck[4] = {0.f, 0.f, 0.f, 0.f};  // ksum of channel 32 jb + lane % 32 over this lane's token half
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  // The next tile's loads (and what its transforms need: 1/rms, rotary factors) are in flight during the MFMAs
-  // of the current one.  (A second register set, two tiles ahead, measured no faster.)
-  u32x4_t kreg[NSLOT], vreg[NSLOT];
-  float rin[has_norm ? NSLOT : 1];
-  f32x4_t cs[has_rope ? NSLOT : 1][2];
-  u32x4_t kw = zero4;
-  if (has_norm && lane_ok) kw = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[0] * 8);
-  // Buffer loads: a resource ends with the last token of the range, so pieces of tokens past it (and everything
-  // of the idle lanes, whose offsets start at 2^31) read as zeros -- no branches or selects around the loads.
-  // The range check covers the vector offset only, so the tile's part of the address goes there.
-  const int row_b = (int)stride_n * 2;
-  const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(kbase), 0, (int)(((int64_t)(t1 - 1) * stride_n + DH) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(vbase), 0, (int)(((int64_t)(t1 - 1) * stride_n + DH) * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(has_norm ? pre.rinv + (int64_t)b * N : nullptr), 0, has_norm ? t1 * 4 : 0, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(pre.rope), 0, has_rope ? t1 * (DH * 4) : 0, 0x00020000);
-  const int idle = (int)0x80000000u;
-  int voff[NSLOT];
+      for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
-  for (int i = 0; i < NSLOT; ++i) voff[i] = lane_ok ? ld_tok[i] * row_b + ld_ch[i] * 16 : idle;
-  auto issue_loads = [&](int tile) {
-#pragma unroll
-    for (int i = 0; i < NSLOT; ++i) {
-      const int off = tile * row_b + voff[i];
-      kreg[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, off, 0, 0));
-      vreg[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, off, 0, 0));
-      if (PRE) {
-        const int tok = lane_ok ? tile + ld_tok[i] : idle / (DH * 4);
-        if (has_norm) rin[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_r, tok * 4, 0, 0));
-        if (has_rope) {
-          const int ro = tok * (DH * 4) + ld_ch[i] * 32;
-          cs[i][0] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_c, ro, 0, 0));
-          cs[i][1] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_c, ro + 16, 0, 0));
-        }
-      }
+        for (int hh = 0; hh < 2; ++hh) o.k[ct][hh] = u32x2_t{relu_pk16(o.k[ct][hh].x), relu_pk16(o.k[ct][hh].y)};
     }
   };
-  // PRE: the MFMA operands in LDS are rotated, ksum needs the unrotated values: a second, unrotated
-  // copy of the K tile would double the LDS traffic, so ksum is accumulated per lane and channel
-  // here and folded over the lanes that share a piece once at the end
-  float ks8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-  const int tile0 = t0 + wave * TT_;
-  if (tile0 < t1) issue_loads(tile0);
-  // operand read mapping: lane -> channel j = lane%32 of a 32-channel block, k-group g = lane/32;
-  // element r of k-step s is token 16*s + 2*r + g of the tile (both operands use the same bijection)
-  const int j = lane & 31, g = lane >> 5;
-  for (int tile = tile0; tile < t1; tile += 4 * TT_) {
+  auto mma = [&](const Ops112& o) __attribute__((always_inline)) {
+    u32x4_t fk[4];
 #pragma unroll
-    for (int i = 0; i < NSLOT; ++i) {
-      u32x4_t kk = kreg[i];
-      if (PRE) {
-        if (has_norm) kk = rms_scale8(kk, rin[i], kw);
-        kk = relu_pk16(kk);
+    for (int ct = 0; ct < 4; ++ct) fk[ct] = u32x4_t{o.k[ct][0].x, o.k[ct][0].y, o.k[ct][1].x, o.k[ct][1].y};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          ks8[2 * e] += bf16_lo(kk[e]);
-          ks8[2 * e + 1] += bf16_hi(kk[e]);
-        }
-        if (has_rope) kk = rope8(kk, cs[i][0], cs[i][1]);
-      } else {
-        kk = relu_pk16(kk);
-      }
-      *reinterpret_cast<u32x4_t*>(lds_k + ld_tok[i] * LR + ld_ch[i] * 8) = kk;
-      *reinterpret_cast<u32x4_t*>(lds_v + ld_tok[i] * LR + ld_ch[i] * 8) = vreg[i];
+    for (int rb = 0; rb < 4; ++rb) {
+      const u32x4_t fv = {o.v[rb][0].x, o.v[rb][0].y, o.v[rb][1].x, o.v[rb][1].y};
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) acc[rb][ct] = mfma16<T>(fv, fk[ct], acc[rb][ct]);  // (zero operand in the padding column block)
     }
-    if (tile + 4 * TT_ < t1) issue_loads(tile + 4 * TT_);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private LDS: in-order, no barrier needed
+  };
+  auto record = [&](int c) __attribute__((always_inline)) {  // the accumulators -> the record of chunk c, then zero
+    // D layout of the 16x16 MFMA: lane -> column lane % 16 (dk within the tile), register s -> row 4 (lane / 16) + s
+    int lane_off = (64 * dvh + 4 * g) * DH + 64 * dkh + R;
+    asm volatile("" : "+v"(lane_off));  // (computed here, per record: hoisted out of the tile loop the 64 store
+                                        // addresses would sit in registers for the whole kernel)
+    float* dst = record_of(c) + lane_off;
 #pragma unroll
-    for (int s = 0; s < TT_ / 16; ++s) {
-      u32x4_t fk[4], fv[4];
+    for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-      for (int blk = 0; blk < 4; ++blk) {
+      for (int ct = 0; ct < 4; ++ct) {
+        if (ct == 3 && !k3_real) continue;
+        if (rb < 3 || v3_real) {
 #pragma unroll
-        for (int r2 = 0; r2 < 4; ++r2) {
-          const int ta = 16 * s + 2 * (2 * r2) + g, tb = 16 * s + 2 * (2 * r2 + 1) + g;
-          const uint32_t klo = lds_k[ta * LR + blk * 32 + j], khi = lds_k[tb * LR + blk * 32 + j];
-          const uint32_t vlo = lds_v[ta * LR + blk * 32 + j], vhi = lds_v[tb * LR + blk * 32 + j];
-          fk[blk][r2] = klo | (khi << 16);
-          fv[blk][r2] = vlo | (vhi << 16);
+          for (int s = 0; s < 4; ++s) dst[(16 * rb + s) * DH + 16 * ct] = acc[rb][ct][s];
+        } else if (!has_rope) {  // row 112: ksum
+          if (g == 0) dst[(16 * rb) * DH + 16 * ct] = acc[rb][ct][0];
         }
       }
 #pragma unroll
-      for (int ib = 0; ib < 4; ++ib)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int jb = 0; jb < 4; ++jb) acc[ib][jb] = mfma_32x32x16<T>(fv[ib], fk[jb], acc[ib][jb]);
-      if (!PRE) {
-#pragma unroll
-        for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-          for (int r2 = 0; r2 < 4; ++r2) acck[jb] = add_pk16<T>(fk[jb][r2], acck[jb]);
-      }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites
-  }
+      for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // the record's stores share the counter the rings wait on (and need not retire in order with the loads):
+    // drain it once per record, so that the counts keep meaning "tiles younger than this one"
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
 
-  if (PRE) {
-    // lanes l, l + 14, l + 28, l + 42 hold the same piece of different tokens: through the wave's own LDS
-    // region ([56 lanes][8] floats), then channel 32 jb + j adds its four entries, two per token half g
-    float* fold = reinterpret_cast<float*>(lds_k);
-    if (lane_ok) {
-      *reinterpret_cast<f32x4_t*>(fold + lane * 8) = f32x4_t{ks8[0], ks8[1], ks8[2], ks8[3]};
-      *reinterpret_cast<f32x4_t*>(fold + lane * 8 + 4) = f32x4_t{ks8[4], ks8[5], ks8[6], ks8[7]};
-    }
+  int it = 0;  // tile whose operands are read in this iteration
+  if (PRE) {   // tile 0 is transformed ahead of the loop
+    wait_tiles(std::integral_constant<int, NKV - 2>(), issued - 1);
+    __builtin_amdgcn_s_barrier();
+    transform_next();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      const int ch = jb * 32 + j;
-      float sum = 0.f;
-      if (ch < DH) {
-        const float* f0 = fold + ((2 * g) * NCH + (ch >> 3)) * 8 + (ch & 7);
-        sum = f0[0] + f0[NCH * 8];
-      }
-      acck[jb] = sum;
-    }
   }
-#pragma unroll
-  for (int jb = 0; jb < 4; ++jb) acck[jb] += __shfl_xor(acck[jb], 32, 64);  // the two token halves
-
-  // Cross-wave sum in LDS, two images of the padded 128 x 128 accumulator (no predicates): waves 2, 3 -> images
-  // 0, 1; waves 0, 1 add them and write their sums back; then all four waves add the two images and store the
-  // 113 x 112 state as whole 16-byte pieces.  ksum travels as row 112 of the image (that accumulator row belongs
-  // to a zero channel).  D layout of 32x32 MFMA: lane -> column j = lane%32, register r -> row 8*(r/4) +
-  // 4*(lane/32) + r%4.
-  float* red = reinterpret_cast<float*>(smem);
-  auto put = [&](float* img) {
-#pragma unroll
-    for (int ib = 0; ib < 4; ++ib)
-#pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          img[(ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + jb * 32 + j] = acc[ib][jb][r];
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the zero row 112 is written before ksum replaces it
-    if (g == 0) {
-#pragma unroll
-      for (int jb = 0; jb < 4; ++jb) img[DH * 128 + jb * 32 + j] = acck[jb];
+#pragma unroll 1
+  while (has_tile(ccur)) {
+    const Tile112 tl = next_tile(ccur);
+    // this wave's loads of tile it (+ 1 with transforms) have landed: all but those of the tiles issued after it
+    wait_tiles(std::integral_constant<int, NKV - 2 - AHEAD>(), issued - 1 - (it + AHEAD));
+    __builtin_amdgcn_s_barrier();  // and everyone else's; every wave is done with tile it - 1 and the transform of
+                                   // tile it is in LDS (no fence: younger loads stay in flight)
+    if (has_tile(icur)) {          // refill the entries of tile it - 1
+      const Tile112 nl = next_tile(icur);
+      issue(nl.start, nl.limit);
     }
-  };
-  auto take = [&](const float* img) {
-#pragma unroll
-    for (int ib = 0; ib < 4; ++ib)
-#pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          acc[ib][jb][r] += img[(ib * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + jb * 32 + j];
-#pragma unroll
-    for (int jb = 0; jb < 4; ++jb) acck[jb] += img[DH * 128 + jb * 32 + j];
-  };
-  __syncthreads();  // staging tiles are dead
-  if (wave >= 2) put(red + (wave - 2) * 128 * 128);
-  __syncthreads();
-  if (wave < 2) {  // a wave rewrites the image it has just read itself: no barrier in between
-    take(red + wave * 128 * 128);
-    put(red + wave * 128 * 128);
-  }
-  __syncthreads();
-  {
-    const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nsplit + split;
-    float* dst = partial + slot * SE;
-    for (int p = threadIdx.x; p < (DH + 1) * (DH / 4); p += 256) {  // 16-byte pieces of the 113 x 112 state
-      const int row = p / (DH / 4), c4 = p - row * (DH / 4);
-      const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(red + row * 128 + c4 * 4);
-      const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(red + 128 * 128 + row * 128 + c4 * 4);
-      *reinterpret_cast<f32x4_t*>(dst + row * DH + c4 * 4) = x0 + x1;
+    if (mma_role) {
+      Ops112 o;
+      read_ops(it, o);
+      wait_ops(o);
+      mma(o);
+      if (tl.last) record(tl.c);
     }
+    if (PRE && has_tile(tcur)) transform_next();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    ++it;
   }
 }
 
-// sum of the partials of one state in partial order (+ inclusive prefix over chunks when causal)
-__global__ __launch_bounds__(256) void reduce112_kernel(const float* partial, float* state,
-                                                        int BH, int n_chunks, int nparts, int causal) {
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (gid >= (int64_t)BH * SE) return;
-  const int64_t bh = gid / SE;
-  const int e = (int)(gid - bh * SE);
-  float run = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
-    const float* p0 = partial + ((bh * n_chunks + c) * nparts) * SE + e;
-    float s = 0.f;
-    for (int sp0 = 0; sp0 < nparts; sp0 += 16) {
-      float v[16];
+// sum of the records of one chunk in range order (+ inclusive prefix over chunks when causal).  A chunk's records
+// are those of the ranges [begin / L, (end - 1) / L] that touch it; with range_tokens == 0 every chunk has exactly
+// nslot records (the in-place scan of finished states: nslot = 1, partial == state, every thread rewrites only
+// what it has read itself).  Workgroup = cl chunks (a power of two, at most 16) x nq >= 64 groups of four adjacent
+// elements, so that a wave reads whole kilobytes of one record: a thread sums the records of ONE (chunk, element
+// group) -- the loads of its first two
+// records (a chunk shorter than a range has no more) in flight together -- and the prefix over chunks goes through
+// LDS, every thread adding up its predecessors in chunk order, which is the order of a running sum.
+__global__ __launch_bounds__(1024) void reduce112_kernel(const float* partial, float* state, const int32_t* chunk_starts,
+                                                         int N, int n_chunks, int nslot, int range_tokens, int causal,
+                                                         int cl, int nblk) {
+  constexpr int SE4 = SE / 4;
+  __shared__ f32x4_t sums[1024];
+  __shared__ f32x4_t carry_sh[256];
+  const int nq = blockDim.x / cl;
+  const int q = threadIdx.x % nq, lc = threadIdx.x / nq;
+  const int64_t bh = blockIdx.x / nblk;
+  const int e4 = (int)(blockIdx.x - bh * nblk) * nq + q;
+  const bool e_ok = e4 < SE4;
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t carry = zero;
+  for (int c0 = 0; c0 < n_chunks; c0 += cl) {  // uniform
+    const int c = c0 + lc;
+    const bool ok = e_ok && c < n_chunks;
+    f32x4_t s = zero;
+    if (ok) {
+      int nparts = nslot;
+      if (range_tokens > 0) {
+        const int cb = chunk_starts ? chunk_starts[c] : 0, ce = chunk_starts ? chunk_starts[c + 1] : N;
+        nparts = (ce - 1) / range_tokens - cb / range_tokens + 1;
+      }
+      const float* p0 = partial + ((bh * n_chunks + c) * nslot) * SE + e4 * 4;
+      const f32x4_t v0 = *reinterpret_cast<const f32x4_t*>(p0);  // (every chunk has a first record)
+      const f32x4_t v1 = nparts > 1 ? *reinterpret_cast<const f32x4_t*>(p0 + SE) : zero;
+      s = v0 + v1;
+      for (int sp0 = 2; sp0 < nparts; sp0 += 8) {  // a chunk spread over more than two ranges: 8 loads at a time
+        f32x4_t w[8];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) v[u] = (sp0 + u < nparts) ? p0[(int64_t)(sp0 + u) * SE] : 0.f;
+        for (int j = 0; j < 8; ++j)
+          w[j] = sp0 + j < nparts ? *reinterpret_cast<const f32x4_t*>(p0 + (int64_t)(sp0 + j) * SE) : zero;
 #pragma unroll
-      for (int u = 0; u < 16; ++u) s += v[u];
+        for (int j = 0; j < 8; ++j) s += w[j];
+      }
     }
     if (causal) {
-      run += s;
+      sums[threadIdx.x] = s;
+      __syncthreads();
+      f32x4_t run = carry;
+      for (int j = 0; j <= lc; ++j) run += sums[j * nq + q];
       s = run;
+      if (lc == cl - 1) carry_sh[q] = run;
+      __syncthreads();
+      carry = carry_sh[q];
     }
-    state[(bh * n_chunks + c) * SE + e] = s;
+    if (ok) *reinterpret_cast<f32x4_t*>(state + (bh * n_chunks + c) * SE + e4 * 4) = s;
   }
 }
 
 // ----------------------------------------------------------------------------
-// phase 2.  1-D grid over units (batch, chunk, token range) x heads, see head_unit; block 256.
+// phase 2.  grid.x over units (chunk, token range) x heads, see head_unit, grid.y = batch; block 256.
 //
 // The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
 // only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
@@ -354,7 +596,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   HeadUnit hu;
   if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
   const int head = hu.head;
-  const int bx = hu.unit % xranges, c = (hu.unit / xranges) % n_chunks, b = hu.unit / (xranges * n_chunks);
+  const int c = uniform(hu.unit / xranges), bx = hu.unit - c * xranges, b = blockIdx.y;
   const ChunkRange cr = chunk_range(chunk_starts, c, N);
   const int t0 = cr.begin + bx * wg_tokens;
   const int t1 = min(cr.end, t0 + wg_tokens);
@@ -525,28 +767,42 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
 constexpr int compute_units112() { return 256; }
 
 struct Plan112 {
-  int nsplit, split_tokens;
+  int range_tokens, nslot;
 };
+// One workgroup (eight waves) per compute unit: each (batch, head) is cut into 256 / (B h) token ranges of equal
+// length, whatever the chunking.  The plan must not depend on N (the workspace query does not know it), so the
+// length comes from the upper bound n_chunks * max_chunk_tokens; a chunk is touched by at most
+// ceil(max_chunk_tokens / L) + 1 ranges, which is the number of record slots per chunk.
 Plan112 plan112(int B, int h, int n_chunks, int max_chunk_tokens) {
-  // one workgroup per CU (256 accumulator registers per wave: one wave per SIMD), splits of at least 512 tokens
-  const int items = B * h * n_chunks;
-  int ns = 256 / items;  // rounding down: 260 workgroups on 256 CUs would take two rounds
-  const int cap = (max_chunk_tokens + 511) / 512;
-  if (ns > cap) ns = cap;
-  if (ns < 1) ns = 1;
-  if (ns > 64) ns = 64;
+  const int64_t n_ub = (int64_t)n_chunks * max_chunk_tokens;
+  int nr = compute_units112() / (B * h);  // rounding down: 260 workgroups on 256 CUs would take two rounds
+  if (nr < 1) nr = 1;
+  int64_t L = ((n_ub + nr - 1) / nr + 63) / 64 * 64;
+  if (L < 256) L = 256;
   Plan112 pl;
-  pl.split_tokens = ((max_chunk_tokens + ns - 1) / ns + 127) / 128 * 128;
-  pl.nsplit = (max_chunk_tokens + pl.split_tokens - 1) / pl.split_tokens;
-  if (pl.nsplit < 1) pl.nsplit = 1;
+  pl.range_tokens = (int)std::min<int64_t>(L, 1 << 30);
+  pl.nslot = (max_chunk_tokens + pl.range_tokens - 1) / pl.range_tokens + 1;
   return pl;
+}
+
+struct Reduce112Plan {
+  int cl, threads, nblk;  // chunks per workgroup (power of two <= 16), its size, workgroups per (batch, head)
+};
+Reduce112Plan reduce112_plan(int n_chunks) {
+  Reduce112Plan p;
+  p.cl = 1;
+  while (p.cl < n_chunks && p.cl < 16) p.cl *= 2;
+  const int nq = std::max(64, 256 / p.cl);
+  p.threads = nq * p.cl;
+  p.nblk = (SE / 4 + nq - 1) / nq;
+  return p;
 }
 
 }  // namespace
 
 size_t workspace_bytes112(int B, int h, int n_chunks, int max_chunk_tokens) {
   const Plan112 pl = plan112(B, h, n_chunks, max_chunk_tokens);
-  return (size_t)B * h * n_chunks * pl.nsplit * SE * sizeof(float);  // the partials are always written
+  return (size_t)B * h * n_chunks * pl.nslot * SE * sizeof(float);  // the records are always written
 }
 
 int launch_state112(const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N,
@@ -562,14 +818,16 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   if (!workspace || workspace_bytes < need) return SANA_ERR_WORKSPACE;
   if (!aligned16(workspace)) return SANA_ERR_ALIGN;
   float* part = static_cast<float*>(workspace);
-  const int64_t units = (int64_t)B * n_chunks * pl.nsplit, nwg = head_unit_grid(units, h);
-  if (nwg > 0x7fffffff) return SANA_ERR_SHAPE;
-  dim3 grid((unsigned)nwg);
+  const int nranges = (N + pl.range_tokens - 1) / pl.range_tokens;
+  const int64_t units = nranges, nwg = head_unit_grid(units, h);
+  if (nwg > 0x7fffffff || units * ((h + 3) / 4) * 8 > 0x7fffffff || B > 65535 || (int64_t)B * h > (1 << 22))
+    return SANA_ERR_SHAPE;
+  dim3 grid((unsigned)nwg, (unsigned)B);
   const uint16_t* kp = static_cast<const uint16_t*>(k);
   const uint16_t* vp = static_cast<const uint16_t*>(v);
 #define SANA_ST112(T, PRE)                                                                                        \
-  hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(256), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
-                     pl.nsplit, pl.split_tokens, (int)units, stride_b, stride_n, pre)
+  hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(512), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
+                     pl.nslot, pl.range_tokens, (int)units, nranges, stride_b, stride_n, pre)
   const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
   if (io_dtype == SANA_DT_F16) SANA_ST112(F16, 0);
   else if (mode == 3) SANA_ST112(BF16, 3);
@@ -578,16 +836,17 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   else SANA_ST112(BF16, 0);
 #undef SANA_ST112
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
-  const int64_t threads = (int64_t)B * h * SE;
-  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, part, state, B * h,
-                     n_chunks, pl.nsplit, (causal && n_chunks > 1) ? 1 : 0);
+  const Reduce112Plan rp = reduce112_plan(n_chunks);
+  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((int64_t)B * h * rp.nblk)), dim3(rp.threads), 0, s, part, state, chunk_starts,
+                     N, n_chunks, pl.nslot, pl.range_tokens, (causal && n_chunks > 1) ? 1 : 0, rp.cl, rp.nblk);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
 int launch_scan112(float* state, int B, int h, int n_chunks, hipStream_t s) {
-  const int64_t threads = (int64_t)B * h * SE;
-  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, state, state, B * h,
-                     n_chunks, 1, 1);
+  if ((int64_t)B * h > (1 << 22)) return SANA_ERR_SHAPE;
+  const Reduce112Plan rp = reduce112_plan(n_chunks);
+  hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((int64_t)B * h * rp.nblk)), dim3(rp.threads), 0, s, state, state,
+                     static_cast<const int32_t*>(nullptr), 0, n_chunks, 1, 0, 1, rp.cl, rp.nblk);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
@@ -615,9 +874,9 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
     }
   }
   const int xranges = (max_chunk_tokens + wg_tokens - 1) / wg_tokens;
-  const int64_t units = (int64_t)xranges * n_chunks * B, total = head_unit_grid(units, h);
-  if (total > 0x7fffffff) return SANA_ERR_SHAPE;
-  dim3 grid((unsigned)total);
+  const int64_t units = (int64_t)xranges * n_chunks, total = head_unit_grid(units, h);
+  if (total > 0x7fffffff || units * ((h + 3) / 4) * 8 > 0x7fffffff || B > 65535) return SANA_ERR_SHAPE;
+  dim3 grid((unsigned)total, (unsigned)B);
   const uint16_t* qp = static_cast<const uint16_t*>(q);
 #define SANA_AP112(F32, PRE)                                                                                         \
   hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
