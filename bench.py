@@ -641,6 +641,9 @@ def main():
     ap.add_argument("--cfg3-only", action="store_true",
                     help="with --kernels-only: skip the video-shape and 112-wide-head launches (counter runs: every "
                          "kernel instance then runs at the cfg3 shape only)")
+    ap.add_argument("--step-only", action="store_true",
+                    help="only the timed cfg3 chain, printed as a short JSON line (profiling runs: every kernel row of a "
+                         "trace is then the cfg3 shape inside the chained step)")
     ap.add_argument("--stock-conv", action="store_true",
                     help="also time the stock convolution beside the temporal-conv GEMM (minutes of library tuning on a fresh machine)")
     args = ap.parse_args()
@@ -679,6 +682,10 @@ def main():
         assert torch.isfinite(out.float()).all()
         ms_per_step = wall * 1e3 / args.steps
         block_ms = ms_per_step / DEPTH
+        if args.step_only:
+            print(json.dumps({"metric": "cfg3 chained step only", "value": round(block_ms, 4), "unit": "ms per block",
+                              "ms_per_step": round(ms_per_step, 3), "steps": args.steps, "warmup": args.warmup}))
+            return
 
         kernels, copy_gbs = ([], None) if args.no_kernels else kernel_rooflines(dev, stock_conv=args.stock_conv)
         ips_bf16 = images_per_s(dev, blocks, 5, 2)

@@ -81,7 +81,8 @@ const char* sana_hip_strerror(int code);
  *                 (may be NULL when that function returns 0)
  * Accumulation is fp32 and deterministic (fixed summation order, no atomics).
  * d = 112 addresses the tokens of one batch entry with 32-bit byte offsets:
- * N * stride_n * 2 must stay below 2^31 (SANA_ERR_SHAPE otherwise).
+ * N * stride_n * 2 and N * 448 must stay below 2^31; its grids also want
+ * B <= 65535 and B * h <= 2^22 (SANA_ERR_SHAPE otherwise).
  */
 size_t sana_hip_linattn_workspace_bytes(int B, int h, int d, int n_chunks, int max_chunk_tokens,
                                         int io_dtype);

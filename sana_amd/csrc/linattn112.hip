@@ -1,17 +1,19 @@
 // ReLU linear attention for head_dim 112 (the `linear_head_dim: 112` video configurations) on gfx950,
 // bf16 / f16 io.  Same two phases and the same state layout as the head_dim-32 kernels --
 // fp32 [B][h][n_chunks][113][112], row 112 = sum_n relu(k_n) -- but one head is now a 112 x 112
-// problem of its own (3.5 x 3.5 MFMA tiles, padded to 4 x 4 with zero channels):
+// problem of its own (7 x 7 MFMA tiles of 16, padded to 8 x 8 with zero channels):
 //
-//   phase 1  workgroup = (batch, head, chunk, token split); each of its four waves takes interleaved
-//            32-token tiles (16 with on-load transforms) and owns a whole 128 x 128 accumulator (256
-//            registers).  Tiles go through wave-private LDS to become token-contiguous MFMA operands, as
-//            in the head_dim-32 kernel; the waves are summed in LDS (two padded accumulator images) and
-//            a second kernel sums the splits in a fixed order.
-//   phase 2  workgroup = (batch, head, chunk, range of 192..512 tokens), steps of 32 tokens through
-//            workgroup-shared LDS tiles; wave w produces output channels [32w, 32w+32) from its own slice
-//            of the state (two bf16 terms of the fp32 values as MFMA 16x16x32 A operands for bf16 output,
-//            three for fp32 output) plus a row block that carries ksum in every row, so each lane gets
+//   phase 1  workgroup = (batch, head, token range): eight waves walk the range in tiles of 32 tokens that come
+//            global -> LDS by direct loads into a ring; four waves accumulate the 128 x 128 state in registers
+//            (operands read transposed from the token-major tiles), four apply the on-load transforms one tile
+//            ahead.  One record per chunk the range touches; a second kernel sums a chunk's records in range
+//            order and runs the prefix over chunks.
+//   phase 2  without on-load transforms the same walk: four MFMA waves, four waves that issue the loads and carry
+//            finished output tiles to global memory.  With transforms: workgroup = (batch, head, chunk, range of
+//            192..512 tokens), 256 threads that all load, transform, multiply and store, steps of 32 tokens
+//            through workgroup-shared LDS tiles.  In both, wave w produces output channels [32w, 32w+32) from its
+//            own slice of the state (two bf16 terms of the fp32 values as MFMA 16x16x32 A operands for bf16
+//            output, three for fp32 output) plus a row block that carries ksum in every row, so each lane gets
 //            its token's denominator.
 #include <algorithm>
 #include <type_traits>
@@ -123,6 +125,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 // loads still in flight (the stages further down the ring) and it would wait for ALL of them (vmcnt(0)) in front of
 // the first read, which would empty the ring at every tile.  Which loads must have landed is the kernel's own
 // business (counted waits + barriers); the waits for the LDS reads themselves are tied to their results.
+// Between such a read and its wait there must be no control flow that merges the result with another value: the
+// compiler, to which the result exists as soon as the statement has run, may copy it then and there.
 // addr: LDS byte address, OFF: immediate byte offset.
 //
 // read_tr16: 4 tokens x 16 channels of a token-major tile -> this lane's channel, 4 tokens; addr points at the
@@ -132,6 +136,12 @@ __device__ __forceinline__ u32x2_t read_tr16(uint32_t addr) {
   u32x2_t v;
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
+}
+// the same into a register that already holds a value (read-write operand: a conditional read then needs no
+// merge of two registers behind it, where the compiler could copy a result that has not arrived yet)
+template <int OFF>
+__device__ __forceinline__ void read_tr16_over(u32x2_t& v, uint32_t addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "+v"(v) : "v"(addr), "n"(OFF));
 }
 template <int OFF>
 __device__ __forceinline__ u32x4_t lds_read128(uint32_t addr) {
@@ -398,13 +408,13 @@ __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restric
     o.v[0][0] = read_tr16<0>(vb), o.v[0][1] = read_tr16<16 * S2_ROW>(vb);
     o.v[1][0] = read_tr16<32>(vb), o.v[1][1] = read_tr16<32 + 16 * S2_ROW>(vb);
     o.v[2][0] = read_tr16<64>(vb), o.v[2][1] = read_tr16<64 + 16 * S2_ROW>(vb);
-    if (v3_real) o.v[3][0] = read_tr16<96>(vb), o.v[3][1] = read_tr16<96 + 16 * S2_ROW>(vb);
-    else o.v[3][0] = o.v[3][1] = ones2;
+    o.v[3][0] = o.v[3][1] = ones2;  // row block 112..127: row 0 of the A operand is all ones
+    if (v3_real) read_tr16_over<96>(o.v[3][0], vb), read_tr16_over<96 + 16 * S2_ROW>(o.v[3][1], vb);
     o.k[0][0] = read_tr16<0>(kb), o.k[0][1] = read_tr16<16 * S2_ROW>(kb);
     o.k[1][0] = read_tr16<32>(kb), o.k[1][1] = read_tr16<32 + 16 * S2_ROW>(kb);
     o.k[2][0] = read_tr16<64>(kb), o.k[2][1] = read_tr16<64 + 16 * S2_ROW>(kb);
-    if (k3_real) o.k[3][0] = read_tr16<96>(kb), o.k[3][1] = read_tr16<96 + 16 * S2_ROW>(kb);
-    else o.k[3][0] = o.k[3][1] = u32x2_t{0u, 0u};
+    o.k[3][0] = o.k[3][1] = u32x2_t{0u, 0u};  // column block 112..127
+    if (k3_real) read_tr16_over<96>(o.k[3][0], kb), read_tr16_over<96 + 16 * S2_ROW>(o.k[3][1], kb);
   };
   auto wait_ops = [&](Ops112& o) __attribute__((always_inline)) {
     asm volatile("s_waitcnt lgkmcnt(0)"
@@ -548,13 +558,26 @@ __global__ __launch_bounds__(1024) void reduce112_kernel(const float* partial, f
 }
 
 // ----------------------------------------------------------------------------
-// phase 2.  grid.x over units (chunk, token range) x heads, see head_unit, grid.y = batch; block 256.
+// phase 2 without on-load transforms.  grid.x over token ranges x heads, see head_unit, grid.y = batch; block 512 =
+// eight waves.
 //
-// The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
-// only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
-// (transforms applied once, here) into an LDS tile, every wave takes its MFMA B operands from that
-// tile, results go to an LDS output tile and leave as whole rows again.  Tiles are double buffered,
-// the next tile's loads are in flight during the MFMAs: one barrier per step.
+// Built like phase 1: a workgroup walks ONE contiguous token range of a (batch, head), cut by token count, in
+// tiles of 32 tokens that never straddle a chunk boundary.  The q rows of a tile come global -> LDS by direct loads
+// into a ring; waves 0..3 run the MFMAs (and the ReLU, on their operands), waves 4..7 issue the loads and carry the
+// finished output tile of the step before from LDS to global memory in whole rows.  A wave that talks to global
+// memory stalls while the memory pipeline is full, which is most of the time in a kernel bound by it: the MFMA
+// waves only ever wait for data that has already landed.  (With on-load transforms the same layout was measured a
+// sixth SLOWER than the kernel further down: four waves are too few for the transform arithmetic of a tile.)
+//
+// q tiles are rows of 16 pieces of 16 bytes (14 of data, 2 of zeros: the padded k range 112..127) with the piece
+// index XORed with the token's low four bits: the 16 tokens of an MFMA B operand read (one piece each, same logical
+// piece) hit 16 different pieces, i.e. all 64 banks once.  Direct loads fill LDS linearly, lane by lane, so the
+// swizzle is applied to the global address a lane fetches.
+//
+// MFMA wave w produces output channels [32 w, 32 w + 32) from its own slice of the chunk's state (two bf16 terms
+// of the fp32 values as MFMA 16x16x32 A operands for bf16 output, three for fp32 output) plus a row block that
+// carries ksum in every row, so each lane gets its token's denominator.  The slice is rebuilt when the walk enters
+// another chunk.
 // ----------------------------------------------------------------------------
 // fp32 -> bf16 terms hi + mid (+ lo), pairwise: one packed convert rounds two values
 template <int NT>
@@ -574,11 +597,271 @@ __device__ __forceinline__ void split_terms(const float x[8], u32x4_t out[NT]) {
   }
 }
 
+constexpr int A2_QT = TILE * 256;   // a q tile: 32 rows of 16 pieces
+constexpr int OROW16 = 272;         // byte row stride of the 16-bit output tile: 68 banks, so the 16 tokens of a b128
+                                    // write land on 16 disjoint groups of 4 banks
+constexpr int OROW32 = 464;         // of the fp32 output tile (116 banks = 52 mod 64: same argument)
+template <bool OUT_F32>
+struct Stage3 {
+  static constexpr int n_q = A2_QT / 1024;   // load instructions per tile: 8, two per issuing wave
+  static constexpr int NQ = 4;               // ring depth
+  static constexpr int out_bytes = TILE * (OUT_F32 ? OROW32 : OROW16);
+  static constexpr int out_off = NQ * A2_QT;
+  static constexpr int bytes = out_off + 2 * out_bytes;
+  static constexpr int per_wave = n_q / 4;
+};
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(512) void apply112_stream_kernel(const uint16_t* __restrict__ Q,
+                                                              const float* __restrict__ state, void* __restrict__ out,
+                                                              const int32_t* __restrict__ chunk_starts, int N, int h,
+                                                              int n_chunks, int range_tokens, int units,
+                                                              int64_t q_stride_b, int64_t q_stride_n, int64_t o_stride_b,
+                                                              int64_t o_stride_n, float eps) {
+  typedef Stage3<OUT_F32> ST;
+  constexpr int NQ = ST::NQ;
+  constexpr int NT = OUT_F32 ? 3 : 2;    // bf16 terms of an fp32 state value: 24 / 16 mantissa bits
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[ST::bytes];
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  HeadUnit hu;
+  if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
+  const int head = hu.head;
+  const int rg = hu.unit, b = blockIdx.y;
+  const int r0 = rg * range_tokens, r1 = min(N, r0 + range_tokens);
+  if (r0 >= r1) return;
+  auto chunk_end = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c + 1] : N; };
+  int c0 = 0;
+  while (chunk_end(c0) <= r0) ++c0;  // the chunk of the range's first token (uniform; a few dozen chunks at most)
+  const uint32_t smem_addr = lds_addr(smem);
+  const bool mma_role = wave < 4;  // wave-uniform
+
+  // ---- global -> LDS, issued by the helper waves (measured: 73 us against 86 with the MFMA waves issuing, whose
+  // instruction stream is the longest here): wave w issues instructions w - 4 and w of a tile, each 4 rows of 16
+  // pieces
+  const int row_b = (int)q_stride_n * 2;
+  const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(Q + (int64_t)b * q_stride_b + head * DH), 0,
+      (int)((int64_t)N * q_stride_n * 2 - (int64_t)head * DH * 2), 0x00020000);
+  const int idle = (int)0x80000000u;
+  // per load instruction of this wave: the lane's token row within the tile and its byte offset from the tile's
+  // first token (the padding pieces: an offset outside the resource, i.e. zeros)
+  int ld_row[ST::per_wave], ld_off[ST::per_wave];
+#pragma unroll
+  for (int j = 0; j < ST::per_wave; ++j) {
+    const int s = ((wave & 3) + 4 * j) * 64 + lane, row = s >> 4, piece = (s & 15) ^ (row & 15);
+    ld_row[j] = row;
+    ld_off[j] = piece < NCH ? row * row_b + piece * 16 : idle;
+  }
+  int issued = 0;  // tiles whose loads have been issued; tile t lives in ring entry t % NQ
+  auto issue = [&](int start, int limit) __attribute__((always_inline)) {
+    if (!mma_role) {
+      unsigned char* qb = smem + (issued % NQ) * A2_QT;
+#pragma unroll
+      for (int j = 0; j < ST::per_wave; ++j) {
+        const int q = (wave & 3) + 4 * j;  // wave-uniform
+        // the tile's first token goes into the scalar offset; rows past the limit get an offset outside the resource
+        const int voff = ld_row[j] < limit - start ? ld_off[j] : idle;
+        auto dst = (__attribute__((address_space(3))) void*)(qb + q * 1024);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, dst, 16, voff, start * row_b, 0, 0);
+      }
+    }
+    ++issued;
+  };
+  // waits until the issuing waves' loads of all but the `keep` youngest tiles have landed; `keep` as a template
+  // argument when it is the steady-state figure, everything otherwise (the tail of the range)
+  auto wait_tiles = [&](int keep) __attribute__((always_inline)) {
+    if (mma_role) return;  // nothing of its own in flight that anyone waits for
+    if (keep == NQ - 2) wait_vmcnt<(NQ - 2) * ST::per_wave>();
+    else wait_vmcnt<0>();
+  };
+  auto has_tile = [&](const TileCur& cur) __attribute__((always_inline)) { return cur.t < r1; };
+  auto next_tile = [&](TileCur& cur) __attribute__((always_inline)) {
+    Tile112 tl;
+    tl.start = cur.t;
+    tl.limit = cur.seg_end;
+    tl.c = cur.c;
+    const int nt = min(cur.t + TILE, cur.seg_end);
+    tl.last = nt == cur.seg_end;
+    cur.t = nt;
+    if (tl.last && nt < r1) {
+      ++cur.c;
+      cur.seg_end = min(chunk_end(cur.c), r1);
+    }
+    return tl;
+  };
+  TileCur icur = {r0, c0, min(chunk_end(c0), r1)}, ccur = icur;
+#pragma unroll 1
+  for (int i = 0; i < NQ - 1 && has_tile(icur); ++i) {
+    const Tile112 tl = next_tile(icur);
+    issue(tl.start, tl.limit);
+  }
+
+  // ---- helper waves: the output tile of a finished step -> global memory, whole rows
+  const int tq = tid - 256;
+  constexpr int OP = OUT_F32 ? 2 * NCH : NCH;                  // 16-byte pieces per output row
+  constexpr int OPT = (TILE * OP + 255) / 256;                 // pieces per helper thread
+  auto store_tile = [&](int buf, int start, int limit) __attribute__((always_inline)) {
+    if (mma_role) return;
+    // (the stores below share the vector memory counter with this wave's loads.  That is harmless for the counted
+    // waits: outstanding stores only add to the count, so "at most k operations outstanding" still means "at most k
+    // loads outstanding", and loads retire in issue order)
+    const uint32_t ta = smem_addr + ST::out_off + buf * ST::out_bytes;
+    u32x4_t v[OPT];
+    int tok[OPT], p[OPT];
+    int tqv = tq;
+    asm volatile("" : "+v"(tqv));  // (addresses are computed here, per tile: hoisted out of the tile loop they
+                                   // would occupy registers for the whole kernel)
+#pragma unroll
+    for (int u = 0; u < OPT; ++u) {
+      // (every thread reads, the surplus ones the last piece again: no branch between a read and its wait, where
+      // the compiler could copy a result that has not arrived yet)
+      const int i = min(tqv + 256 * u, TILE * OP - 1);
+      tok[u] = i / OP;
+      p[u] = i - tok[u] * OP;
+      v[u] = lds_read128<0>(ta + tok[u] * (OUT_F32 ? OROW32 : OROW16) + p[u] * 16);
+    }
+    if (OPT == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[OPT - 1]));
+    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[OPT - 2]), "+v"(v[OPT - 1]));
+    unsigned char* ob = reinterpret_cast<unsigned char*>(out) +
+                        ((int64_t)b * o_stride_b + head * DH) * (OUT_F32 ? 4 : 2);
+#pragma unroll
+    for (int u = 0; u < OPT; ++u) {
+      const int i = tqv + 256 * u;
+      if (i < TILE * OP && start + tok[u] < limit)
+        *reinterpret_cast<u32x4_t*>(ob + (int64_t)(start + tok[u]) * o_stride_n * (OUT_F32 ? 4 : 2) + p[u] * 16) = v[u];
+    }
+  };
+
+  // ---- MFMA waves.  A operands: MFMA 16x16x32 A lane -> row lane % 16, k = 8 (lane / 16) + e.  Row r of row block
+  // rb of this wave is output channel 32 wave + 8 (r / 4) + 4 rb + r % 4, so that a lane (token n, group g') ends
+  // up with the 8 contiguous channels 32 wave + 8 g' .. + 7 (registers s of blocks 0 and 1).  Block 2 carries ksum
+  // in every row.  Channels and k indices past 112 are zero.
+  const int n = lane & 15, g = lane >> 4;
+  u32x4_t a[3][4][NT];  // [row block][k block][term]
+  auto load_state = [&](int c) __attribute__((always_inline)) {
+    const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * SE;
+    // buffer loads: rows / k groups outside the head's state get an out-of-range offset and read as zero
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sp), 0, SE * 4, 0x00020000);
+#pragma unroll
+    for (int rb = 0; rb < 3; ++rb) {
+      const int ch = 32 * (wave & 3) + 8 * (n >> 2) + 4 * rb + (n & 3);
+      const int row = rb < 2 ? ch : DH;
+      const bool row_ok = rb == 2 || ch < DH;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const int k0 = kb * 32 + 8 * g;
+        const int off = (row_ok && k0 < DH) ? (row * DH + k0) * 4 : idle;
+        const f32x4_t x0 = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, off, 0, 0));
+        const f32x4_t x1 = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, off + 16, 0, 0));
+        const float x[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        split_terms<NT>(x, a[rb][kb]);
+      }
+    }
+  };
+  // B operand of k block kb: piece 4 kb + g of the lane's token, at its swizzled place
+  uint32_t qoff[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) qoff[kb] = n * 256 + (((4 * kb + g) ^ n) << 4);
+  const int och = 32 * (wave & 3) + 8 * g;  // this lane's 8 output channels
+  auto mma_tile = [&](int tile) __attribute__((always_inline)) {
+    const uint32_t sa = smem_addr + (tile % NQ) * A2_QT;
+    const uint32_t to = smem_addr + ST::out_off + (tile & 1) * ST::out_bytes;
+    // [token half][k block].  With bf16 output both halves are read up front (the second arrives during the MFMAs
+    // of the first); with fp32 output the third state term has taken the registers: one half at a time
+    constexpr bool BOTH = !OUT_F32;
+    u32x4_t qd[2][4];
+    auto read_half = [&](int ss) __attribute__((always_inline)) {
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) qd[ss][kb] = ss ? lds_read128<16 * 256>(sa + qoff[kb]) : lds_read128<0>(sa + qoff[kb]);
+    };
+    read_half(0);
+    if (BOTH) read_half(1);
+#pragma unroll
+    for (int ss = 0; ss < 2; ++ss) {
+      if (!BOTH && ss == 1) read_half(1);
+      if (BOTH && ss == 0)
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(qd[0][0]), "+v"(qd[0][1]), "+v"(qd[0][2]), "+v"(qd[0][3]));
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(qd[ss][0]), "+v"(qd[ss][1]), "+v"(qd[ss][2]), "+v"(qd[ss][3]));
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) qd[ss][kb] = relu_pk16(qd[ss][kb]);
+      f32x4_t acc[3];
+#pragma unroll
+      for (int rb = 0; rb < 3; ++rb) acc[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int term = NT - 1; term >= 0; --term)  // smallest term first
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int rb = 0; rb < 3; ++rb)  // three independent chains back to back
+            acc[rb] = mfma_16x16x32_bf16(a[rb][kb][term], qd[ss][kb], acc[rb]);
+      if (och < DH) {
+        const float den = acc[2][0] + eps;
+        if (OUT_F32) {
+          f32x4_t o0, o1;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            o0[s] = acc[0][s] / den;
+            o1[s] = acc[1][s] / den;
+          }
+          const uint32_t oa = to + (16 * ss + n) * OROW32 + och * 4;
+          lds_write128<0>(oa, __builtin_bit_cast(u32x4_t, o0));
+          lds_write128<16>(oa, __builtin_bit_cast(u32x4_t, o1));
+        } else {
+          const float inv = __builtin_amdgcn_rcpf(den);
+          u32x4_t o;
+          o.x = pack_bf16(acc[0][0] * inv, acc[0][1] * inv);
+          o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
+          o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
+          o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
+          lds_write128<0>(to + (16 * ss + n) * OROW16 + och * 2, o);
+        }
+      }
+    }
+  };
+
+  int it = 0, cur_c = -1;
+  Tile112 prev = {0, 0, 0, false};
+#pragma unroll 1
+  while (has_tile(ccur)) {
+    const Tile112 tl = next_tile(ccur);
+    if (mma_role && tl.c != cur_c) {  // uniform: the walk enters another chunk
+      load_state(tl.c);
+      cur_c = tl.c;
+    }
+    wait_tiles(issued - 1 - it);
+    __builtin_amdgcn_s_barrier();  // tile it has landed, every wave is done with tile it - 1 and its output tile is
+                                   // complete (no fence: younger loads stay in flight)
+    if (has_tile(icur)) {          // refill the ring entry of tile it - 1
+      const Tile112 nl = next_tile(icur);
+      issue(nl.start, nl.limit);
+    }
+    if (mma_role) mma_tile(it);
+    if (it > 0) store_tile((it - 1) & 1, prev.start, prev.limit);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    prev = tl;
+    ++it;
+  }
+  __builtin_amdgcn_s_barrier();
+  store_tile((it - 1) & 1, prev.start, prev.limit);
+}
+
+// ----------------------------------------------------------------------------
+// phase 2 with on-load transforms (q/k RMSNorm, rotary embedding).  grid.x over units (chunk, token range) x heads,
+// see head_unit, grid.y = batch; block 256: every wave loads, transforms, multiplies and stores, and two or three
+// workgroups share a compute unit.
+//
+// The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
+// only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
+// (transforms applied once, here) into an LDS tile, every wave takes its MFMA B operands from that
+// tile, results go to an LDS output tile and leave as whole rows again.  Tiles are double buffered,
+// the next tile's loads are in flight during the MFMAs: one barrier per step.
+// ----------------------------------------------------------------------------
 constexpr int TT = 32;             // tokens per step
-constexpr int QROW = 136;          // LDS row stride of the 16-bit tiles, elements: 272 B = 68 banks, so the 16 tokens
+constexpr int QROWE = 136;          // LDS row stride of the 16-bit tiles, elements: 272 B = 68 banks, so the 16 tokens
                                    // of a b128 operand read land on 16 disjoint groups of 4 banks; pieces 14
                                    // and 15 of a row (the padded k range 112..127) stay zero
-constexpr int OROW32 = 116;        // row stride of the fp32 output tile, floats (same argument: 116 % 64 = 52)
+constexpr int OROWF = 116;        // row stride of the fp32 output tile, floats (same argument: 116 % 64 = 52)
 
 template <bool OUT_F32, int PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
@@ -589,8 +872,8 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
   constexpr int NQ = (PRE & 2) ? 2 : 1;  // with a rotary embedding: rotated (numerator) and unrotated (denominator) tiles
-  constexpr int OT = OUT_F32 ? TT * OROW32 * 2 : TT * QROW;  // output tile, in 16-bit units
-  __shared__ __attribute__((aligned(16))) uint16_t lds_q[2 * NQ * TT * QROW];
+  constexpr int OT = OUT_F32 ? TT * OROWF * 2 : TT * QROWE;  // output tile, in 16-bit units
+  __shared__ __attribute__((aligned(16))) uint16_t lds_q[2 * NQ * TT * QROWE];
   __shared__ __attribute__((aligned(16))) uint16_t lds_o[2 * OT];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   HeadUnit hu;
@@ -667,37 +950,37 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
     }
   };
   auto stage = [&](int buf) {  // registers -> LDS tile(s); tokens past the range are zeros
-    uint16_t* td = lds_q + buf * NQ * TT * QROW;  // unrotated: the denominator operand (and the numerator without rope)
+    uint16_t* td = lds_q + buf * NQ * TT * QROWE;  // unrotated: the denominator operand (and the numerator without rope)
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       if (!ld_ok[i]) continue;
       u32x4_t x = qreg[i];
       if (has_norm) x = rms_scale8(x, rin[i], qw[i]);
       x = relu_pk16(x);
-      *reinterpret_cast<u32x4_t*>(td + ld_tok[i] * QROW + ld_ch[i] * 8) = x;
+      *reinterpret_cast<u32x4_t*>(td + ld_tok[i] * QROWE + ld_ch[i] * 8) = x;
       if (has_rope)
-        *reinterpret_cast<u32x4_t*>(td + TT * QROW + ld_tok[i] * QROW + ld_ch[i] * 8) = rope8(x, cs[i][0], cs[i][1]);
+        *reinterpret_cast<u32x4_t*>(td + TT * QROWE + ld_tok[i] * QROWE + ld_ch[i] * 8) = rope8(x, cs[i][0], cs[i][1]);
     }
   };
 
   const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
   for (int i = tid; i < 2 * NQ * TT * 3; i += 256)  // pieces 14..16 of every q tile row: written once, as zeros
-    *reinterpret_cast<u32x4_t*>(lds_q + (i / 3) * QROW + (NCH + i % 3) * 8) = zero4;
+    *reinterpret_cast<u32x4_t*>(lds_q + (i / 3) * QROWE + (NCH + i % 3) * 8) = zero4;
   issue(t0);
   stage(0);
   if (t0 + TT < t1) issue(t0 + TT);
   __syncthreads();
   int buf = 0;
   for (int t = t0; t < t1; t += TT, buf ^= 1) {
-    const uint16_t* td = lds_q + buf * NQ * TT * QROW;
-    const uint16_t* tb = has_rope ? td + TT * QROW : td;
+    const uint16_t* td = lds_q + buf * NQ * TT * QROWE;
+    const uint16_t* tb = has_rope ? td + TT * QROWE : td;
     uint16_t* to = lds_o + buf * OT;
 #pragma unroll
     for (int ss = 0; ss < TT / 16; ++ss) {
       u32x4_t qd[4], qb[4];
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const int off = (16 * ss + n) * QROW + (kb * 4 + g) * 8;  // pieces 14, 15 (kb = 3, g >= 2) hold zeros
+        const int off = (16 * ss + n) * QROWE + (kb * 4 + g) * 8;  // pieces 14, 15 (kb = 3, g >= 2) hold zeros
         qb[kb] = *reinterpret_cast<const u32x4_t*>(tb + off);
         if (has_rope) qd[kb] = *reinterpret_cast<const u32x4_t*>(td + off);
       }
@@ -720,7 +1003,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
             o0[s] = acc[0][s] / den;
             o1[s] = acc[1][s] / den;
           }
-          float* op = reinterpret_cast<float*>(to) + (16 * ss + n) * OROW32 + och;
+          float* op = reinterpret_cast<float*>(to) + (16 * ss + n) * OROWF + och;
           *reinterpret_cast<f32x4_t*>(op) = o0;
           *reinterpret_cast<f32x4_t*>(op + 4) = o1;
         } else {
@@ -730,7 +1013,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
           o.y = pack_bf16(acc[0][2] * inv, acc[0][3] * inv);
           o.z = pack_bf16(acc[1][0] * inv, acc[1][1] * inv);
           o.w = pack_bf16(acc[1][2] * inv, acc[1][3] * inv);
-          *reinterpret_cast<u32x4_t*>(to + (16 * ss + n) * QROW + och) = o;
+          *reinterpret_cast<u32x4_t*>(to + (16 * ss + n) * QROWE + och) = o;
         }
       }
     }
@@ -749,7 +1032,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
         const int id = tid + 256 * i, tok = id / (2 * NCH), piece = id - tok * (2 * NCH);
         if (id < TT * 2 * NCH && t + tok < t1)
           *reinterpret_cast<f32x4_t*>(ob + (int64_t)(t + tok) * o_stride_n + piece * 4) =
-              *reinterpret_cast<const f32x4_t*>(tf + tok * OROW32 + piece * 4);
+              *reinterpret_cast<const f32x4_t*>(tf + tok * OROWF + piece * 4);
       }
     } else {
       uint16_t* ob = reinterpret_cast<uint16_t*>(out) + (int64_t)b * o_stride_b + head * DH;
@@ -757,7 +1040,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
       for (int i = 0; i < 2; ++i) {
         if (ld_ok[i] && t + ld_tok[i] < t1)
           *reinterpret_cast<u32x4_t*>(ob + (int64_t)(t + ld_tok[i]) * o_stride_n + ld_ch[i] * 8) =
-              *reinterpret_cast<const u32x4_t*>(to + ld_tok[i] * QROW + ld_ch[i] * 8);
+              *reinterpret_cast<const u32x4_t*>(to + ld_tok[i] * QROWE + ld_ch[i] * 8);
       }
     }
   }
@@ -850,7 +1133,7 @@ int launch_scan112(float* state, int B, int h, int n_chunks, hipStream_t s) {
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
-int launch_apply112(const void* q, const float* state, void* out, int B, int N, int h, int64_t q_stride_b,
+static int launch_apply112_pre(const void* q, const float* state, void* out, int B, int N, int h, int64_t q_stride_b,
                     int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts,
                     int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
                     hipStream_t s) {
@@ -893,6 +1176,38 @@ int launch_apply112(const void* q, const float* state, void* out, int B, int N, 
     else SANA_AP112(false, 0);
   }
 #undef SANA_AP112
+  return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
+}
+
+
+int launch_apply112(const void* q, const float* state, void* out, int B, int N, int h, int64_t q_stride_b,
+                    int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n, const int32_t* chunk_starts,
+                    int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
+                    hipStream_t s) {
+  if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
+  const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
+  // the streaming kernel addresses one batch entry's tokens with 32-bit byte offsets (buffer loads)
+  if (mode != 0 || (int64_t)N * q_stride_n * 2 >= (int64_t)1 << 31)
+    return launch_apply112_pre(q, state, out, B, N, h, q_stride_b, q_stride_n, o_stride_b, o_stride_n, chunk_starts, n_chunks,
+                               max_chunk_tokens, eps, io_dtype, out_dtype, pre, s);
+  // one workgroup (eight waves) per compute unit: 256 / (B h) token ranges of equal length per (batch, head)
+  int nr = compute_units112() / (B * h);
+  if (nr < 1) nr = 1;
+  int64_t L = (((int64_t)N + nr - 1) / nr + TILE - 1) / TILE * TILE;
+  if (L < 256) L = 256;
+  const int range_tokens = (int)L;
+  const int nranges = (N + range_tokens - 1) / range_tokens;
+  const int64_t units = nranges, total = head_unit_grid(units, h);
+  if (total > 0x7fffffff || units * ((h + 3) / 4) * 8 > 0x7fffffff || B > 65535) return SANA_ERR_SHAPE;
+  (void)max_chunk_tokens;
+  dim3 grid((unsigned)total, (unsigned)B);
+  const uint16_t* qp = static_cast<const uint16_t*>(q);
+#define SANA_AP112S(F32)                                                                                            \
+  hipLaunchKernelGGL((apply112_stream_kernel<F32>), grid, dim3(512), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
+                     range_tokens, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps)
+  if (out_dtype == SANA_DT_F32) SANA_AP112S(true);
+  else SANA_AP112S(false);
+#undef SANA_AP112S
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
