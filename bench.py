@@ -57,7 +57,7 @@ def dominant_kernel_traffic_bytes():
     try:
         for line in open(TRAFFIC_PROFILE):
             if line.startswith(DOMINANT_KERNEL_ROW):
-                cols = line[len(DOMINANT_KERNEL_ROW):].split()
+                cols = line.split()[-7:]   # FETCH_SIZE read_MB alg_rd_MB WRITE_SIZE write_MB alg_wr_MB traffic/alg
                 return int(round((float(cols[1]) + float(cols[4])) * 1e6))   # read_MB + write_MB
     except (OSError, ValueError, IndexError):
         pass
