@@ -39,6 +39,8 @@ CASES = [
     (1, 1, 224),          # one token
     (3, 129, 112),
     (1, 21 * 1560, 224),  # cfg5 token count (long splits)
+    (13, 300, 2240),      # 260 (batch, head) pairs: more than compute units, one token range each
+    (2, 2100, 1120),      # ranges of 192 tokens that end inside tiles
 ]
 
 
@@ -95,7 +97,9 @@ def test_deterministic_and_additive(cuda):
     assert (out - 1.5).abs().max().item() < 1e-4
 
 
-@pytest.mark.parametrize("frames,hw,chunk_frames", [(4, 6, [0, 1, 2, 3]), (5, 37, [0, 2]), (21, 1560, [0, 11])])
+@pytest.mark.parametrize("frames,hw,chunk_frames", [(4, 6, [0, 1, 2, 3]), (5, 37, [0, 2]), (21, 1560, [0, 11]),
+                                                    (40, 30, list(range(40))),        # 40 chunks shorter than a tile
+                                                    (33, 100, list(range(0, 33, 2)))])  # 17 chunks, several per range
 def test_chunk_causal_matches_oracle(cuda, frames, hw, chunk_frames):
     B, C, eps = 1, 224, 1e-8
     N = frames * hw

@@ -134,6 +134,24 @@ def test_rotation_is_numerator_only_and_unit_rotation_is_identity(cuda):
 
 
 @pytest.mark.parametrize("qk_norm", [False, True])
+@pytest.mark.parametrize("frames,hw,chunk_index", [(24, (5, 6), list(range(24))),      # every chunk shorter than a tile
+                                                   (9, (20, 23), [0, 1, 2, 5, 8])])   # chunks of 460 .. 1380 tokens
+def test_chunk_causal_with_rope_head_dim_112_many_chunks(cuda, qk_norm, frames, hw, chunk_index):
+    """The 112-wide-head kernels walk token ranges across chunk boundaries: records per (range, chunk), the unrotated
+    key sums folded when a chunk ends (at every tile in the first case), the state operands rebuilt per chunk."""
+    B, C = 2, 448
+    N = frames * hw[0] * hw[1]
+    om, hm = make("ChunkCausalAttention", C, qk_norm, seed=9, head_dim=112)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(N)).bfloat16()
+    fr = freqs(N, 2, head_dim=112)
+    with torch.no_grad():
+        ref = ref64(om, x, HW=(frames, *hw), rotary_emb=fr, chunk_index=chunk_index)
+        out = hm(x.to(cuda), HW=(frames, *hw), rotary_emb=fr.to(cuda), chunk_index=chunk_index)
+    check(out, ref, "ChunkCausalAttention d=112 + rope, many chunks")
+
+
+@pytest.mark.parametrize("qk_norm", [False, True])
 @pytest.mark.parametrize("C,head_dim", [(160, 32), (224, 112)])
 def test_chunk_causal_with_rope(cuda, qk_norm, C, head_dim):
     B, (f, h, w) = 1, (5, 6, 8)
