@@ -63,8 +63,11 @@ inline int64_t head_unit_grid(int64_t units, int h) { return (units * ((h + 3) /
 // A workgroup walks ONE contiguous token range of a (batch, head) -- ranges are cut by token count, not by chunk,
 // so every workgroup has the same work whatever the chunking -- in tiles of 32 tokens that never straddle a chunk
 // boundary, and writes one record (113 x 112 fp32) per chunk its range touches:
-//   record[(bh * n_chunks + c) * nslot + (range - first range touching c)]
-// reduce112_kernel adds a chunk's records in range order (and runs the prefix over chunks when causal).
+//   record[bh * nrec + range + c]
+// (walking along the tokens, every new (range, chunk) pair increases the range or the chunk index or both, so
+// range + c is different for every pair that occurs and at most ranges + chunks - 2; the records of a chunk are
+// consecutive).  reduce112_kernel adds a chunk's records in range order (and runs the prefix over chunks when
+// causal).
 //
 // Everything a tile needs comes global -> LDS by direct loads (`buffer_load_dwordx4 ... lds`, 16 bytes per lane,
 // no staging registers) into rings: K and V rows of the head (224 bytes = 14 pieces, stored back to back: a row
@@ -177,7 +180,7 @@ template <typename T, int PRE>
 __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
                                                        float* __restrict__ partial,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int nslot, int range_tokens, int units,
+                                                       int n_chunks, int nrec, int range_tokens, int units,
                                                        int nranges, int64_t stride_b, int64_t stride_n, const QkPre pre) {
   typedef Stage2<PRE> ST;
   constexpr bool has_norm = ST::has_norm, has_rope = ST::has_rope;
@@ -192,7 +195,6 @@ __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restric
   const int r0 = rg * range_tokens, r1 = min(N, r0 + range_tokens);
   if (r0 >= r1) return;
   auto chunk_end = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c + 1] : N; };
-  auto chunk_begin = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c] : 0; };
   int c0 = 0;
   while (chunk_end(c0) <= r0) ++c0;  // the chunk of the range's first token (uniform; a few dozen chunks at most)
   const uint32_t smem_addr = lds_addr(smem);
@@ -299,8 +301,7 @@ __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restric
     issue(tl.start, tl.limit);
   }
   auto record_of = [&](int c) __attribute__((always_inline)) {
-    const int first = uniform(chunk_begin(c) / range_tokens);  // first range touching the chunk
-    const int64_t slot = ((int64_t)(b * h + head) * n_chunks + c) * nslot + (rg - first);
+    const int64_t slot = (int64_t)(b * h + head) * nrec + rg + c;
     return partial + slot * SE;
   };
 
@@ -500,15 +501,15 @@ __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restric
 }
 
 // sum of the records of one chunk in range order (+ inclusive prefix over chunks when causal).  A chunk's records
-// are those of the ranges [begin / L, (end - 1) / L] that touch it; with range_tokens == 0 every chunk has exactly
-// nslot records (the in-place scan of finished states: nslot = 1, partial == state, every thread rewrites only
-// what it has read itself).  Workgroup = cl chunks (a power of two, at most 16) x nq >= 64 groups of four adjacent
+// are those of the ranges [begin / L, (end - 1) / L] that touch it, at record index range + chunk; with
+// range_tokens == 0 every chunk has exactly one record, its own (the in-place scan of finished states: partial ==
+// state, nrec == n_chunks, every thread rewrites only what it has read itself).  Workgroup = cl chunks (a power of two, at most 16) x nq >= 64 groups of four adjacent
 // elements, so that a wave reads whole kilobytes of one record: a thread sums the records of ONE (chunk, element
 // group) -- the loads of its first two
 // records (a chunk shorter than a range has no more) in flight together -- and the prefix over chunks goes through
 // LDS, every thread adding up its predecessors in chunk order, which is the order of a running sum.
 __global__ __launch_bounds__(1024) void reduce112_kernel(const float* partial, float* state, const int32_t* chunk_starts,
-                                                         int N, int n_chunks, int nslot, int range_tokens, int causal,
+                                                         int N, int n_chunks, int nrec, int range_tokens, int causal,
                                                          int cl, int nblk) {
   constexpr int SE4 = SE / 4;
   __shared__ f32x4_t sums[1024];
@@ -525,12 +526,13 @@ __global__ __launch_bounds__(1024) void reduce112_kernel(const float* partial, f
     const bool ok = e_ok && c < n_chunks;
     f32x4_t s = zero;
     if (ok) {
-      int nparts = nslot;
+      int nparts = 1, first = c;
       if (range_tokens > 0) {
         const int cb = chunk_starts ? chunk_starts[c] : 0, ce = chunk_starts ? chunk_starts[c + 1] : N;
         nparts = (ce - 1) / range_tokens - cb / range_tokens + 1;
+        first = cb / range_tokens + c;
       }
-      const float* p0 = partial + ((bh * n_chunks + c) * nslot) * SE + e4 * 4;
+      const float* p0 = partial + (bh * nrec + first) * SE + e4 * 4;
       const f32x4_t v0 = *reinterpret_cast<const f32x4_t*>(p0);  // (every chunk has a first record)
       const f32x4_t v1 = nparts > 1 ? *reinterpret_cast<const f32x4_t*>(p0 + SE) : zero;
       s = v0 + v1;
@@ -1050,12 +1052,12 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
 constexpr int compute_units112() { return 256; }
 
 struct Plan112 {
-  int range_tokens, nslot;
+  int range_tokens, nrec;  // tokens per range; records per (batch, head)
 };
 // One workgroup (eight waves) per compute unit: each (batch, head) is cut into 256 / (B h) token ranges of equal
 // length, whatever the chunking.  The plan must not depend on N (the workspace query does not know it), so the
-// length comes from the upper bound n_chunks * max_chunk_tokens; a chunk is touched by at most
-// ceil(max_chunk_tokens / L) + 1 ranges, which is the number of record slots per chunk.
+// length comes from the upper bound n_chunks * max_chunk_tokens, and so does the number of ranges the records
+// are sized for.
 Plan112 plan112(int B, int h, int n_chunks, int max_chunk_tokens) {
   const int64_t n_ub = (int64_t)n_chunks * max_chunk_tokens;
   int nr = compute_units112() / (B * h);  // rounding down: 260 workgroups on 256 CUs would take two rounds
@@ -1064,7 +1066,7 @@ Plan112 plan112(int B, int h, int n_chunks, int max_chunk_tokens) {
   if (L < 256) L = 256;
   Plan112 pl;
   pl.range_tokens = (int)std::min<int64_t>(L, 1 << 30);
-  pl.nslot = (max_chunk_tokens + pl.range_tokens - 1) / pl.range_tokens + 1;
+  pl.nrec = (int)((n_ub + pl.range_tokens - 1) / pl.range_tokens) + n_chunks - 1;  // index range + chunk
   return pl;
 }
 
@@ -1085,7 +1087,7 @@ Reduce112Plan reduce112_plan(int n_chunks) {
 
 size_t workspace_bytes112(int B, int h, int n_chunks, int max_chunk_tokens) {
   const Plan112 pl = plan112(B, h, n_chunks, max_chunk_tokens);
-  return (size_t)B * h * n_chunks * pl.nslot * SE * sizeof(float);  // the records are always written
+  return (size_t)B * h * pl.nrec * SE * sizeof(float);  // the records are always written
 }
 
 int launch_state112(const void* k, const void* v, float* state, void* workspace, size_t workspace_bytes, int B, int N,
@@ -1102,6 +1104,7 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   if (!aligned16(workspace)) return SANA_ERR_ALIGN;
   float* part = static_cast<float*>(workspace);
   const int nranges = (N + pl.range_tokens - 1) / pl.range_tokens;
+  if (nranges + n_chunks - 1 > pl.nrec) return SANA_ERR_SHAPE;  // N beyond n_chunks * max_chunk_tokens
   const int64_t units = nranges, nwg = head_unit_grid(units, h);
   if (nwg > 0x7fffffff || units * ((h + 3) / 4) * 8 > 0x7fffffff || B > 65535 || (int64_t)B * h > (1 << 22))
     return SANA_ERR_SHAPE;
@@ -1110,7 +1113,7 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   const uint16_t* vp = static_cast<const uint16_t*>(v);
 #define SANA_ST112(T, PRE)                                                                                        \
   hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(512), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
-                     pl.nslot, pl.range_tokens, (int)units, nranges, stride_b, stride_n, pre)
+                     pl.nrec, pl.range_tokens, (int)units, nranges, stride_b, stride_n, pre)
   const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
   if (io_dtype == SANA_DT_F16) SANA_ST112(F16, 0);
   else if (mode == 3) SANA_ST112(BF16, 3);
@@ -1121,7 +1124,7 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   if (hipGetLastError() != hipSuccess) return SANA_ERR_LAUNCH;
   const Reduce112Plan rp = reduce112_plan(n_chunks);
   hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((int64_t)B * h * rp.nblk)), dim3(rp.threads), 0, s, part, state, chunk_starts,
-                     N, n_chunks, pl.nslot, pl.range_tokens, (causal && n_chunks > 1) ? 1 : 0, rp.cl, rp.nblk);
+                     N, n_chunks, pl.nrec, pl.range_tokens, (causal && n_chunks > 1) ? 1 : 0, rp.cl, rp.nblk);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 
@@ -1129,7 +1132,7 @@ int launch_scan112(float* state, int B, int h, int n_chunks, hipStream_t s) {
   if ((int64_t)B * h > (1 << 22)) return SANA_ERR_SHAPE;
   const Reduce112Plan rp = reduce112_plan(n_chunks);
   hipLaunchKernelGGL(reduce112_kernel, dim3((unsigned)((int64_t)B * h * rp.nblk)), dim3(rp.threads), 0, s, state, state,
-                     static_cast<const int32_t*>(nullptr), 0, n_chunks, 1, 0, 1, rp.cl, rp.nblk);
+                     static_cast<const int32_t*>(nullptr), 0, n_chunks, n_chunks, 0, 1, rp.cl, rp.nblk);
   return hipGetLastError() == hipSuccess ? SANA_OK : SANA_ERR_LAUNCH;
 }
 

@@ -174,7 +174,7 @@ def _head_dim(d: int) -> int:
     return d
 
 
-NOALLOC_SCRATCH_BYTES = 24 << 20   # SANA_HIP_NOALLOC_SCRATCH_BYTES of include/sana_hip.h
+NOALLOC_SCRATCH_BYTES = 32 << 20   # SANA_HIP_NOALLOC_SCRATCH_BYTES of include/sana_hip.h
 
 
 def linattn_state(k: torch.Tensor, v: torch.Tensor, chunk_tokens=None, causal: bool = False,

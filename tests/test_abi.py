@@ -74,10 +74,10 @@ def test_workspace_query():
     assert lib.sana_hip_linattn_workspace_bytes(16, 70, 32, 1, 256, 1) == 0
     assert lib.sana_hip_linattn_workspace_bytes(64, 70, 32, 4, 300, 1) == 0
     # head_dim 112 always goes through records of token ranges: 20 heads at the video shape -> 256 // 20 = 12 ranges
-    # of 2752 tokens (a multiple of 64) per head; a chunk of 32760 tokens is touched by at most 12 + 1 of them
-    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 1, 32760, 1) == 20 * 13 * 113 * 112 * 4
-    # 21 chunks of 1560 tokens: the same ranges, each chunk touched by at most 1 + 1
-    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 21, 1560, 1) == 20 * 21 * 2 * 113 * 112 * 4
+    # of 2752 tokens (a multiple of 64) per head, one record per (range, chunk) pair that occurs, indexed range + chunk
+    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 1, 32760, 1) == 20 * 12 * 113 * 112 * 4
+    # 21 chunks of 1560 tokens: the same ranges, 12 + 21 - 1 records
+    assert lib.sana_hip_linattn_workspace_bytes(1, 20, 112, 21, 1560, 1) == 20 * 32 * 113 * 112 * 4
     assert lib.sana_hip_linattn_workspace_bytes(1, 20, 64, 1, 32760, 1) == 0   # no kernel for this head dim
 
 

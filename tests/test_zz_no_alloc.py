@@ -99,6 +99,17 @@ def test_head_dim_112_with_rotary_table_then_a_smaller_call(cuda):
     assert need > 0 and torch.equal(ref, out) and not torch.isnan(out).any()
 
 
+def test_head_dim_112_video_shape_with_21_causal_chunks_fits(cuda):
+    """One video of 21 x 1560 tokens, 20 heads of 112, a causal chunk per frame: 32 records per head, 30.9 MiB."""
+    lib = _lib.load()
+    per, n_chunks = 1560, 21
+    a = _qkv(1, per * n_chunks, 2240, 8, cuda)
+    ref, out, grew, lost, need = _both(lib, a, 112, [f * per for f in range(n_chunks)], True, None, cuda)
+    print(f"d=112 N={per * n_chunks} 21 causal chunks, partial states {need / 2**20:.1f} MiB", flush=True)
+    assert 30 * 2**20 < need <= ops.NOALLOC_SCRATCH_BYTES
+    assert torch.equal(ref, out) and not torch.isnan(out).any() and grew == 0 and lost <= 0
+
+
 def test_python_wrapper_and_the_size_limit(cuda):
     lib = _lib.load()
     qkv = _qkv(2, 3000, 256, 6, cuda)
