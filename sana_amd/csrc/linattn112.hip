@@ -1142,15 +1142,16 @@ static int launch_apply112_pre(const void* q, const float* state, void* out, int
                     hipStream_t s) {
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
   // Tokens per workgroup (a multiple of the 32-token step): long enough to pay for building the state
-  // operands once (~256), and such that the grid fills whole rounds of the chip -- 3 workgroups per CU
-  // fit (2 with transforms or fp32 output: registers), so 4 rounds of 256 tokens with the last one a third
-  // full lose to 3 rounds of 288.
+  // operands once (worth ~48 tokens of work), and such that the grid fills whole rounds of the chip -- 3
+  // workgroups per CU fit (2 with transforms or fp32 output: registers), so 4 rounds of 256 tokens with the last
+  // one a third full lose to 3 rounds of 288, and at the video shape one round of 1280 (one chunk) or of a whole
+  // 1560-token chunk (21 chunks) beats three or four rounds of ~400 by 6 - 8 %.
   const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
   int wg_tokens = 256;
   {
     const int64_t slots = (int64_t)compute_units112() * ((mode || out_dtype == SANA_DT_F32) ? 2 : 3);
     double best = 1e30;
-    for (int t = 192; t <= 512; t += 32) {
+    for (int t = 192; t <= 2048; t += 32) {
       const int64_t wgs = (int64_t)((max_chunk_tokens + t - 1) / t) * n_chunks * B * h;
       const double cost = (double)((wgs + slots - 1) / slots) * (t + 48);  // + the operand build, in token-equivalents
       if (cost < best) {
