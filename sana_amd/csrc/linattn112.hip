@@ -180,8 +180,8 @@ template <typename T, int PRE>
 __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
                                                        float* __restrict__ partial,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int nrec, int range_tokens, int units,
-                                                       int nranges, int64_t stride_b, int64_t stride_n, const QkPre pre) {
+                                                       int nrec, int range_tokens, int units, int64_t stride_b,
+                                                       int64_t stride_n, const QkPre pre) {
   typedef Stage2<PRE> ST;
   constexpr bool has_norm = ST::has_norm, has_rope = ST::has_rope;
   constexpr int NKV = ST::NKV, NR = ST::NR;
@@ -1112,8 +1112,8 @@ int launch_state112(const void* k, const void* v, float* state, void* workspace,
   const uint16_t* kp = static_cast<const uint16_t*>(k);
   const uint16_t* vp = static_cast<const uint16_t*>(v);
 #define SANA_ST112(T, PRE)                                                                                        \
-  hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(512), 0, s, kp, vp, part, chunk_starts, N, h, n_chunks, \
-                     pl.nrec, pl.range_tokens, (int)units, nranges, stride_b, stride_n, pre)
+  hipLaunchKernelGGL((state112_kernel<T, PRE>), grid, dim3(512), 0, s, kp, vp, part, chunk_starts, N, h, pl.nrec, \
+                     pl.range_tokens, (int)units, stride_b, stride_n, pre)
   const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
   if (io_dtype == SANA_DT_F16) SANA_ST112(F16, 0);
   else if (mode == 3) SANA_ST112(BF16, 3);
