@@ -9,8 +9,8 @@
 //            ahead.  One record per chunk the range touches; a second kernel sums a chunk's records in range
 //            order and runs the prefix over chunks.
 //   phase 2  without on-load transforms the same walk: four MFMA waves, four waves that issue the loads and carry
-//            finished output tiles to global memory.  With transforms: workgroup = (batch, head, chunk, range of
-//            192..512 tokens), 256 threads that all load, transform, multiply and store, steps of 32 tokens
+//            finished output tiles to global memory.  With transforms: workgroup = (batch, head, token range of
+//            192..2048 tokens), 256 threads that all load, transform, multiply and store, steps of 32 tokens
 //            through workgroup-shared LDS tiles.  In both, wave w produces output channels [32w, 32w+32) from its
 //            own slice of the state (two bf16 terms of the fp32 values as MFMA 16x16x32 A operands for bf16
 //            output, three for fp32 output) plus a row block that carries ksum in every row, so each lane gets
@@ -849,11 +849,13 @@ __global__ __launch_bounds__(512) void apply112_stream_kernel(const uint16_t* __
 }
 
 // ----------------------------------------------------------------------------
-// phase 2 with on-load transforms (q/k RMSNorm, rotary embedding).  grid.x over units (chunk, token range) x heads,
-// see head_unit, grid.y = batch; block 256: every wave loads, transforms, multiplies and stores, and two or three
-// workgroups share a compute unit.
+// phase 2 with on-load transforms (q/k RMSNorm, rotary embedding).  grid.x over token ranges x heads, see head_unit,
+// grid.y = batch; block 256: every wave loads, transforms, multiplies and stores, and two or three workgroups share
+// a compute unit.
 //
-// The workgroup walks its token range in steps of 32 tokens.  Global memory is touched in whole rows
+// As in the kernels above a workgroup walks ONE contiguous token range of a (batch, head), cut by token count
+// whatever the chunking, in steps of 32 tokens that never straddle a chunk boundary; the state operands are
+// rebuilt when the walk enters another chunk.  Global memory is touched in whole rows
 // only: consecutive threads load consecutive 16-byte pieces of the tokens' 224-byte head rows
 // (transforms applied once, here) into an LDS tile, every wave takes its MFMA B operands from that
 // tile, results go to an LDS output tile and leave as whole rows again.  Tiles are double buffered,
@@ -869,7 +871,7 @@ template <bool OUT_F32, int PRE>
 __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restrict__ Q, const float* __restrict__ state,
                                                        void* __restrict__ out,
                                                        const int32_t* __restrict__ chunk_starts, int N, int h,
-                                                       int n_chunks, int xranges, int wg_tokens, int units,
+                                                       int n_chunks, int range_tokens, int units,
                                                        int64_t q_stride_b,
                                                        int64_t q_stride_n, int64_t o_stride_b, int64_t o_stride_n,
                                                        float eps, const QkPre pre) {
@@ -881,11 +883,12 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   HeadUnit hu;
   if (!head_unit(blockIdx.x, units, h, hu)) return;  // uniform over the workgroup
   const int head = hu.head;
-  const int c = uniform(hu.unit / xranges), bx = hu.unit - c * xranges, b = blockIdx.y;
-  const ChunkRange cr = chunk_range(chunk_starts, c, N);
-  const int t0 = cr.begin + bx * wg_tokens;
-  const int t1 = min(cr.end, t0 + wg_tokens);
-  if (t0 >= t1) return;  // uniform over the workgroup
+  const int b = blockIdx.y;
+  const int r0 = hu.unit * range_tokens, r1 = min(N, r0 + range_tokens);
+  if (r0 >= r1) return;  // uniform over the workgroup
+  auto chunk_end = [&](int c) __attribute__((always_inline)) { return chunk_starts ? chunk_starts[c + 1] : N; };
+  int c0 = 0;
+  while (chunk_end(c0) <= r0) ++c0;  // the chunk of the range's first token (uniform; a few dozen chunks at most)
   const int n = lane & 15, g = lane >> 4;
   constexpr bool has_norm = (PRE & 1) != 0, has_rope = (PRE & 2) != 0;
 
@@ -893,10 +896,10 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   // wave is output channel 32*wave + 8*(r/4) + 4*rb + r%4, so that a lane (token n, group g') ends up
   // with the 8 contiguous channels 32*wave + 8*g' .. +7 (registers s of blocks 0 and 1).  Block 2
   // carries ksum in every row.  Channels and k indices past 112 are zero.
-  const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * SE;
   constexpr int NT = OUT_F32 ? 3 : 2;  // bf16 terms of an fp32 state value: 24 / 16 mantissa bits
   u32x4_t a[3][4][NT];                 // [row block][k block][term]
-  {
+  auto load_state = [&](int c) __attribute__((always_inline)) {
+    const float* sp = state + ((int64_t)(b * h + head) * n_chunks + c) * SE;
     // buffer loads: rows / k groups outside the head's state get an out-of-range offset and read as zero
     const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sp), 0, SE * 4, 0x00020000);
 #pragma unroll
@@ -914,7 +917,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
         split_terms<NT>(x, a[rb][kb]);
       }
     }
-  }
+  };
 
   // tile load mapping: piece id = tid + 256 i (i < 2, id < 448): token id / 14, 16-byte piece id % 14
   int ld_tok[2], ld_ch[2];
@@ -937,7 +940,7 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
     for (int i = 0; i < 2; ++i)
       if (ld_ok[i]) qw[i] = *reinterpret_cast<const u32x4_t*>(pre.weight + head * DH + ld_ch[i] * 8);
   }
-  auto issue = [&](int t) {
+  auto issue = [&](int t, int t1) {  // the 32 tokens from t, those before t1
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int tok = t + ld_tok[i];
@@ -968,12 +971,40 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
   const int och = 32 * wave + 8 * g;  // this lane's 8 output channels
   for (int i = tid; i < 2 * NQ * TT * 3; i += 256)  // pieces 14..16 of every q tile row: written once, as zeros
     *reinterpret_cast<u32x4_t*>(lds_q + (i / 3) * QROWE + (NCH + i % 3) * 8) = zero4;
-  issue(t0);
+  auto has_tile = [&](const TileCur& cur) __attribute__((always_inline)) { return cur.t < r1; };
+  auto next_tile = [&](TileCur& cur) __attribute__((always_inline)) {
+    Tile112 tl;
+    tl.start = cur.t;
+    tl.limit = cur.seg_end;
+    tl.c = cur.c;
+    const int nt = min(cur.t + TT, cur.seg_end);
+    tl.last = nt == cur.seg_end;
+    cur.t = nt;
+    if (tl.last && nt < r1) {
+      ++cur.c;
+      cur.seg_end = min(chunk_end(cur.c), r1);
+    }
+    return tl;
+  };
+  TileCur icur = {r0, c0, min(chunk_end(c0), r1)}, ccur = icur;
+  {
+    const Tile112 ti = next_tile(icur);
+    issue(ti.start, ti.limit);
+  }
   stage(0);
-  if (t0 + TT < t1) issue(t0 + TT);
+  if (has_tile(icur)) {
+    const Tile112 ti = next_tile(icur);
+    issue(ti.start, ti.limit);
+  }
   __syncthreads();
-  int buf = 0;
-  for (int t = t0; t < t1; t += TT, buf ^= 1) {
+  int cur_c = -1;
+  for (int buf = 0; has_tile(ccur); buf ^= 1) {
+    const Tile112 tl = next_tile(ccur);
+    const int t = tl.start, t1 = tl.limit;
+    if (tl.c != cur_c) {  // uniform: the walk enters another chunk
+      load_state(tl.c);
+      cur_c = tl.c;
+    }
     const uint16_t* td = lds_q + buf * NQ * TT * QROWE;
     const uint16_t* tb = has_rope ? td + TT * QROWE : td;
     uint16_t* to = lds_o + buf * OT;
@@ -1020,9 +1051,12 @@ __global__ __launch_bounds__(256) void apply112_kernel(const uint16_t* __restric
       }
     }
     // next tile: registers -> the other q tile (its last readers passed the previous barrier); loads of the one after
-    if (t + TT < t1) {
+    if (has_tile(ccur)) {
       stage(buf ^ 1);
-      if (t + 2 * TT < t1) issue(t + 2 * TT);
+      if (has_tile(icur)) {
+        const Tile112 ti = next_tile(icur);
+        issue(ti.start, ti.limit);
+      }
     }
     __syncthreads();
     // this step's output tile leaves as whole rows (it is next written two steps from now, behind the next barrier)
@@ -1141,33 +1175,33 @@ static int launch_apply112_pre(const void* q, const float* state, void* out, int
                     int n_chunks, int max_chunk_tokens, float eps, int io_dtype, int out_dtype, const QkPre& pre,
                     hipStream_t s) {
   if (io_dtype != SANA_DT_BF16) return SANA_ERR_DTYPE;
-  // Tokens per workgroup (a multiple of the 32-token step): long enough to pay for building the state
-  // operands once (worth ~48 tokens of work), and such that the grid fills whole rounds of the chip -- 3
-  // workgroups per CU fit (2 with transforms or fp32 output: registers), so 4 rounds of 256 tokens with the last
-  // one a third full lose to 3 rounds of 288, and at the video shape one round of 1280 (one chunk) or of a whole
-  // 1560-token chunk (21 chunks) beats three or four rounds of ~400 by 6 - 8 %.
+  // Tokens per workgroup (a multiple of the 32-token step), whatever the chunking: long enough to pay for building
+  // the state operands (worth ~48 tokens of work, once per chunk the range touches), and such that the grid fills
+  // whole rounds of the chip -- 3 workgroups per CU fit (2 with transforms or fp32 output: registers), so 4 rounds
+  // of 256 tokens with the last one a third full lose to 3 rounds of 288, and at the video shape one round of
+  // 1312-token ranges beats three or four rounds of ~400 by 6 - 8 %.
   const int mode = (pre.rinv ? 1 : 0) | (pre.rope ? 2 : 0);
-  int wg_tokens = 256;
+  int range_tokens = 256;
   {
     const int64_t slots = (int64_t)compute_units112() * ((mode || out_dtype == SANA_DT_F32) ? 2 : 3);
     double best = 1e30;
     for (int t = 192; t <= 2048; t += 32) {
-      const int64_t wgs = (int64_t)((max_chunk_tokens + t - 1) / t) * n_chunks * B * h;
-      const double cost = (double)((wgs + slots - 1) / slots) * (t + 48);  // + the operand build, in token-equivalents
+      const int64_t wgs = (int64_t)((N + t - 1) / t) * B * h;
+      const double builds = 1.0 + (double)t / std::max(max_chunk_tokens, 1);  // chunks a range touches, roughly
+      const double cost = (double)((wgs + slots - 1) / slots) * (t + 48.0 * builds);
       if (cost < best) {
         best = cost;
-        wg_tokens = t;
+        range_tokens = t;
       }
     }
   }
-  const int xranges = (max_chunk_tokens + wg_tokens - 1) / wg_tokens;
-  const int64_t units = (int64_t)xranges * n_chunks, total = head_unit_grid(units, h);
+  const int64_t units = (N + range_tokens - 1) / range_tokens, total = head_unit_grid(units, h);
   if (total > 0x7fffffff || units * ((h + 3) / 4) * 8 > 0x7fffffff || B > 65535) return SANA_ERR_SHAPE;
   dim3 grid((unsigned)total, (unsigned)B);
   const uint16_t* qp = static_cast<const uint16_t*>(q);
 #define SANA_AP112(F32, PRE)                                                                                         \
   hipLaunchKernelGGL((apply112_kernel<F32, PRE>), grid, dim3(256), 0, s, qp, state, out, chunk_starts, N, h, n_chunks, \
-                     xranges, wg_tokens, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
+                     range_tokens, (int)units, q_stride_b, q_stride_n, o_stride_b, o_stride_n, eps, pre)
   if (out_dtype == SANA_DT_F32) {
     if (mode == 3) SANA_AP112(true, 3);
     else if (mode == 2) SANA_AP112(true, 2);
