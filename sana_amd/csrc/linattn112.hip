@@ -305,7 +305,7 @@ __global__ __launch_bounds__(512) void state112_kernel(const uint16_t* __restric
     return partial + slot * SE;
   };
 
-  // ---- roles.  Waves 0..3 run the MFMAs, waves 4..7 the transforms; all eight issue loads.
+  // ---- roles.  Waves 0..3 run the MFMAs (and issue the loads), waves 4..7 the transforms.
   const bool mma_role = wave < 4;  // wave-uniform
 
   // ---- transform side: 16-byte piece i of a tile = piece i % 14 of token i / 14; thread tid - 256 takes pieces
