@@ -285,3 +285,35 @@ def test_litela_rotary_tables_without_pair_structure_take_the_stock_pass(cuda, c
             out = hm(x.to(cuda), rotary_emb=(cos.to(cuda), sin.to(cuda)))
     assert any("LiteLA rotary embedding" in r.getMessage() for r in caplog.records)
     check(out, ref, "LiteLA generic real tables")
+
+
+def test_chunk_causal_head_dim_112_replays_from_a_hip_graph(cuda):
+    """The 112-wide-head kernels (rings of direct-to-LDS loads, counted waits, records per range and chunk) captured
+    once: every replay, with eager launches and synchronisations between them, equals the eager result bit for bit,
+    also after the input changes."""
+    B, C, (f, h, w) = 1, 448, (6, 10, 13)
+    N = f * h * w
+    om, hm = make("ChunkCausalAttention", C, True, seed=12, head_dim=112)
+    hm = hm.to(cuda)
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(1)).bfloat16().to(cuda)
+    fr = freqs(N, 3, head_dim=112).to(cuda)
+    kw = dict(HW=(f, h, w), rotary_emb=fr, chunk_index=[0, 1, 4])
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):           # warm-up off the default stream, as capture requires
+            for _ in range(2):
+                hm(x, **kw)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = hm(x, **kw)
+        for r in range(3):
+            if r == 2:
+                x.copy_(torch.randn(x.shape, generator=torch.Generator().manual_seed(9)).bfloat16())
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = hm(x, **kw)
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {r}"
+        check(out, ref64(om, x.cpu(), HW=(f, h, w), rotary_emb=fr.cpu(), chunk_index=[0, 1, 4]), "graph replay, d=112")
